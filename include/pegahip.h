@@ -1,0 +1,314 @@
+/*
+ * pegahip.h — C ABI of libpegahip.so: the MI355X (gfx950) implementation of
+ * PegaFlow's layer-wise KV block transfer path.
+ *
+ * This is the boundary a `-sys` crate (or any FFI) binds in place of the CUDA
+ * bindings the reference uses on this path.  Every entry point is `extern "C"`,
+ * takes plain pointers and sizes, and cites the reference interface it stands
+ * in for (paths are relative to the reference checkout).
+ *
+ * Conventions (reference: pegaflow-core/src/transfer/mod.rs:15-16,46-52):
+ *  - Transfer calls only ENQUEUE onto the caller's stream and never synchronise.
+ *    The caller keeps descriptors' device and host memory alive until it has
+ *    synchronised the stream (or an event recorded after the call).
+ *  - Return value: 0 = success; > 0 = a hipError_t from the HIP runtime;
+ *    < 0 = one of the PF_ERR_* classes below.  After any non-zero return,
+ *    pf_last_error() gives the message for the calling thread.
+ *  - Handles are opaque pointers.  A backend / transfer handle belongs to one
+ *    worker thread at a time (the reference's `TransferBackend: Send`, not
+ *    `Sync`); pools and allocators are internally locked.
+ *  - There is no CPU fallback: every call that moves bytes needs a HIP device
+ *    and fails with a HIP error when none is present.
+ */
+#ifndef PEGAHIP_H
+#define PEGAHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------ */
+/* Status                                                                    */
+/* ------------------------------------------------------------------------ */
+
+/* Error classes; mirror `EngineError` (pegaflow-core/src/lib.rs, variants
+ * InvalidArgument / Storage / CudaInit / WorkerMissing). */
+#define PF_OK 0
+#define PF_ERR_INVALID_ARGUMENT (-1)
+#define PF_ERR_STORAGE (-2)
+#define PF_ERR_DEVICE_INIT (-3)
+#define PF_ERR_WORKER_MISSING (-4)
+#define PF_ERR_INSTANCE_MISSING (-5)
+#define PF_ERR_BUFFER_TOO_SMALL (-6)
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* pf_last_error(void);
+/* Library version string. */
+const char* pf_version(void);
+
+/* ------------------------------------------------------------------------ */
+/* Device, stream, event                                                     */
+/* Replaces cudarc CudaContext::new / new_stream / record_event /            */
+/* event.synchronize (pegaflow-core/src/gpu_worker.rs:278-298,443-449).      */
+/* ------------------------------------------------------------------------ */
+
+typedef struct pf_stream_s* pf_stream_t; /* wraps a hipStream_t */
+typedef struct pf_event_s* pf_event_t;   /* wraps a hipEvent_t */
+
+int pf_device_count(int* out_count);
+int pf_set_device(int device);
+int pf_get_device(int* out_device);
+int pf_device_synchronize(void);
+/* NUMA node of the device from /sys/bus/pci/devices/<bdf>/numa_node; -1 when
+ * unknown.  Replaces `nvidia-smi topo --get-numa-id-of-nearby-cpu`
+ * (pegaflow-common/src/numa.rs:266-287). */
+int pf_device_numa_node(int device, int* out_node);
+int pf_device_name(int device, char* buf, size_t cap);
+
+/* Non-blocking stream at the default priority. */
+int pf_stream_create(pf_stream_t* out);
+/* Wrap an existing hipStream_t (e.g. torch's) without owning it. */
+int pf_stream_wrap(void* hip_stream, pf_stream_t* out);
+int pf_stream_destroy(pf_stream_t s);
+int pf_stream_synchronize(pf_stream_t s);
+int pf_stream_wait_event(pf_stream_t s, pf_event_t e);
+void* pf_stream_native(pf_stream_t s);
+
+int pf_event_create(int enable_timing, pf_event_t* out);
+int pf_event_destroy(pf_event_t e);
+int pf_event_record(pf_event_t e, pf_stream_t s);
+int pf_event_synchronize(pf_event_t e);
+/* *out_done = 1 when complete, 0 when still pending. */
+int pf_event_query(pf_event_t e, int* out_done);
+int pf_event_elapsed_ms(pf_event_t start, pf_event_t stop, float* out_ms);
+
+/* ------------------------------------------------------------------------ */
+/* Pinned host memory                                                        */
+/* Replaces PinnedMemory (pegaflow-core/src/pinned_mem.rs:100-397).          */
+/* ------------------------------------------------------------------------ */
+
+/* AllocStrategy, pinned_mem.rs:100-111. */
+#define PF_HOST_REGULAR 0   /* mmap + parallel NUMA pre-touch + hipHostRegister(Mapped) */
+#define PF_HOST_HIP_ALLOC 1 /* hipHostMalloc(Mapped); the default strategy */
+#define PF_HOST_HUGEPAGES 2 /* mmap(MAP_HUGETLB) + pre-touch + hipHostRegister(Mapped) */
+
+typedef struct pf_host_mem {
+  void* host;          /* host virtual address */
+  uint64_t device;     /* device-visible address of the same bytes */
+  uint64_t size;       /* actual size (huge pages round up) */
+  int32_t strategy;    /* PF_HOST_* */
+  int32_t numa_node;   /* requested node, -1 = none */
+} pf_host_mem;
+
+/* numa_node < 0: placement follows the calling thread's affinity. */
+int pf_host_alloc(uint64_t size, int strategy, int numa_node, pf_host_mem* out);
+int pf_host_free(pf_host_mem* mem);
+/* Worker count of the parallel pre-touch (pinned_mem.rs:368-376). */
+uint64_t pf_touch_threads(uint64_t size);
+/* Hugepagesize from /proc/meminfo in bytes, 0 when unavailable
+ * (pinned_mem.rs:46-60). */
+uint64_t pf_huge_page_size(void);
+
+/* Device memory helpers for tests and benches; replace the reference's
+ * test-only cuMemAlloc/cuMemcpy/cuMemset helpers
+ * (pegaflow-core/tests/common/gpu_buffer.rs:13-69). */
+int pf_dev_malloc(uint64_t size, uint64_t* out_ptr);
+int pf_dev_free(uint64_t ptr);
+int pf_dev_memset(uint64_t ptr, int value, uint64_t size);
+int pf_dev_copy_from_host(uint64_t dst, const void* src, uint64_t size);
+int pf_dev_copy_to_host(void* dst, uint64_t src, uint64_t size);
+/* One contiguous async copy between device memory and pinned host memory on
+ * `s`; the link-peak yardstick of the benches. */
+int pf_memcpy_h2d_async(uint64_t dst, const void* src, uint64_t size, pf_stream_t s);
+int pf_memcpy_d2h_async(void* dst, uint64_t src, uint64_t size, pf_stream_t s);
+
+/* ------------------------------------------------------------------------ */
+/* KV cache layout                                                           */
+/* Replaces KVCacheLayout / BlockCopy / BlockCopies                          */
+/* (pegaflow-core/src/layout.rs:13-286).                                     */
+/* ------------------------------------------------------------------------ */
+
+typedef struct pf_kv_layout {
+  uint64_t data_ptr;             /* device base of this layer's cache */
+  uint64_t size_bytes;           /* registered region size */
+  uint64_t num_blocks;
+  uint64_t block_stride_bytes;   /* step between consecutive blocks */
+  uint64_t segment_bytes;        /* one of K or V (unpadded) */
+  uint64_t segments;             /* 1, or 2 for K/V */
+  uint64_t padded_segment_bytes; /* host-side stride of one segment */
+  uint64_t kv_stride_bytes;      /* distance K -> V when split, else 0 */
+  uint32_t split;                /* 1 = K and V in separate regions */
+  uint32_t reserved;
+} pf_kv_layout;
+
+typedef struct pf_block_copy {
+  uint64_t addr;
+  uint64_t bytes;
+} pf_block_copy;
+
+/* KVCacheLayout::new, layout.rs:73-130. */
+int pf_layout_new(uint64_t data_ptr, uint64_t size_bytes, uint64_t num_blocks,
+                  uint64_t segment_bytes, uint64_t kv_stride_bytes,
+                  uint64_t segments, pf_kv_layout* out);
+/* KVCacheLayout::with_block_stride, layout.rs:140-153. */
+int pf_layout_with_block_stride(pf_kv_layout* layout, uint64_t stride);
+/* KVCacheLayout::with_ssd_padding, layout.rs:157-160. */
+int pf_layout_with_ssd_padding(pf_kv_layout* layout, uint64_t alignment);
+/* KVCacheLayout::block_copies, layout.rs:231-255: *out_n is 1 (contiguous) or
+ * 2 (split: out[0] = K, out[1] = V). */
+int pf_layout_block_copies(const pf_kv_layout* layout, uint64_t block_idx,
+                           pf_block_copy out[2], uint32_t* out_n);
+/* padded_block_bytes, layout.rs:283-285. */
+uint64_t pf_layout_padded_block_bytes(const pf_kv_layout* layout);
+/* block_bytes, layout.rs:271-273. */
+uint64_t pf_layout_block_bytes(const pf_kv_layout* layout);
+
+/* ------------------------------------------------------------------------ */
+/* Copy descriptors and the two reference transfer backends                  */
+/* Replaces CopyDesc / TransferBackend / TransferMode                        */
+/* (pegaflow-core/src/transfer/mod.rs:36-76), MemcpyBackend                  */
+/* (transfer/memcpy.rs:25-102) and KernelBackend (transfer/kernel.rs:25-135).*/
+/* ------------------------------------------------------------------------ */
+
+typedef struct pf_copy_desc {
+  uint64_t device;            /* absolute device address */
+  void* host;                 /* host virtual address */
+  uint64_t host_device;       /* device-visible address of `host` */
+  uint64_t size;
+  uint64_t device_allocation; /* layer index */
+  uint64_t host_allocation;   /* identity of the pinned allocation */
+} pf_copy_desc;
+
+typedef struct pf_merged_range {
+  uint64_t device;
+  void* host;
+  uint64_t size;
+} pf_merged_range;
+
+#define PF_MODE_DIRECT 0 /* one DMA copy per merged range ("direct") */
+#define PF_MODE_KERNEL 1 /* one copy kernel over mapped host memory ("kernel") */
+
+typedef struct pf_backend_s* pf_backend_t;
+
+/* merge(), memcpy.rs:25-55.  `out` needs room for n entries. */
+int pf_merge_copies(const pf_copy_desc* copies, uint64_t n, pf_merged_range* out,
+                    uint64_t* out_n);
+/* build_backend, gpu_worker.rs:264-276.  Binds to the current device. */
+int pf_backend_create(int mode, pf_backend_t* out);
+int pf_backend_destroy(pf_backend_t b);
+/* TransferBackend::name: "direct" or "kernel". */
+const char* pf_backend_name(pf_backend_t b);
+/* TransferBackend::h2d / d2h.  Enqueue only. */
+int pf_backend_h2d(pf_backend_t b, const pf_copy_desc* copies, uint64_t n, pf_stream_t s);
+int pf_backend_d2h(pf_backend_t b, const pf_copy_desc* copies, uint64_t n, pf_stream_t s);
+/* TransferMode from the connector's string ("direct" | "kernel"),
+ * python/pegaflow/connector/common.py:577-594. */
+int pf_transfer_mode_from_name(const char* name, int* out_mode);
+
+/* ------------------------------------------------------------------------ */
+/* Descriptor construction from layouts x blocks                             */
+/* Replaces build_copy_descs (pegaflow-core/src/gpu_worker.rs:353-423) and   */
+/* the host-block view it reads (block.rs:62-199, gpu_worker.rs:63-94).      */
+/* ------------------------------------------------------------------------ */
+
+typedef struct pf_host_block {
+  void* seg_host[2];       /* host address of segment 0 / 1 */
+  uint64_t seg_device[2];  /* device-visible address of segment 0 / 1 */
+  uint64_t seg_alloc[2];   /* allocation identity of segment 0 / 1 */
+  uint64_t seg_size[2];    /* (padded) size of segment 0 / 1 */
+  uint32_t num_segments;   /* 1 or 2 */
+  uint32_t reserved;
+  uint64_t host_offset;    /* page-first byte offset of this layer; else 0 */
+} pf_host_block;
+
+typedef struct pf_layer_transfer {
+  const char* layer_name;
+  pf_kv_layout layout;
+  const uint64_t* block_idx;   /* device slot of each block */
+  const pf_host_block* blocks; /* host image of each block */
+  uint64_t n_blocks;
+} pf_layer_transfer;
+
+/* Writes up to `cap` descriptors; *out_n is the count needed.  Returns
+ * PF_ERR_BUFFER_TOO_SMALL when cap < *out_n (nothing else is wrong). */
+int pf_build_copy_descs(const pf_layer_transfer* layers, uint64_t n_layers,
+                        pf_copy_desc* out, uint64_t cap, uint64_t* out_n,
+                        uint64_t* out_total_bytes);
+
+/* ------------------------------------------------------------------------ */
+/* Block-ID gather / scatter (the MI355X fast path)                          */
+/* Same bytes as build_copy_descs + TransferBackend::{d2h,h2d}               */
+/* (gpu_worker.rs:353-423,441,494) with no per-fragment descriptor: the      */
+/* kernels compute `data_ptr + id*block_stride (+ kv_stride)` themselves.    */
+/* ------------------------------------------------------------------------ */
+
+typedef struct pf_layer_blocks {
+  const char* layer_name;    /* for error messages; may be NULL */
+  pf_kv_layout layout;
+  const uint32_t* block_ids; /* host array: device slot of block i */
+  uint64_t n_blocks;
+  /* Host image.  Segment s of block i lives at
+   *   host[s] + i*host_stride                       (page_host == NULL), or
+   *   page_host[i] + page_offset + s*segment_bytes  (page_host != NULL).
+   * For a contiguous (non-split) layout only host[0] is used and one block
+   * is one fragment of block_bytes. */
+  void* host[2];
+  uint64_t host_device[2];
+  uint64_t host_len[2];         /* bytes available behind host[s] */
+  uint64_t host_stride;
+  const uint64_t* page_host;        /* optional per-block page bases (host VA) */
+  const uint64_t* page_host_device; /* same, device-visible */
+  uint64_t page_offset;
+  uint64_t page_len;                /* bytes available behind each page base */
+} pf_layer_blocks;
+
+/* How bytes cross the host link. */
+#define PF_PATH_AUTO 0     /* pick per shape */
+#define PF_PATH_ZEROCOPY 1 /* kernel reads/writes mapped host memory */
+#define PF_PATH_STAGED 2   /* device gather/scatter + one DMA copy per unit */
+
+typedef struct pf_xfer_config {
+  uint64_t staging_slot_bytes; /* 0 = default */
+  uint32_t staging_slots;      /* 0 = default (2) */
+  uint32_t zerocopy_max_workgroups; /* 0 = default; caps CUs used next to compute */
+  uint64_t auto_staged_min_bytes;   /* 0 = default threshold for PF_PATH_AUTO */
+  uint32_t tile_unroll;             /* 16-byte loads in flight per lane: 1,2,4,8; 0 = default */
+  uint32_t reserved;
+} pf_xfer_config;
+
+typedef struct pf_xfer_s* pf_xfer_t;
+
+int pf_xfer_create(const pf_xfer_config* cfg, pf_xfer_t* out);
+int pf_xfer_destroy(pf_xfer_t x);
+/* Save: gather the listed blocks of every layer into their host images. */
+int pf_xfer_save(pf_xfer_t x, const pf_layer_blocks* layers, uint64_t n_layers,
+                 int path, pf_stream_t s);
+/* Load: scatter host images into the listed device slots. */
+int pf_xfer_load(pf_xfer_t x, const pf_layer_blocks* layers, uint64_t n_layers,
+                 int path, pf_stream_t s);
+/* Optional per-layer completion events: when set (n >= n_layers of the next
+ * call) each layer's event is recorded when that layer's bytes have landed.
+ * Pass NULL to clear. */
+int pf_xfer_set_layer_events(pf_xfer_t x, pf_event_t* events, uint64_t n);
+/* Path the last call took for layer 0 (PF_PATH_ZEROCOPY or PF_PATH_STAGED). */
+int pf_xfer_last_path(pf_xfer_t x);
+/* Timing of the device-side gather/scatter kernels of the last call: total
+ * milliseconds and launches, measured with events on the stream the kernels
+ * ran on.  Blocks until those events have completed. */
+int pf_xfer_last_kernel_ms(pf_xfer_t x, float* out_ms, uint32_t* out_launches);
+int pf_xfer_set_kernel_timing(pf_xfer_t x, int enable);
+
+/* Plain device-to-device copy with the same tile shape as the gather/scatter
+ * kernels (pointers and size 16-byte aligned).  A copy of known size: the
+ * yardstick for the HBM copy ceiling and for scaling hardware counters.  No
+ * counterpart in the reference. */
+int pf_plain_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t tile_unroll,
+                  pf_stream_t s);
+
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+#endif /* PEGAHIP_H */

@@ -1,0 +1,201 @@
+"""ctypes binding of ``libpegahip.so`` (declared in ``include/pegahip.h``).
+
+The library is the product: if it is missing this module raises, there is no
+Python or CPU fallback for anything that moves bytes.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libpegahip.so")
+
+PF_OK = 0
+PF_ERR_INVALID_ARGUMENT = -1
+PF_ERR_STORAGE = -2
+PF_ERR_DEVICE_INIT = -3
+PF_ERR_WORKER_MISSING = -4
+PF_ERR_INSTANCE_MISSING = -5
+PF_ERR_BUFFER_TOO_SMALL = -6
+
+PF_HOST_REGULAR = 0
+PF_HOST_HIP_ALLOC = 1
+PF_HOST_HUGEPAGES = 2
+
+PF_MODE_DIRECT = 0
+PF_MODE_KERNEL = 1
+
+PF_PATH_AUTO = 0
+PF_PATH_ZEROCOPY = 1
+PF_PATH_STAGED = 2
+
+u64 = C.c_uint64
+u32 = C.c_uint32
+vp = C.c_void_p
+
+
+class PfHostMem(C.Structure):
+    _fields_ = [("host", vp), ("device", u64), ("size", u64), ("strategy", C.c_int32),
+                ("numa_node", C.c_int32)]
+
+
+class PfKvLayout(C.Structure):
+    _fields_ = [
+        ("data_ptr", u64), ("size_bytes", u64), ("num_blocks", u64), ("block_stride_bytes", u64),
+        ("segment_bytes", u64), ("segments", u64), ("padded_segment_bytes", u64),
+        ("kv_stride_bytes", u64), ("split", u32), ("reserved", u32),
+    ]
+
+
+class PfBlockCopy(C.Structure):
+    _fields_ = [("addr", u64), ("bytes", u64)]
+
+
+class PfCopyDesc(C.Structure):
+    _fields_ = [("device", u64), ("host", vp), ("host_device", u64), ("size", u64),
+                ("device_allocation", u64), ("host_allocation", u64)]
+
+
+class PfMergedRange(C.Structure):
+    _fields_ = [("device", u64), ("host", vp), ("size", u64)]
+
+
+class PfHostBlock(C.Structure):
+    _fields_ = [("seg_host", vp * 2), ("seg_device", u64 * 2), ("seg_alloc", u64 * 2),
+                ("seg_size", u64 * 2), ("num_segments", u32), ("reserved", u32),
+                ("host_offset", u64)]
+
+
+class PfLayerTransfer(C.Structure):
+    _fields_ = [("layer_name", C.c_char_p), ("layout", PfKvLayout),
+                ("block_idx", C.POINTER(u64)), ("blocks", C.POINTER(PfHostBlock)),
+                ("n_blocks", u64)]
+
+
+class PfLayerBlocks(C.Structure):
+    _fields_ = [
+        ("layer_name", C.c_char_p), ("layout", PfKvLayout), ("block_ids", C.POINTER(u32)),
+        ("n_blocks", u64), ("host", vp * 2), ("host_device", u64 * 2), ("host_len", u64 * 2),
+        ("host_stride", u64), ("page_host", C.POINTER(u64)), ("page_host_device", C.POINTER(u64)),
+        ("page_offset", u64), ("page_len", u64),
+    ]
+
+
+class PfXferConfig(C.Structure):
+    _fields_ = [("staging_slot_bytes", u64), ("staging_slots", u32),
+                ("zerocopy_max_workgroups", u32), ("auto_staged_min_bytes", u64),
+                ("tile_unroll", u32), ("reserved", u32)]
+
+
+# name -> (restype, argtypes).  Every symbol include/pegahip.h declares.
+PROTOTYPES = {
+    "pf_last_error": (C.c_char_p, []),
+    "pf_version": (C.c_char_p, []),
+    "pf_device_count": (C.c_int, [C.POINTER(C.c_int)]),
+    "pf_set_device": (C.c_int, [C.c_int]),
+    "pf_get_device": (C.c_int, [C.POINTER(C.c_int)]),
+    "pf_device_synchronize": (C.c_int, []),
+    "pf_device_numa_node": (C.c_int, [C.c_int, C.POINTER(C.c_int)]),
+    "pf_device_name": (C.c_int, [C.c_int, C.c_char_p, C.c_size_t]),
+    "pf_stream_create": (C.c_int, [C.POINTER(vp)]),
+    "pf_stream_wrap": (C.c_int, [vp, C.POINTER(vp)]),
+    "pf_stream_destroy": (C.c_int, [vp]),
+    "pf_stream_synchronize": (C.c_int, [vp]),
+    "pf_stream_wait_event": (C.c_int, [vp, vp]),
+    "pf_stream_native": (vp, [vp]),
+    "pf_event_create": (C.c_int, [C.c_int, C.POINTER(vp)]),
+    "pf_event_destroy": (C.c_int, [vp]),
+    "pf_event_record": (C.c_int, [vp, vp]),
+    "pf_event_synchronize": (C.c_int, [vp]),
+    "pf_event_query": (C.c_int, [vp, C.POINTER(C.c_int)]),
+    "pf_event_elapsed_ms": (C.c_int, [vp, vp, C.POINTER(C.c_float)]),
+    "pf_host_alloc": (C.c_int, [u64, C.c_int, C.c_int, C.POINTER(PfHostMem)]),
+    "pf_host_free": (C.c_int, [C.POINTER(PfHostMem)]),
+    "pf_touch_threads": (u64, [u64]),
+    "pf_huge_page_size": (u64, []),
+    "pf_dev_malloc": (C.c_int, [u64, C.POINTER(u64)]),
+    "pf_dev_free": (C.c_int, [u64]),
+    "pf_dev_memset": (C.c_int, [u64, C.c_int, u64]),
+    "pf_dev_copy_from_host": (C.c_int, [u64, vp, u64]),
+    "pf_dev_copy_to_host": (C.c_int, [vp, u64, u64]),
+    "pf_memcpy_h2d_async": (C.c_int, [u64, vp, u64, vp]),
+    "pf_memcpy_d2h_async": (C.c_int, [vp, u64, u64, vp]),
+    "pf_layout_new": (C.c_int, [u64, u64, u64, u64, u64, u64, C.POINTER(PfKvLayout)]),
+    "pf_layout_with_block_stride": (C.c_int, [C.POINTER(PfKvLayout), u64]),
+    "pf_layout_with_ssd_padding": (C.c_int, [C.POINTER(PfKvLayout), u64]),
+    "pf_layout_block_copies": (C.c_int, [C.POINTER(PfKvLayout), u64, C.POINTER(PfBlockCopy),
+                                         C.POINTER(u32)]),
+    "pf_layout_padded_block_bytes": (u64, [C.POINTER(PfKvLayout)]),
+    "pf_layout_block_bytes": (u64, [C.POINTER(PfKvLayout)]),
+    "pf_merge_copies": (C.c_int, [C.POINTER(PfCopyDesc), u64, C.POINTER(PfMergedRange),
+                                  C.POINTER(u64)]),
+    "pf_backend_create": (C.c_int, [C.c_int, C.POINTER(vp)]),
+    "pf_backend_destroy": (C.c_int, [vp]),
+    "pf_backend_name": (C.c_char_p, [vp]),
+    "pf_backend_h2d": (C.c_int, [vp, C.POINTER(PfCopyDesc), u64, vp]),
+    "pf_backend_d2h": (C.c_int, [vp, C.POINTER(PfCopyDesc), u64, vp]),
+    "pf_transfer_mode_from_name": (C.c_int, [C.c_char_p, C.POINTER(C.c_int)]),
+    "pf_build_copy_descs": (C.c_int, [C.POINTER(PfLayerTransfer), u64, C.POINTER(PfCopyDesc), u64,
+                                      C.POINTER(u64), C.POINTER(u64)]),
+    "pf_xfer_create": (C.c_int, [C.POINTER(PfXferConfig), C.POINTER(vp)]),
+    "pf_xfer_destroy": (C.c_int, [vp]),
+    "pf_xfer_save": (C.c_int, [vp, C.POINTER(PfLayerBlocks), u64, C.c_int, vp]),
+    "pf_xfer_load": (C.c_int, [vp, C.POINTER(PfLayerBlocks), u64, C.c_int, vp]),
+    "pf_xfer_set_layer_events": (C.c_int, [vp, C.POINTER(vp), u64]),
+    "pf_xfer_last_path": (C.c_int, [vp]),
+    "pf_xfer_last_kernel_ms": (C.c_int, [vp, C.POINTER(C.c_float), C.POINTER(u32)]),
+    "pf_xfer_set_kernel_timing": (C.c_int, [vp, C.c_int]),
+    "pf_plain_copy": (C.c_int, [u64, u64, u64, u32, vp]),
+}
+
+
+class PegaHipError(RuntimeError):
+    """A non-zero status from libpegahip; ``code`` > 0 is a hipError_t."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"[pegahip {code}] {message}")
+        self.code = code
+        self.message = message
+
+
+class InvalidArgument(PegaHipError, ValueError):
+    pass
+
+
+class StorageError(PegaHipError):
+    pass
+
+
+_lib = None
+
+
+def load():
+    """Load libpegahip.so and set every prototype.  Raises if it is absent."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `make -C pegaflow_amd/csrc` "
+            "(or `python -c 'import __graft_entry__ as g; g.build()'`). "
+            "pegaflow_amd has no fallback path.")
+    lib = C.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in PROTOTYPES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def check(status: int) -> None:
+    if status == PF_OK:
+        return
+    msg = load().pf_last_error().decode(errors="replace")
+    if status == PF_ERR_INVALID_ARGUMENT:
+        raise InvalidArgument(status, msg)
+    if status == PF_ERR_STORAGE:
+        raise StorageError(status, msg)
+    raise PegaHipError(status, msg)

@@ -1,0 +1,261 @@
+// gfx950 copy kernels of the KV block transfer path.
+//
+// All of them are pure byte movers bounded by HBM (device <-> device staging)
+// or by the host link (device <-> mapped pinned host memory).  Shape:
+//   * a workgroup is 256 lanes = 4 wavefronts of 64;
+//   * a tile is 256 lanes x U x 16 bytes; every lane issues its U 16-byte
+//     loads before the first store so U global_load_dwordx4 are in flight per
+//     lane, and consecutive lanes touch consecutive 16-byte words, so each
+//     wavefront's access is one 1 KiB contiguous burst;
+//   * loads and stores are non-temporal: the data is touched once;
+//   * all per-tile address arithmetic is wave-uniform (scalar registers).
+#include "pf_kernels.hpp"
+
+#include "pf_common.hpp"
+
+namespace pf {
+
+namespace {
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+// Address-space-1 (global) views, so the compiler emits global_load/store
+// instead of flat accesses for addresses that arrive as integers.
+typedef __attribute__((address_space(1))) u32x4 g_u32x4;
+typedef __attribute__((address_space(1))) unsigned int g_u32;
+typedef __attribute__((address_space(1))) unsigned char g_u8;
+// Address-space-4 (constant) views for the read-only, wave-uniform id list
+// and page table: uniform constant loads become scalar loads.
+typedef __attribute__((address_space(4))) const uint32_t c_u32;
+typedef __attribute__((address_space(4))) const uint64_t c_u64;
+
+constexpr int kLanes = 256;
+
+// Copy `bytes` <= U*4096 from src to dst; both 16-byte aligned.
+template <int U>
+__device__ __forceinline__ void copy_tile_vec(uint64_t dst, uint64_t src, uint32_t bytes) {
+  constexpr uint32_t kTile = U * kLanes * 16;
+  const uint32_t lane = threadIdx.x;
+  const g_u32x4* __restrict__ s = reinterpret_cast<const g_u32x4*>(src);
+  g_u32x4* __restrict__ d = reinterpret_cast<g_u32x4*>(dst);
+  u32x4 v[U];
+  if (bytes == kTile) {
+#pragma unroll
+    for (int k = 0; k < U; ++k) v[k] = __builtin_nontemporal_load(s + lane + k * kLanes);
+#pragma unroll
+    for (int k = 0; k < U; ++k) __builtin_nontemporal_store(v[k], d + lane + k * kLanes);
+    return;
+  }
+  const uint32_t nvec = bytes >> 4;
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t idx = lane + k * kLanes;
+    if (idx < nvec) v[k] = __builtin_nontemporal_load(s + idx);
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t idx = lane + k * kLanes;
+    if (idx < nvec) __builtin_nontemporal_store(v[k], d + idx);
+  }
+  // Fewer than 16 trailing bytes (fragment size not a multiple of 16).
+  const uint32_t j = (nvec << 4) + lane;
+  if (j < bytes) {
+    reinterpret_cast<g_u8*>(dst)[j] = reinterpret_cast<const g_u8*>(src)[j];
+  }
+}
+
+// Copy `bytes` with no alignment assumption: 4-byte words when both sides
+// allow it, single bytes otherwise.
+__device__ __forceinline__ void copy_tile_any(uint64_t dst, uint64_t src, uint32_t bytes) {
+  const uint32_t lane = threadIdx.x;
+  const g_u8* __restrict__ sb = reinterpret_cast<const g_u8*>(src);
+  g_u8* __restrict__ db = reinterpret_cast<g_u8*>(dst);
+  if (((dst | src) & 3ull) == 0) {
+    const uint32_t nword = bytes >> 2;
+    const g_u32* __restrict__ s = reinterpret_cast<const g_u32*>(src);
+    g_u32* __restrict__ d = reinterpret_cast<g_u32*>(dst);
+    for (uint32_t j = lane; j < nword; j += kLanes) d[j] = s[j];
+    for (uint32_t j = (nword << 2) + lane; j < bytes; j += kLanes) db[j] = sb[j];
+  } else {
+    for (uint32_t j = lane; j < bytes; j += kLanes) db[j] = sb[j];
+  }
+}
+
+// Descriptor-table copy: table[3i..3i+2] = dst, src, size.  blockIdx.x strides
+// over descriptors, blockIdx.y over the tiles inside one descriptor, so a
+// batch of few large copies still spreads over the whole chip.
+template <int U>
+__global__ __launch_bounds__(kLanes) void desc_copy_kernel(const uint64_t* __restrict__ table,
+                                                           uint32_t n) {
+  constexpr uint64_t kTile = static_cast<uint64_t>(U) * kLanes * 16;
+  for (uint32_t i = blockIdx.x; i < n; i += gridDim.x) {
+    const uint64_t dst = table[3ull * i + 0];
+    const uint64_t src = table[3ull * i + 1];
+    const uint64_t size = table[3ull * i + 2];
+    const uint64_t n_tiles = (size + kTile - 1) / kTile;
+    const bool vec = ((dst | src) & 15ull) == 0;
+    for (uint64_t t = blockIdx.y; t < n_tiles; t += gridDim.y) {
+      const uint64_t off = t * kTile;
+      const uint64_t left = size - off;
+      const uint32_t bytes = left < kTile ? static_cast<uint32_t>(left) : static_cast<uint32_t>(kTile);
+      if (vec) {
+        copy_tile_vec<U>(dst + off, src + off, bytes);
+      } else {
+        copy_tile_any(dst + off, src + off, bytes);
+      }
+    }
+  }
+}
+
+// Block-ID gather / scatter.  blockIdx.y selects the unit, blockIdx.x strides
+// over its tiles.  Tile order is (segment, list position, tile in fragment),
+// so consecutive workgroups touch consecutive far-side addresses.
+template <int U, bool TO_FAR>
+__global__ __launch_bounds__(kLanes) void block_units_kernel(const BlockUnit* __restrict__ units) {
+  constexpr uint64_t kTile = static_cast<uint64_t>(U) * kLanes * 16;
+  // Every field below is wave-uniform: read once into scalar registers.
+  const BlockUnit* __restrict__ up = units + blockIdx.y;
+  const uint64_t near_base = up->near_base;
+  const uint64_t block_stride = up->block_stride;
+  const uint64_t kv_stride = up->kv_stride;
+  const uint64_t frag_bytes = up->frag_bytes;
+  const uint64_t far_base0 = up->far_base[0];
+  const uint64_t far_base1 = up->far_base[1];
+  const uint64_t far_stride = up->far_stride;
+  c_u32* ids = reinterpret_cast<c_u32*>(reinterpret_cast<uint64_t>(up->ids));
+  c_u64* far_table = reinterpret_cast<c_u64*>(reinterpret_cast<uint64_t>(up->far_table));
+  const bool paged = up->far_table != nullptr;
+  const uint64_t far_table_off = up->far_table_off;
+  const uint32_t tiles_per_frag = up->tiles_per_frag;
+  const bool vec_ok = up->vec_ok != 0;
+  // The host keeps a unit's tile count below 2^32, so 32-bit scalar division.
+  const uint32_t tiles_per_seg = up->n_blocks * tiles_per_frag;
+  const uint32_t n_tiles = tiles_per_seg * up->n_seg;
+  for (uint32_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
+    const uint32_t seg = t >= tiles_per_seg ? 1u : 0u;
+    const uint32_t r = seg ? t - tiles_per_seg : t;
+    // The quotient is wave-uniform; pin it to a scalar register so the id and
+    // page-table reads below are scalar loads.
+    const uint32_t pos = __builtin_amdgcn_readfirstlane(r / tiles_per_frag);
+    const uint32_t c = r - pos * tiles_per_frag;
+    const uint64_t off = static_cast<uint64_t>(c) * kTile;
+    const uint64_t left = frag_bytes - off;
+    const uint32_t bytes = left < kTile ? static_cast<uint32_t>(left) : static_cast<uint32_t>(kTile);
+    const uint64_t id = ids[pos];
+    const uint64_t near_addr = near_base + id * block_stride + (seg ? kv_stride : 0) + off;
+    uint64_t far_addr;
+    if (paged) {
+      far_addr = far_table[pos] + far_table_off + (seg ? frag_bytes : 0) + off;
+    } else {
+      far_addr = (seg ? far_base1 : far_base0) + static_cast<uint64_t>(pos) * far_stride + off;
+    }
+    const uint64_t dst = TO_FAR ? far_addr : near_addr;
+    const uint64_t src = TO_FAR ? near_addr : far_addr;
+    if (vec_ok) {
+      copy_tile_vec<U>(dst, src, bytes);
+    } else {
+      copy_tile_any(dst, src, bytes);
+    }
+  }
+}
+
+template <int U>
+__global__ __launch_bounds__(kLanes) void plain_copy_kernel(uint64_t dst, uint64_t src,
+                                                            uint64_t bytes) {
+  constexpr uint64_t kTile = static_cast<uint64_t>(U) * kLanes * 16;
+  const uint64_t n_tiles = (bytes + kTile - 1) / kTile;
+  for (uint64_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
+    const uint64_t off = t * kTile;
+    const uint64_t left = bytes - off;
+    copy_tile_vec<U>(dst + off, src + off,
+                     left < kTile ? static_cast<uint32_t>(left) : static_cast<uint32_t>(kTile));
+  }
+}
+
+constexpr uint32_t kMaxGridX = 1u << 22;  // the kernels grid-stride past this
+constexpr int kDescUnroll = 4;
+
+}  // namespace
+
+bool unroll_supported(int unroll) { return unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8; }
+
+int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipStream_t s);
+
+int launch_block_units(const BlockUnit* units, uint32_t n_units, uint64_t max_tiles, bool to_far,
+                       int unroll, uint32_t max_workgroups_x, hipStream_t s) {
+  if (n_units == 0 || max_tiles == 0) return PF_OK;
+  if (n_units > 65535u) {
+    return fail(PF_ERR_INVALID_ARGUMENT, "too many units in one launch: %u", n_units);
+  }
+  if (max_tiles > 0x7FFFFFFFull) {
+    return fail(PF_ERR_INVALID_ARGUMENT, "unit of %llu tiles exceeds the kernel limit",
+                static_cast<unsigned long long>(max_tiles));
+  }
+  uint64_t gx = max_tiles < kMaxGridX ? max_tiles : kMaxGridX;
+  if (max_workgroups_x != 0 && gx > max_workgroups_x) gx = max_workgroups_x;
+  dim3 grid(static_cast<uint32_t>(gx), n_units, 1);
+  dim3 block(kLanes, 1, 1);
+#define PF_LAUNCH_UNITS(U_)                                                          \
+  case U_:                                                                           \
+    if (to_far) {                                                                    \
+      hipLaunchKernelGGL((block_units_kernel<U_, true>), grid, block, 0, s, units);  \
+    } else {                                                                         \
+      hipLaunchKernelGGL((block_units_kernel<U_, false>), grid, block, 0, s, units); \
+    }                                                                                \
+    break;
+  switch (unroll) {
+    PF_LAUNCH_UNITS(1)
+    PF_LAUNCH_UNITS(2)
+    PF_LAUNCH_UNITS(4)
+    PF_LAUNCH_UNITS(8)
+    default:
+      return fail(PF_ERR_INVALID_ARGUMENT, "unsupported tile unroll %d", unroll);
+  }
+#undef PF_LAUNCH_UNITS
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail_hip(e, "block_units_kernel launch");
+  return PF_OK;
+}
+
+int launch_plain_copy(void* dst, const void* src, uint64_t bytes, int unroll, hipStream_t s) {
+  if (bytes == 0) return PF_OK;
+  if ((bytes & 15ull) != 0 || (reinterpret_cast<uint64_t>(dst) & 15ull) != 0 ||
+      (reinterpret_cast<uint64_t>(src) & 15ull) != 0) {
+    return fail(PF_ERR_INVALID_ARGUMENT, "plain copy needs 16-byte aligned pointers and size");
+  }
+  const uint64_t tile = tile_bytes(unroll);
+  uint64_t tiles = (bytes + tile - 1) / tile;
+  uint32_t gx = static_cast<uint32_t>(tiles < kMaxGridX ? tiles : kMaxGridX);
+  dim3 grid(gx, 1, 1), block(kLanes, 1, 1);
+  const uint64_t d = reinterpret_cast<uint64_t>(dst);
+  const uint64_t c = reinterpret_cast<uint64_t>(src);
+  switch (unroll) {
+    case 1: hipLaunchKernelGGL(plain_copy_kernel<1>, grid, block, 0, s, d, c, bytes); break;
+    case 2: hipLaunchKernelGGL(plain_copy_kernel<2>, grid, block, 0, s, d, c, bytes); break;
+    case 4: hipLaunchKernelGGL(plain_copy_kernel<4>, grid, block, 0, s, d, c, bytes); break;
+    case 8: hipLaunchKernelGGL(plain_copy_kernel<8>, grid, block, 0, s, d, c, bytes); break;
+    default: return fail(PF_ERR_INVALID_ARGUMENT, "unsupported tile unroll %d", unroll);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail_hip(e, "plain_copy_kernel launch");
+  return PF_OK;
+}
+
+int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipStream_t s) {
+  if (n == 0) return PF_OK;
+  constexpr uint64_t kTile = tile_bytes(kDescUnroll);
+  uint64_t gx = n < kMaxGridX ? n : kMaxGridX;
+  uint64_t gy = (max_size + kTile - 1) / kTile;
+  if (gy < 1) gy = 1;
+  if (gy > 64) gy = 64;
+  // Keep the launch to a few million workgroups; the kernel strides in both
+  // dimensions, so a smaller grid only means more iterations per workgroup.
+  while (gx * gy > (1ull << 22) && gy > 1) gy >>= 1;
+  dim3 grid(static_cast<uint32_t>(gx), static_cast<uint32_t>(gy), 1), block(kLanes, 1, 1);
+  hipLaunchKernelGGL(desc_copy_kernel<kDescUnroll>, grid, block, 0, s, table,
+                     static_cast<uint32_t>(n));
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail_hip(e, "desc_copy_kernel launch");
+  return PF_OK;
+}
+
+}  // namespace pf

@@ -1,0 +1,51 @@
+// Launch interface of the gfx950 copy kernels (implemented in pf_kernels.hip).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace pf {
+
+// One unit of block-ID work, read by the kernel from device memory.
+// "near" is the paged KV cache in HBM; "far" is the other side: mapped pinned
+// host memory (zero-copy) or a device staging buffer (staged).
+//
+// Fragment f = (segment s, list position i) covers
+//   near: near_base + ids[i]*block_stride + s*kv_stride          [frag_bytes]
+//   far : far_table ? far_table[i] + far_table_off + s*frag_bytes
+//                   : far_base[s] + i*far_stride                 [frag_bytes]
+struct BlockUnit {
+  uint64_t near_base;
+  uint64_t block_stride;
+  uint64_t kv_stride;
+  uint64_t frag_bytes;
+  uint64_t far_base[2];
+  uint64_t far_stride;
+  const uint32_t* ids;        // device pointer, n_blocks entries
+  const uint64_t* far_table;  // device pointer or null
+  uint64_t far_table_off;
+  uint32_t n_blocks;
+  uint32_t n_seg;             // fragments per block: 1 or 2
+  uint32_t tiles_per_frag;    // ceil(frag_bytes / tile_bytes)
+  uint32_t vec_ok;            // every address and stride is 16-byte aligned
+};
+
+// Bytes one workgroup moves per tile for the given unroll (256 lanes x 16 B x U).
+constexpr uint32_t tile_bytes(int unroll) { return static_cast<uint32_t>(unroll) * 256u * 16u; }
+
+// Unroll factors the kernels are instantiated for.
+bool unroll_supported(int unroll);
+
+// Launch the block-ID kernel over `n_units` units (grid.y) starting at
+// `units` (device).  `max_tiles` is the largest tile count of any of them;
+// `max_workgroups_x` (0 = no cap) bounds grid.x, the kernel grid-strides.
+// to_far: true = gather near -> far (save), false = scatter far -> near (load).
+int launch_block_units(const BlockUnit* units, uint32_t n_units, uint64_t max_tiles, bool to_far,
+                       int unroll, uint32_t max_workgroups_x, hipStream_t s);
+
+// Plain device copy kernel of the same tile shape, for calibrating counters
+// and measuring the HBM copy ceiling: copies `bytes` (multiple of 16).
+int launch_plain_copy(void* dst, const void* src, uint64_t bytes, int unroll, hipStream_t s);
+
+}  // namespace pf

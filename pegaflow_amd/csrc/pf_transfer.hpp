@@ -1,0 +1,95 @@
+// Copy descriptors, the merge rule, descriptor construction and the two
+// reference-compatible transfer backends.  Follows
+// pegaflow-core/src/transfer/{mod,memcpy,kernel}.rs and
+// pegaflow-core/src/gpu_worker.rs:353-423 of the reference.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "../../include/pegahip.h"
+#include "pf_layout.hpp"
+
+namespace pf {
+
+using CopyDesc = pf_copy_desc;       // transfer/mod.rs:36-44
+using MergedRange = pf_merged_range; // transfer/memcpy.rs:16-20
+
+// transfer/mod.rs:62-76.
+enum class TransferMode : int { Direct = PF_MODE_DIRECT, Kernel = PF_MODE_KERNEL };
+
+// transfer/memcpy.rs:25-55: greedy left-to-right join of list-adjacent copies
+// that share both allocations and are contiguous on both sides.
+std::vector<MergedRange> merge(const CopyDesc* copies, uint64_t n);
+
+// gpu_worker.rs:353-423.  Returns false with *err = "layer <name>: <cause>".
+bool build_copy_descs(const pf_layer_transfer* layers, uint64_t n_layers,
+                      std::vector<CopyDesc>* out, uint64_t* total_bytes, std::string* err);
+
+// A pinned host slab with a device twin, recycled once the stream work that
+// reads it has finished.  Used for descriptor tables and block-id lists.
+class SlabPool {
+ public:
+  struct Slab {
+    void* host = nullptr;
+    void* dev = nullptr;
+    uint64_t cap = 0;
+    hipEvent_t done = nullptr;
+    bool in_flight = false;
+  };
+  ~SlabPool();
+  // A slab of at least `bytes` whose previous use (if any) has completed.
+  int acquire(uint64_t bytes, Slab** out);
+  // Mark the slab busy until everything enqueued on `s` so far has run.
+  int release_after(Slab* slab, hipStream_t s);
+
+ private:
+  std::vector<std::unique_ptr<Slab>> slabs_;
+};
+
+// transfer/mod.rs:53-60.
+class TransferBackend {
+ public:
+  virtual ~TransferBackend() = default;
+  virtual int h2d(const CopyDesc* copies, uint64_t n, hipStream_t s) = 0;
+  virtual int d2h(const CopyDesc* copies, uint64_t n, hipStream_t s) = 0;
+  virtual const char* name() const = 0;
+};
+
+// transfer/memcpy.rs:57-102: one DMA copy per merged range.
+class MemcpyBackend : public TransferBackend {
+ public:
+  int h2d(const CopyDesc* copies, uint64_t n, hipStream_t s) override;
+  int d2h(const CopyDesc* copies, uint64_t n, hipStream_t s) override;
+  const char* name() const override { return "direct"; }
+};
+
+// transfer/kernel.rs:51-151: one kernel launch for the whole batch, host side
+// addressed through its device-visible mapping.
+class KernelBackend : public TransferBackend {
+ public:
+  int h2d(const CopyDesc* copies, uint64_t n, hipStream_t s) override {
+    return submit(copies, n, true, s);
+  }
+  int d2h(const CopyDesc* copies, uint64_t n, hipStream_t s) override {
+    return submit(copies, n, false, s);
+  }
+  const char* name() const override { return "kernel"; }
+
+ private:
+  int submit(const CopyDesc* copies, uint64_t n, bool host_is_src, hipStream_t s);
+  SlabPool slabs_;
+};
+
+// gpu_worker.rs:264-276.
+std::unique_ptr<TransferBackend> build_backend(TransferMode mode);
+
+// Launch the descriptor-table copy kernel: `table` is a device array of
+// 3*n u64 words [dst, src, size].  `max_size` is the largest size in it.
+int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipStream_t s);
+
+}  // namespace pf

@@ -1,0 +1,639 @@
+// Block-ID gather / scatter engine: the MI355X fast path of the KV transfer.
+//
+// It moves the same bytes as descriptor construction + a transfer backend
+// (pegaflow-core/src/gpu_worker.rs:353-423 + transfer/{memcpy,kernel}.rs in
+// the reference) without a per-fragment descriptor: per layer it uploads the
+// block-id list once and the kernels derive every address from
+// `data_ptr + id*block_stride (+ kv_stride)`.
+//
+// Two ways across the host link, chosen per layer:
+//   zero-copy : one kernel reads/writes the mapped pinned host image directly;
+//   staged    : a gather kernel packs the selected blocks into a device staging
+//               slot (HBM-bound, microseconds), then one DMA copy per segment
+//               drains the slot to the host image on a side stream while the
+//               next slot is being packed (and the mirror image for loads).
+#include <algorithm>
+#include <cstring>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "pf_common.hpp"
+#include "pf_kernels.hpp"
+#include "pf_layout.hpp"
+#include "pf_transfer.hpp"
+
+namespace pf {
+
+namespace {
+
+constexpr uint64_t kDefaultSlotBytes = 64ull << 20;
+constexpr uint32_t kDefaultSlots = 3;
+constexpr uint64_t kDefaultAutoStagedMin = 4ull << 20;
+constexpr int kDefaultUnroll = 4;
+
+bool aligned16(uint64_t v) { return (v & 15ull) == 0; }
+
+struct LayerPlan {
+  std::string name;
+  KVCacheLayout layout;
+  uint64_t frag_bytes = 0;
+  uint32_t n_seg = 0;
+  uint64_t n_blocks = 0;
+  const uint32_t* ids = nullptr;
+  uint8_t* host[2] = {nullptr, nullptr};
+  uint64_t host_dev[2] = {0, 0};
+  uint64_t host_stride = 0;
+  const uint64_t* page_dev = nullptr;  // device-visible page bases, host array
+  uint64_t page_offset = 0;
+  bool staged = false;
+  bool vec_ok = false;
+  uint64_t ids_slab_off = 0;    // byte offset of the id list inside the slab
+  uint64_t table_slab_off = 0;  // byte offset of the page table inside the slab
+  uint64_t layer_bytes = 0;
+  size_t src_index = 0;         // index in the caller's layer array
+};
+
+}  // namespace
+
+class Xfer {
+ public:
+  explicit Xfer(const pf_xfer_config* cfg) {
+    if (cfg) {
+      if (cfg->staging_slot_bytes) slot_bytes_ = cfg->staging_slot_bytes;
+      if (cfg->staging_slots) n_slots_ = cfg->staging_slots;
+      zc_max_wg_ = cfg->zerocopy_max_workgroups;
+      if (cfg->auto_staged_min_bytes) auto_min_ = cfg->auto_staged_min_bytes;
+      if (cfg->tile_unroll) unroll_ = static_cast<int>(cfg->tile_unroll);
+    }
+  }
+
+  ~Xfer() {
+    if (side_) {
+      (void)hipStreamSynchronize(side_);
+      (void)hipStreamDestroy(side_);
+    }
+    for (auto& sl : slots_) {
+      if (sl.ready) (void)hipEventDestroy(sl.ready);
+      if (sl.freed) (void)hipEventDestroy(sl.freed);
+      if (sl.buf) (void)hipFree(sl.buf);
+    }
+    if (fork_) (void)hipEventDestroy(fork_);
+    if (join_) (void)hipEventDestroy(join_);
+    for (auto& p : timing_pool_) {
+      (void)hipEventDestroy(p.first);
+      (void)hipEventDestroy(p.second);
+    }
+    (void)hipGetLastError();
+  }
+
+  int init() {
+    if (!unroll_supported(unroll_)) {
+      return fail(PF_ERR_INVALID_ARGUMENT, "tile_unroll must be 1, 2, 4 or 8, got %d", unroll_);
+    }
+    if (n_slots_ < 2 || n_slots_ > 16) {
+      return fail(PF_ERR_INVALID_ARGUMENT, "staging_slots must be in [2, 16], got %u", n_slots_);
+    }
+    hipError_t e = hipGetDevice(&device_);
+    if (e != hipSuccess) {
+      fail_hip(e, "hipGetDevice");
+      return fail(PF_ERR_DEVICE_INIT, "transfer engine init failed: %s", last_error().c_str());
+    }
+    PF_HIP(hipStreamCreateWithFlags(&side_, hipStreamNonBlocking));
+    PF_HIP(hipEventCreateWithFlags(&fork_, hipEventDisableTiming));
+    PF_HIP(hipEventCreateWithFlags(&join_, hipEventDisableTiming));
+    slots_.resize(n_slots_);
+    for (auto& sl : slots_) {
+      PF_HIP(hipEventCreateWithFlags(&sl.ready, hipEventDisableTiming));
+      PF_HIP(hipEventCreateWithFlags(&sl.freed, hipEventDisableTiming));
+    }
+    return PF_OK;
+  }
+
+  int run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save, hipStream_t s);
+
+  void set_layer_events(pf_event_t* events, uint64_t n) {
+    layer_events_.clear();
+    if (events) {
+      for (uint64_t i = 0; i < n; ++i) layer_events_.push_back(native(events[i]));
+    }
+  }
+  int last_path() const { return last_path_; }
+  void set_timing(bool on) { timing_ = on; }
+  int last_kernel_ms(float* out_ms, uint32_t* out_launches);
+
+ private:
+  struct Slot {
+    void* buf = nullptr;
+    uint64_t cap = 0;
+    hipEvent_t ready = nullptr;  // contents complete (gather done / fill done)
+    hipEvent_t freed = nullptr;  // contents consumed (drain done / scatter done)
+    bool used = false;
+  };
+
+  int plan_layer(const pf_layer_blocks& in, size_t index, int path, LayerPlan* out, bool* skip);
+  int ensure_slot(Slot& sl, uint64_t bytes);
+  int launch(const BlockUnit* dev_units, uint32_t n_units, uint64_t max_tiles, bool to_far,
+             uint32_t max_wg, hipStream_t s);
+
+  int device_ = 0;
+  uint64_t slot_bytes_ = kDefaultSlotBytes;
+  uint32_t n_slots_ = kDefaultSlots;
+  uint32_t zc_max_wg_ = 0;
+  uint64_t auto_min_ = kDefaultAutoStagedMin;
+  int unroll_ = kDefaultUnroll;
+
+  hipStream_t side_ = nullptr;
+  hipEvent_t fork_ = nullptr;
+  hipEvent_t join_ = nullptr;
+  std::vector<Slot> slots_;
+  uint32_t next_slot_ = 0;
+  SlabPool slabs_;
+  std::vector<hipEvent_t> layer_events_;
+  int last_path_ = 0;
+
+  bool timing_ = false;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> timing_pool_;
+  size_t timing_used_ = 0;
+};
+
+int Xfer::ensure_slot(Slot& sl, uint64_t bytes) {
+  if (sl.cap >= bytes) return PF_OK;
+  if (sl.buf) {
+    // Grow-only: the old buffer may still be in flight.
+    if (sl.used) PF_HIP(hipEventSynchronize(sl.freed));
+    PF_HIP(hipFree(sl.buf));
+    sl.buf = nullptr;
+    sl.cap = 0;
+    sl.used = false;
+  }
+  uint64_t cap = std::max(bytes, slot_bytes_);
+  PF_HIP(hipMalloc(&sl.buf, cap));
+  sl.cap = cap;
+  return PF_OK;
+}
+
+int Xfer::launch(const BlockUnit* dev_units, uint32_t n_units, uint64_t max_tiles, bool to_far,
+                 uint32_t max_wg, hipStream_t s) {
+  if (timing_) {
+    if (timing_used_ == timing_pool_.size()) {
+      hipEvent_t a = nullptr, b = nullptr;
+      PF_HIP(hipEventCreate(&a));
+      PF_HIP(hipEventCreate(&b));
+      timing_pool_.emplace_back(a, b);
+    }
+    PF_HIP(hipEventRecord(timing_pool_[timing_used_].first, s));
+  }
+  int st = launch_block_units(dev_units, n_units, max_tiles, to_far, unroll_, max_wg, s);
+  if (st != PF_OK) return st;
+  if (timing_) {
+    PF_HIP(hipEventRecord(timing_pool_[timing_used_].second, s));
+    ++timing_used_;
+  }
+  return PF_OK;
+}
+
+int Xfer::last_kernel_ms(float* out_ms, uint32_t* out_launches) {
+  float total = 0.f;
+  for (size_t i = 0; i < timing_used_; ++i) {
+    PF_HIP(hipEventSynchronize(timing_pool_[i].second));
+    float ms = 0.f;
+    PF_HIP(hipEventElapsedTime(&ms, timing_pool_[i].first, timing_pool_[i].second));
+    total += ms;
+  }
+  *out_ms = total;
+  *out_launches = static_cast<uint32_t>(timing_used_);
+  return PF_OK;
+}
+
+int Xfer::plan_layer(const pf_layer_blocks& in, size_t index, int path, LayerPlan* out,
+                     bool* skip) {
+  LayerPlan& p = *out;
+  p.src_index = index;
+  p.name = in.layer_name ? in.layer_name : ("#" + std::to_string(index));
+  *skip = false;
+  std::string cause;
+  if (!KVCacheLayout::from_c(in.layout, &p.layout, &cause)) {
+    return fail(PF_ERR_STORAGE, "layer %s: %s", p.name.c_str(), cause.c_str());
+  }
+  if (in.n_blocks == 0) {
+    *skip = true;
+    return PF_OK;
+  }
+  if (!in.block_ids) {
+    return fail(PF_ERR_INVALID_ARGUMENT, "layer %s: block_ids must not be null", p.name.c_str());
+  }
+  if (in.n_blocks > 0xFFFFFFFFull) {
+    return fail(PF_ERR_INVALID_ARGUMENT, "layer %s: too many blocks (%llu)", p.name.c_str(),
+                static_cast<unsigned long long>(in.n_blocks));
+  }
+  p.n_blocks = in.n_blocks;
+  p.ids = in.block_ids;
+  const uint64_t num_blocks = p.layout.num_blocks();
+  for (uint64_t i = 0; i < p.n_blocks; ++i) {
+    if (p.ids[i] >= num_blocks) {
+      // Same wording as KVCacheLayout::block_copies wrapped by the worker
+      // (layout.rs:232-237, gpu_worker.rs:363-366).
+      return fail(PF_ERR_STORAGE, "layer %s: block %u out of range (%llu blocks)", p.name.c_str(),
+                  p.ids[i], static_cast<unsigned long long>(num_blocks));
+    }
+  }
+  p.frag_bytes = p.layout.fragment_bytes();
+  p.n_seg = p.layout.fragments_per_block();
+  p.layer_bytes = p.frag_bytes * p.n_seg * p.n_blocks;
+
+  const bool paged = in.page_host != nullptr || in.page_host_device != nullptr;
+  bool far_aligned = true;
+  if (paged) {
+    if (!in.page_host || !in.page_host_device) {
+      return fail(PF_ERR_INVALID_ARGUMENT,
+                  "layer %s: page_host and page_host_device must both be set", p.name.c_str());
+    }
+    uint64_t need = 0;
+    if (__builtin_add_overflow(in.page_offset, p.frag_bytes * p.n_seg, &need) ||
+        need > in.page_len) {
+      return fail(PF_ERR_INVALID_ARGUMENT,
+                  "layer %s: page slice [%llu, +%llu) exceeds page length %llu", p.name.c_str(),
+                  static_cast<unsigned long long>(in.page_offset),
+                  static_cast<unsigned long long>(p.frag_bytes * p.n_seg),
+                  static_cast<unsigned long long>(in.page_len));
+    }
+    for (uint64_t i = 0; i < p.n_blocks; ++i) {
+      if (in.page_host[i] == 0 || in.page_host_device[i] == 0) {
+        return fail(PF_ERR_INVALID_ARGUMENT, "layer %s: page %llu has a null base",
+                    p.name.c_str(), static_cast<unsigned long long>(i));
+      }
+      far_aligned = far_aligned && aligned16(in.page_host_device[i]);
+    }
+    far_aligned = far_aligned && aligned16(in.page_offset);
+    p.page_dev = in.page_host_device;
+    p.page_offset = in.page_offset;
+  } else {
+    if (in.host_stride < p.frag_bytes) {
+      return fail(PF_ERR_INVALID_ARGUMENT,
+                  "layer %s: host_stride %llu < fragment size %llu: host images would overlap",
+                  p.name.c_str(), static_cast<unsigned long long>(in.host_stride),
+                  static_cast<unsigned long long>(p.frag_bytes));
+    }
+    p.host_stride = in.host_stride;
+    for (uint32_t sgm = 0; sgm < p.n_seg; ++sgm) {
+      if (!in.host[sgm] || in.host_device[sgm] == 0) {
+        return fail(PF_ERR_INVALID_ARGUMENT, "layer %s: host segment %u is null", p.name.c_str(),
+                    sgm);
+      }
+      uint64_t need = (p.n_blocks - 1) * in.host_stride + p.frag_bytes;
+      if (need > in.host_len[sgm]) {
+        return fail(PF_ERR_INVALID_ARGUMENT,
+                    "layer %s: host segment %u needs %llu bytes, has %llu", p.name.c_str(), sgm,
+                    static_cast<unsigned long long>(need),
+                    static_cast<unsigned long long>(in.host_len[sgm]));
+      }
+      p.host[sgm] = static_cast<uint8_t*>(in.host[sgm]);
+      p.host_dev[sgm] = in.host_device[sgm];
+      far_aligned = far_aligned && aligned16(in.host_device[sgm]);
+    }
+    far_aligned = far_aligned && aligned16(in.host_stride);
+  }
+  const bool near_aligned = aligned16(p.layout.data_ptr()) &&
+                            aligned16(p.layout.block_stride_bytes()) &&
+                            aligned16(p.layout.kv_stride_bytes());
+  // A fragment size that is not a multiple of 16 is fine for the vector path
+  // (the kernel copies the tail bytewise) as long as every fragment START is
+  // aligned, which the stride checks above guarantee.
+  p.vec_ok = near_aligned && far_aligned && (p.n_seg == 1 || !paged || aligned16(p.frag_bytes));
+
+  const bool dense = !paged && in.host_stride == p.frag_bytes;
+  switch (path) {
+    case PF_PATH_ZEROCOPY:
+      p.staged = false;
+      break;
+    case PF_PATH_STAGED:
+      if (!dense) {
+        return fail(PF_ERR_INVALID_ARGUMENT,
+                    "layer %s: the staged path needs a dense host image (host_stride == fragment "
+                    "size, no page table)",
+                    p.name.c_str());
+      }
+      p.staged = true;
+      break;
+    case PF_PATH_AUTO:
+      p.staged = dense && p.layer_bytes >= auto_min_;
+      break;
+    default:
+      return fail(PF_ERR_INVALID_ARGUMENT, "unknown transfer path %d", path);
+  }
+  return PF_OK;
+}
+
+int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save,
+              hipStream_t s) {
+  timing_used_ = 0;
+  if (n_layers == 0) return PF_OK;
+  if (!layers) return fail(PF_ERR_INVALID_ARGUMENT, "layers must not be null");
+  if (!layer_events_.empty() && layer_events_.size() < n_layers) {
+    return fail(PF_ERR_INVALID_ARGUMENT, "%zu layer events set, call has %llu layers",
+                layer_events_.size(), static_cast<unsigned long long>(n_layers));
+  }
+
+  // ---- 1. validate everything before touching the stream ----------------
+  std::vector<LayerPlan> plans;
+  plans.reserve(n_layers);
+  for (uint64_t li = 0; li < n_layers; ++li) {
+    LayerPlan p;
+    bool skip = false;
+    int st = plan_layer(layers[li], li, path, &p, &skip);
+    if (st != PF_OK) return st;
+    if (!skip) plans.push_back(std::move(p));
+  }
+  const bool want_events = !layer_events_.empty();
+  if (plans.empty()) {
+    // Nothing to move: layers' events still fire so a waiter is released.
+    if (want_events) {
+      for (uint64_t li = 0; li < n_layers; ++li) PF_HIP(hipEventRecord(layer_events_[li], s));
+    }
+    return PF_OK;
+  }
+  last_path_ = plans.front().staged ? PF_PATH_STAGED : PF_PATH_ZEROCOPY;
+
+  // ---- 2. lay out the slab: units, id lists, page tables ----------------
+  const uint32_t tile = tile_bytes(unroll_);
+  struct UnitRef {
+    size_t plan;
+    uint64_t first;  // first list position
+    uint64_t count;
+  };
+  std::vector<UnitRef> unit_refs;
+  uint64_t max_unit_bytes = 0;
+  for (size_t pi = 0; pi < plans.size(); ++pi) {
+    LayerPlan& p = plans[pi];
+    if (!p.staged) {
+      unit_refs.push_back({pi, 0, p.n_blocks});
+      continue;
+    }
+    const uint64_t block_bytes = p.frag_bytes * p.n_seg;
+    uint64_t per_unit = std::max<uint64_t>(slot_bytes_ / block_bytes, 1);
+    for (uint64_t first = 0; first < p.n_blocks; first += per_unit) {
+      uint64_t count = std::min(per_unit, p.n_blocks - first);
+      unit_refs.push_back({pi, first, count});
+      max_unit_bytes = std::max(max_unit_bytes, count * block_bytes);
+    }
+  }
+  uint64_t slab_bytes = unit_refs.size() * sizeof(BlockUnit);
+  slab_bytes = (slab_bytes + 255) & ~255ull;
+  for (size_t pi = 0; pi < plans.size(); ++pi) {
+    LayerPlan& p = plans[pi];
+    // Layers that pass the very same id array share one upload.
+    bool shared = false;
+    for (size_t pj = 0; pj < pi; ++pj) {
+      if (plans[pj].ids == p.ids && plans[pj].n_blocks == p.n_blocks) {
+        p.ids_slab_off = plans[pj].ids_slab_off;
+        shared = true;
+        break;
+      }
+    }
+    if (!shared) {
+      p.ids_slab_off = slab_bytes;
+      slab_bytes += (p.n_blocks * sizeof(uint32_t) + 255) & ~255ull;
+    }
+    if (p.page_dev) {
+      bool tshared = false;
+      for (size_t pj = 0; pj < pi; ++pj) {
+        if (plans[pj].page_dev == p.page_dev && plans[pj].n_blocks == p.n_blocks) {
+          p.table_slab_off = plans[pj].table_slab_off;
+          tshared = true;
+          break;
+        }
+      }
+      if (!tshared) {
+        p.table_slab_off = slab_bytes;
+        slab_bytes += (p.n_blocks * sizeof(uint64_t) + 255) & ~255ull;
+      }
+    }
+  }
+  SlabPool::Slab* slab = nullptr;
+  int st = slabs_.acquire(slab_bytes, &slab);
+  if (st != PF_OK) return st;
+  uint8_t* slab_host = static_cast<uint8_t*>(slab->host);
+  const uint64_t slab_dev = reinterpret_cast<uint64_t>(slab->dev);
+  for (size_t pi = 0; pi < plans.size(); ++pi) {
+    LayerPlan& p = plans[pi];
+    std::memcpy(slab_host + p.ids_slab_off, p.ids, p.n_blocks * sizeof(uint32_t));
+    if (p.page_dev) {
+      std::memcpy(slab_host + p.table_slab_off, p.page_dev, p.n_blocks * sizeof(uint64_t));
+    }
+  }
+
+  // ---- 3. staging slots ---------------------------------------------------
+  std::vector<uint32_t> unit_slot(unit_refs.size(), 0);
+  if (max_unit_bytes != 0) {
+    for (auto& sl : slots_) {
+      st = ensure_slot(sl, max_unit_bytes);
+      if (st != PF_OK) return st;
+    }
+  }
+  BlockUnit* units_host = reinterpret_cast<BlockUnit*>(slab_host);
+  const BlockUnit* units_dev = reinterpret_cast<const BlockUnit*>(slab_dev);
+  uint32_t slot_cursor = next_slot_;
+  for (size_t ui = 0; ui < unit_refs.size(); ++ui) {
+    const UnitRef& r = unit_refs[ui];
+    const LayerPlan& p = plans[r.plan];
+    BlockUnit& u = units_host[ui];
+    std::memset(&u, 0, sizeof(u));
+    u.near_base = p.layout.data_ptr();
+    u.block_stride = p.layout.block_stride_bytes();
+    u.kv_stride = p.layout.kv_stride_bytes();
+    u.frag_bytes = p.frag_bytes;
+    u.ids = reinterpret_cast<const uint32_t*>(slab_dev + p.ids_slab_off) + r.first;
+    u.n_blocks = static_cast<uint32_t>(r.count);
+    u.n_seg = p.n_seg;
+    u.tiles_per_frag = static_cast<uint32_t>((p.frag_bytes + tile - 1) / tile);
+    if (p.staged) {
+      uint32_t slot = slot_cursor;
+      slot_cursor = (slot_cursor + 1) % n_slots_;
+      unit_slot[ui] = slot;
+      const uint64_t base = reinterpret_cast<uint64_t>(slots_[slot].buf);
+      u.far_base[0] = base;
+      u.far_base[1] = base + r.count * p.frag_bytes;
+      u.far_stride = p.frag_bytes;
+      // Staging is 256-byte aligned device memory; only the near side and the
+      // fragment size decide whether 16-byte vectors are safe.
+      u.vec_ok = aligned16(p.layout.data_ptr()) && aligned16(p.layout.block_stride_bytes()) &&
+                 aligned16(p.layout.kv_stride_bytes()) && aligned16(p.frag_bytes);
+    } else {
+      if (p.page_dev) {
+        u.far_table = reinterpret_cast<const uint64_t*>(slab_dev + p.table_slab_off);
+        u.far_table_off = p.page_offset;
+      } else {
+        u.far_base[0] = p.host_dev[0];
+        u.far_base[1] = p.host_dev[1];
+        u.far_stride = p.host_stride;
+      }
+      u.vec_ok = p.vec_ok ? 1 : 0;
+    }
+  }
+  next_slot_ = slot_cursor;
+
+  // ---- 4. enqueue ---------------------------------------------------------
+  PF_HIP(hipMemcpyAsync(slab->dev, slab->host, slab_bytes, hipMemcpyHostToDevice, s));
+  bool side_used = false;
+  auto fork_side = [&]() -> int {
+    if (side_used) return PF_OK;
+    PF_HIP(hipEventRecord(fork_, s));
+    PF_HIP(hipStreamWaitEvent(side_, fork_, 0));
+    side_used = true;
+    return PF_OK;
+  };
+  auto tiles_of = [&](const BlockUnit& u) -> uint64_t {
+    return static_cast<uint64_t>(u.n_blocks) * u.tiles_per_frag * u.n_seg;
+  };
+  // Skipped (empty) layers fire their event at the position of the next
+  // planned layer; track the caller index we have fired up to.
+  uint64_t events_fired = 0;
+  auto fire_events_through = [&](uint64_t caller_index, hipStream_t on) -> int {
+    if (!want_events) return PF_OK;
+    for (; events_fired <= caller_index; ++events_fired) {
+      PF_HIP(hipEventRecord(layer_events_[events_fired], on));
+    }
+    return PF_OK;
+  };
+
+  size_t ui = 0;
+  while (ui < unit_refs.size()) {
+    const LayerPlan& p = plans[unit_refs[ui].plan];
+    if (!p.staged) {
+      // Batch consecutive zero-copy layers into one launch unless the caller
+      // wants a completion event per layer.
+      size_t uj = ui + 1;
+      uint64_t max_tiles = tiles_of(units_host[ui]);
+      if (!want_events) {
+        while (uj < unit_refs.size() && !plans[unit_refs[uj].plan].staged && uj - ui < 65535) {
+          max_tiles = std::max(max_tiles, tiles_of(units_host[uj]));
+          ++uj;
+        }
+      }
+      st = launch(units_dev + ui, static_cast<uint32_t>(uj - ui), max_tiles, save, zc_max_wg_, s);
+      if (st != PF_OK) return st;
+      st = fire_events_through(plans[unit_refs[uj - 1].plan].src_index, s);
+      if (st != PF_OK) return st;
+      ui = uj;
+      continue;
+    }
+
+    // Staged unit.
+    st = fork_side();
+    if (st != PF_OK) return st;
+    const UnitRef& r = unit_refs[ui];
+    Slot& sl = slots_[unit_slot[ui]];
+    const BlockUnit& u = units_host[ui];
+    const bool last_of_layer =
+        ui + 1 == unit_refs.size() || unit_refs[ui + 1].plan != unit_refs[ui].plan;
+    if (save) {
+      if (sl.used) PF_HIP(hipStreamWaitEvent(s, sl.freed, 0));
+      st = launch(units_dev + ui, 1, tiles_of(u), true, 0, s);
+      if (st != PF_OK) return st;
+      PF_HIP(hipEventRecord(sl.ready, s));
+      PF_HIP(hipStreamWaitEvent(side_, sl.ready, 0));
+      for (uint32_t sgm = 0; sgm < p.n_seg; ++sgm) {
+        PF_HIP(hipMemcpyAsync(p.host[sgm] + r.first * p.host_stride,
+                              reinterpret_cast<const void*>(u.far_base[sgm]),
+                              r.count * p.frag_bytes, hipMemcpyDeviceToHost, side_));
+      }
+      PF_HIP(hipEventRecord(sl.freed, side_));
+      sl.used = true;
+      if (last_of_layer) {
+        st = fire_events_through(p.src_index, side_);
+        if (st != PF_OK) return st;
+      }
+    } else {
+      if (sl.used) PF_HIP(hipStreamWaitEvent(side_, sl.freed, 0));
+      for (uint32_t sgm = 0; sgm < p.n_seg; ++sgm) {
+        PF_HIP(hipMemcpyAsync(reinterpret_cast<void*>(u.far_base[sgm]),
+                              p.host[sgm] + r.first * p.host_stride, r.count * p.frag_bytes,
+                              hipMemcpyHostToDevice, side_));
+      }
+      PF_HIP(hipEventRecord(sl.ready, side_));
+      PF_HIP(hipStreamWaitEvent(s, sl.ready, 0));
+      st = launch(units_dev + ui, 1, tiles_of(u), false, 0, s);
+      if (st != PF_OK) return st;
+      PF_HIP(hipEventRecord(sl.freed, s));
+      sl.used = true;
+      if (last_of_layer) {
+        st = fire_events_through(p.src_index, s);
+        if (st != PF_OK) return st;
+      }
+    }
+    ++ui;
+  }
+  if (side_used && save) {
+    // Join: everything the side stream drained is ordered before whatever the
+    // caller enqueues (or records) next on its stream.
+    PF_HIP(hipEventRecord(join_, side_));
+    PF_HIP(hipStreamWaitEvent(s, join_, 0));
+  }
+  // Trailing empty layers.
+  if (want_events && events_fired < n_layers) {
+    st = fire_events_through(n_layers - 1, s);
+    if (st != PF_OK) return st;
+  }
+  return slabs_.release_after(slab, s);
+}
+
+}  // namespace pf
+
+extern "C" {
+
+int pf_xfer_create(const pf_xfer_config* cfg, pf_xfer_t* out) {
+  PF_REQUIRE_PTR(out);
+  std::unique_ptr<pf::Xfer> x(new pf::Xfer(cfg));
+  int st = x->init();
+  if (st != PF_OK) return st;
+  *out = reinterpret_cast<pf_xfer_t>(x.release());
+  return PF_OK;
+}
+
+int pf_xfer_destroy(pf_xfer_t x) {
+  delete reinterpret_cast<pf::Xfer*>(x);
+  return PF_OK;
+}
+
+int pf_xfer_save(pf_xfer_t x, const pf_layer_blocks* layers, uint64_t n_layers, int path,
+                 pf_stream_t s) {
+  PF_REQUIRE_PTR(x);
+  return reinterpret_cast<pf::Xfer*>(x)->run(layers, n_layers, path, true, pf::native(s));
+}
+
+int pf_xfer_load(pf_xfer_t x, const pf_layer_blocks* layers, uint64_t n_layers, int path,
+                 pf_stream_t s) {
+  PF_REQUIRE_PTR(x);
+  return reinterpret_cast<pf::Xfer*>(x)->run(layers, n_layers, path, false, pf::native(s));
+}
+
+int pf_xfer_set_layer_events(pf_xfer_t x, pf_event_t* events, uint64_t n) {
+  PF_REQUIRE_PTR(x);
+  reinterpret_cast<pf::Xfer*>(x)->set_layer_events(events, n);
+  return PF_OK;
+}
+
+int pf_xfer_last_path(pf_xfer_t x) { return x ? reinterpret_cast<pf::Xfer*>(x)->last_path() : 0; }
+
+int pf_xfer_last_kernel_ms(pf_xfer_t x, float* out_ms, uint32_t* out_launches) {
+  PF_REQUIRE_PTR(x);
+  PF_REQUIRE_PTR(out_ms);
+  PF_REQUIRE_PTR(out_launches);
+  return reinterpret_cast<pf::Xfer*>(x)->last_kernel_ms(out_ms, out_launches);
+}
+
+int pf_plain_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t tile_unroll,
+                  pf_stream_t s) {
+  int unroll = tile_unroll ? static_cast<int>(tile_unroll) : 4;
+  return pf::launch_plain_copy(reinterpret_cast<void*>(dst), reinterpret_cast<const void*>(src),
+                               bytes, unroll, pf::native(s));
+}
+
+int pf_xfer_set_kernel_timing(pf_xfer_t x, int enable) {
+  PF_REQUIRE_PTR(x);
+  reinterpret_cast<pf::Xfer*>(x)->set_timing(enable != 0);
+  return PF_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,334 @@
+"""GPU parity of the block-ID gather/scatter path (pf_xfer_save / pf_xfer_load)
+against the CPU oracle, for both link paths (zero-copy and staged) and every
+layout the reference supports: K/V split, contiguous (MLA), adjacent K/V,
+strided fused buffer, padded host strides, page-first pages."""
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from pegaflow_amd import _lib
+from pegaflow_amd.layout import KVCacheLayout
+from pegaflow_amd.runtime import DeviceBuffer, Event, PinnedMemory, Stream
+from pegaflow_amd.transfer import BlockTransfer, LayerBlocks, TransferPath
+from tests.helpers import random_bytes
+
+pytestmark = pytest.mark.gpu
+
+ZC, ST = TransferPath.ZEROCOPY, TransferPath.STAGED
+SENT = 0xC3
+
+
+@pytest.fixture(scope="module")
+def stream(gpu):
+    s = Stream()
+    yield s
+    s.close()
+
+
+@pytest.fixture(scope="module")
+def xfer(gpu):
+    # Small staging slots so that modest test sizes already span several
+    # units and reuse slots.
+    x = BlockTransfer(staging_slot_bytes=1 << 20, staging_slots=2)
+    yield x
+    x.close()
+
+
+class Case:
+    """One layer: device cache + host image, mirrored for product and oracle."""
+
+    def __init__(self, rng, num_blocks, seg, segments, kv_stride=None, block_stride=None,
+                 pad_to=None, n_ids=None, base_off=0):
+        self.seg, self.segments, self.num_blocks = seg, segments, num_blocks
+        if segments == 2 and kv_stride is None:
+            kv_stride = num_blocks * (block_stride or seg)
+        kv = kv_stride or 0
+        probe = O.Layout(0x1000, 1 << 40, num_blocks, seg, kv, segments)
+        if block_stride:
+            probe.with_block_stride(block_stride)
+        stride = probe.c.block_stride_bytes
+        frag = probe.fragment_bytes
+        self.size = (num_blocks - 1) * stride + frag + (kv if probe.is_split else 0)
+        self.base_off = base_off
+        self.cache0 = random_bytes(rng, self.size + base_off)
+        self.dev = DeviceBuffer(self.size + base_off)
+        self.args = (self.size, num_blocks, seg, kv, segments)
+        self.block_stride = block_stride
+        self.pad_to = pad_to
+        n_ids = n_ids if n_ids is not None else max(1, num_blocks // 2)
+        self.ids = rng.choice(num_blocks, n_ids, replace=False).astype(np.uint32)
+
+    def product_layout(self):
+        L = KVCacheLayout(self.dev.ptr + self.base_off, *self.args)
+        if self.block_stride:
+            L.with_block_stride(self.block_stride)
+        if self.pad_to:
+            L.with_ssd_padding(self.pad_to)
+        return L
+
+    def oracle_layout(self, cache):
+        L = O.Layout(cache.ctypes.data + self.base_off, *self.args)
+        if self.block_stride:
+            L.with_block_stride(self.block_stride)
+        if self.pad_to:
+            L.with_ssd_padding(self.pad_to)
+        return L
+
+    def close(self):
+        self.dev.close()
+
+
+def _dense_layer(case, L, host, ids):
+    """LayerBlocks over the layer-first batch image: K buffer then V buffer."""
+    n = len(ids)
+    stride = L.host_stride
+    nseg = 2 if L.is_split else 1
+    buf = n * stride
+    return LayerBlocks(
+        layout=L, block_ids=ids,
+        host=tuple(host.host_ptr + s * buf for s in range(nseg)),
+        host_device=tuple(host.device_ptr + s * buf for s in range(nseg)),
+        host_len=tuple(buf for _ in range(nseg)), host_stride=stride, layer_name="layer_0")
+
+
+def _roundtrip(case, xfer, stream, path):
+    L = case.product_layout()
+    n = len(case.ids)
+    stride = L.host_stride
+    nseg = 2 if L.is_split else 1
+    buf = n * stride
+    host = PinnedMemory(nseg * buf)
+    hv = host.as_numpy()
+
+    # ---- save: device -> host image, compare with the oracle ------------
+    case.dev.copy_from_host(case.cache0)
+    hv[:] = SENT
+    xfer.save([_dense_layer(case, L, host, case.ids)], stream, path)
+    stream.synchronize()
+    assert xfer.last_path == path
+    ocache = case.cache0.copy()
+    oL = case.oracle_layout(ocache)
+    ok = np.full(buf, SENT, dtype=np.uint8)
+    ov = np.full(buf, SENT, dtype=np.uint8) if nseg == 2 else None
+    O.transfer_layer(oL, case.ids, ok, ov, host_is_src=False)
+    assert np.array_equal(hv[:buf], ok), "saved K/contiguous image differs from the oracle"
+    if nseg == 2:
+        assert np.array_equal(hv[buf:], ov), "saved V image differs from the oracle"
+    assert np.array_equal(case.dev.copy_to_host(), case.cache0), "save modified device memory"
+
+    # ---- load: host image -> other device slots, compare whole cache ----
+    rng = np.random.default_rng(int(case.ids.sum()) + 1)
+    dest = rng.choice(case.num_blocks, n, replace=False).astype(np.uint32)
+    case.dev.fill(SENT)
+    xfer.load([_dense_layer(case, L, host, dest)], stream, path)
+    stream.synchronize()
+    ocache2 = np.full_like(case.cache0, SENT)
+    oL2 = case.oracle_layout(ocache2)
+    O.transfer_layer(oL2, dest, ok, ov, host_is_src=True)
+    assert np.array_equal(case.dev.copy_to_host(), ocache2), "loaded cache differs from the oracle"
+    host.close()
+
+
+LAYOUTS = {
+    # name: kwargs of Case
+    "llama_split_32k": dict(num_blocks=96, seg=32768, segments=2),
+    "fp8_split_16k": dict(num_blocks=128, seg=16384, segments=2),
+    "mla_contiguous_72k": dict(num_blocks=48, seg=73728, segments=1),
+    "adjacent_kv": dict(num_blocks=64, seg=8192, segments=2, kv_stride=8192),
+    "fused_strided": dict(num_blocks=40, seg=8192, segments=1, block_stride=16384),
+    # V segments interleaved between the K segments of a strided buffer
+    "sparse_split": dict(num_blocks=32, seg=4096, segments=2, kv_stride=139264, block_stride=16384),
+    "tail_4112": dict(num_blocks=70, seg=4112, segments=2),
+    "tiny_528": dict(num_blocks=300, seg=528, segments=1, n_ids=300),
+    "odd_size_1000": dict(num_blocks=50, seg=1000, segments=2),
+    "misaligned_base": dict(num_blocks=50, seg=4096, segments=2, base_off=4),
+}
+
+
+@pytest.mark.parametrize("path", [ZC, ST], ids=["zerocopy", "staged"])
+@pytest.mark.parametrize("name", sorted(LAYOUTS))
+def test_save_load_matches_oracle(name, path, xfer, stream):
+    rng = np.random.default_rng(abs(hash(name)) % (1 << 31))
+    case = Case(rng, **LAYOUTS[name])
+    try:
+        _roundtrip(case, xfer, stream, path)
+    finally:
+        case.close()
+
+
+@pytest.mark.parametrize("kw", [
+    dict(num_blocks=60, seg=8848, segments=2, pad_to=512),
+    # fragment size not a multiple of 16 while every fragment START is aligned:
+    # the 16-byte vector path with a bytewise tail
+    dict(num_blocks=40, seg=1000, segments=1, block_stride=1024, pad_to=512),
+], ids=["split_8848_to_9216", "contiguous_1000_to_1024"])
+def test_padded_host_stride_leaves_padding_untouched(kw, xfer, stream):
+    """SSD padding: the host stride is the segment size rounded up to 512;
+    copies use the unpadded size and the pad tail is never written
+    (layout.rs:157-160, offload.rs:472-474).  The staged path needs a dense
+    image and must refuse; zero-copy and AUTO must work."""
+    rng = np.random.default_rng(77)
+    case = Case(rng, **kw)
+    L = case.product_layout()
+    seg, stride = L.fragment_bytes, L.host_stride
+    assert stride > seg and stride % 512 == 0
+    nseg = 2 if L.is_split else 1
+    host = PinnedMemory(nseg * len(case.ids) * stride)
+    with pytest.raises(_lib.InvalidArgument, match="dense host image"):
+        xfer.save([_dense_layer(case, L, host, case.ids)], stream, ST)
+    _roundtrip(case, xfer, stream, ZC)
+    # AUTO picks zero-copy for a non-dense image
+    host.as_numpy()[:] = SENT
+    case.dev.copy_from_host(case.cache0)
+    xfer.save([_dense_layer(case, L, host, case.ids)], stream, TransferPath.AUTO)
+    stream.synchronize()
+    assert xfer.last_path == ZC
+    img = host.as_numpy().reshape(nseg, len(case.ids), stride)
+    assert (img[:, :, seg:] == SENT).all()
+    assert not (img[:, :, :seg] == SENT).all()
+    host.close()
+    case.close()
+
+
+def test_page_first_pages(xfer, stream):
+    """Page-first host layout: one page per block, each layer at its own byte
+    offset (instance.rs:107-162, offload.rs:182-282).  Three layers of
+    distinct sizes 512/1024/1536 -> offsets 0/512/1536 as in the reference's
+    page_first_multi_layer_roundtrip."""
+    rng = np.random.default_rng(5)
+    sizes = [512, 1024, 1536]
+    placement = O.build_page_layout([[0, 1, 2]], 3, sizes)
+    assert placement["layer_offsets"] == [0, 512, 1536]
+    page = placement["shard_page_sizes"][0]
+    num_blocks, n = 16, 11
+    ids = rng.choice(num_blocks, n, replace=False).astype(np.uint32)
+    # pages deliberately not in address order and not evenly spaced
+    slots = rng.permutation(2 * n)[:n]
+    pool = PinnedMemory(2 * n * page)
+    pool.as_numpy()[:] = SENT
+    page_host = np.array([pool.host_ptr + int(s) * page for s in slots], dtype=np.uint64)
+    page_dev = np.array([pool.device_ptr + int(s) * page for s in slots], dtype=np.uint64)
+    cases = [Case(rng, num_blocks=num_blocks, seg=sz, segments=1) for sz in sizes]
+    layers = []
+    for li, c in enumerate(cases):
+        c.dev.copy_from_host(c.cache0)
+        layers.append(LayerBlocks(layout=c.product_layout(), block_ids=ids, page_host=page_host,
+                                  page_host_device=page_dev,
+                                  page_offset=placement["layer_offsets"][li], page_len=page,
+                                  layer_name=f"layer_{li}"))
+    xfer.save(layers, stream, TransferPath.AUTO)
+    stream.synchronize()
+    assert xfer.last_path == ZC
+    # oracle on a host-resident pool image
+    opool = np.full(2 * n * page, SENT, dtype=np.uint8)
+    opages = np.array([opool.ctypes.data + int(s) * page for s in slots], dtype=np.uint64)
+    for li, c in enumerate(cases):
+        oc = c.cache0.copy()
+        O.transfer_layer_paged(c.oracle_layout(oc), ids, opages, placement["layer_offsets"][li],
+                               host_is_src=False)
+    assert np.array_equal(pool.as_numpy(), opool)
+    # load back into permuted slots
+    dest = rng.choice(num_blocks, n, replace=False).astype(np.uint32)
+    for li, c in enumerate(cases):
+        c.dev.fill(SENT)
+        layers[li].block_ids = dest
+    xfer.load(layers, stream, TransferPath.AUTO)
+    stream.synchronize()
+    for li, c in enumerate(cases):
+        oc = np.full_like(c.cache0, SENT)
+        O.transfer_layer_paged(c.oracle_layout(oc), dest, opages, placement["layer_offsets"][li],
+                               host_is_src=True)
+        assert np.array_equal(c.dev.copy_to_host(), oc), li
+        c.close()
+    pool.close()
+
+
+def test_multi_layer_batch_with_layer_events_and_empty_layer(xfer, stream):
+    """Several layers in one call, one of them empty; per-layer events all
+    fire; mixed paths in one call."""
+    rng = np.random.default_rng(13)
+    cases = [Case(rng, num_blocks=64, seg=32768, segments=2, n_ids=40),
+             Case(rng, num_blocks=64, seg=4096, segments=2, n_ids=1),
+             Case(rng, num_blocks=64, seg=16384, segments=1, n_ids=30)]
+    cases[1].ids = np.zeros(0, dtype=np.uint32)  # empty layer
+    hosts, layers, Ls = [], [], []
+    for c in cases:
+        L = c.product_layout()
+        Ls.append(L)
+        nseg = 2 if L.is_split else 1
+        h = PinnedMemory(max(1, nseg * len(c.ids) * L.host_stride))
+        h.as_numpy()[:] = SENT
+        hosts.append(h)
+        c.dev.copy_from_host(c.cache0)
+        layers.append(_dense_layer(c, L, h, c.ids))
+    events = [Event() for _ in cases]
+    big = BlockTransfer(staging_slot_bytes=1 << 20, staging_slots=2, auto_staged_min_bytes=1 << 20)
+    big.set_layer_events(events)
+    big.save(layers, stream, TransferPath.AUTO)
+    for e in events:
+        e.synchronize()
+    stream.synchronize()
+    assert all(e.query() for e in events)
+    for c, L, h in zip(cases, Ls, hosts):
+        if len(c.ids) == 0:
+            continue
+        n, stride = len(c.ids), L.host_stride
+        oc = c.cache0.copy()
+        ok = np.full(n * stride, SENT, dtype=np.uint8)
+        ov = np.full(n * stride, SENT, dtype=np.uint8) if L.is_split else None
+        O.transfer_layer(c.oracle_layout(oc), c.ids, ok, ov, host_is_src=False)
+        hv = h.as_numpy()
+        assert np.array_equal(hv[: n * stride], ok)
+        if ov is not None:
+            assert np.array_equal(hv[n * stride: 2 * n * stride], ov)
+    big.set_layer_events(None)
+    big.close()
+    for c, h in zip(cases, hosts):
+        c.close()
+        h.close()
+
+
+def test_errors_are_reported_before_anything_is_enqueued(xfer, stream):
+    rng = np.random.default_rng(2)
+    case = Case(rng, num_blocks=16, seg=4096, segments=2, n_ids=4)
+    L = case.product_layout()
+    host = PinnedMemory(2 * 4 * 4096)
+    host.as_numpy()[:] = SENT
+    bad = _dense_layer(case, L, host, np.array([1, 2, 16, 3], dtype=np.uint32))
+    bad.layer_name = "model.layers.7"
+    with pytest.raises(_lib.StorageError,
+                       match=r"layer model.layers.7: block 16 out of range \(16 blocks\)"):
+        xfer.save([bad], stream)
+    short = _dense_layer(case, L, host, case.ids)
+    short.host_len = (4 * 4096 - 1, 4 * 4096)
+    with pytest.raises(_lib.InvalidArgument, match="needs 16384 bytes, has 16383"):
+        xfer.save([short], stream)
+    stream.synchronize()
+    assert (host.as_numpy() == SENT).all()
+    # zero layers / zero blocks are fine
+    xfer.save([], stream)
+    xfer.load([_dense_layer(case, L, host, np.zeros(0, dtype=np.uint32))], stream)
+    stream.synchronize()
+    host.close()
+    case.close()
+
+
+def test_duplicate_source_ids_get_their_own_host_image(xfer, stream):
+    """Duplicate block ids in one save list are not rejected; each occurrence
+    gets its own host image (offload.rs:348-360)."""
+    rng = np.random.default_rng(21)
+    case = Case(rng, num_blocks=8, seg=4096, segments=2, n_ids=1)
+    case.ids = np.array([3, 3, 5, 3], dtype=np.uint32)
+    L = case.product_layout()
+    host = PinnedMemory(2 * 4 * 4096)
+    case.dev.copy_from_host(case.cache0)
+    for path in (ZC, ST):
+        host.as_numpy()[:] = SENT
+        xfer.save([_dense_layer(case, L, host, case.ids)], stream, path)
+        stream.synchronize()
+        ek, ev = O.np_save_split(case.cache0, 8, 4096, case.ids)
+        img = host.as_numpy().reshape(2, 4, 4096)
+        assert np.array_equal(img[0], ek) and np.array_equal(img[1], ev)
+    host.close()
+    case.close()
