@@ -273,9 +273,10 @@ typedef struct pf_layer_blocks {
 typedef struct pf_xfer_config {
   uint64_t staging_slot_bytes; /* 0 = default */
   uint32_t staging_slots;      /* 0 = default (2) */
-  uint32_t zerocopy_max_workgroups; /* 0 = default; caps CUs used next to compute */
+  uint32_t zerocopy_max_workgroups; /* 0 = default (64); workgroups of a zero-copy launch */
   uint64_t auto_staged_min_bytes;   /* 0 = default threshold for PF_PATH_AUTO */
-  uint32_t tile_unroll;             /* 16-byte loads in flight per lane: 1,2,4,8; 0 = default */
+  uint32_t tile_unroll;             /* zero-copy kernel: 16-byte loads in flight per lane:
+                                       1,2,4,8; 0 = default (4) */
   uint32_t reserved;
 } pf_xfer_config;
 
@@ -302,7 +303,9 @@ int pf_xfer_last_kernel_ms(pf_xfer_t x, float* out_ms, uint32_t* out_launches);
 int pf_xfer_set_kernel_timing(pf_xfer_t x, int enable);
 
 /* Plain device-to-device copy with the same tile shape as the gather/scatter
- * kernels (pointers and size 16-byte aligned).  A copy of known size: the
+ * kernels (pointers and size 16-byte aligned).  tile_unroll 0 = the
+ * one-tile-per-workgroup form of the staged path; 1/2/4/8 = the grid-stride
+ * form of the zero-copy path.  A copy of known size: the
  * yardstick for the HBM copy ceiling and for scaling hardware counters.  No
  * counterpart in the reference. */
 int pf_plain_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t tile_unroll,

@@ -39,13 +39,24 @@ bool unroll_supported(int unroll);
 
 // Launch the block-ID kernel over `n_units` units (grid.y) starting at
 // `units` (device).  `max_tiles` is the largest tile count of any of them;
-// `max_workgroups_x` (0 = no cap) bounds grid.x, the kernel grid-strides.
+// `max_workgroups_x` (0 = no cap) bounds the workgroups of the whole launch
+// (all units together); the kernel grid-strides.
 // to_far: true = gather near -> far (save), false = scatter far -> near (load).
 int launch_block_units(const BlockUnit* units, uint32_t n_units, uint64_t max_tiles, bool to_far,
                        int unroll, uint32_t max_workgroups_x, hipStream_t s);
 
+// Limits of one block_tiles launch (grid.y and grid.z are 16-bit).
+constexpr uint32_t kMaxTileBlocks = 65535;
+constexpr uint32_t kMaxTileUnits = 32767;
+
+// Launch the one-tile-per-workgroup form over `n_units` units: the HBM-bound
+// kernel of the staged path.  Every unit needs n_blocks <= kMaxTileBlocks.
+int launch_block_tiles(const BlockUnit* units, uint32_t n_units, uint32_t max_blocks,
+                       uint64_t max_frag_bytes, bool to_far, hipStream_t s);
+
 // Plain device copy kernel of the same tile shape, for calibrating counters
 // and measuring the HBM copy ceiling: copies `bytes` (multiple of 16).
+// unroll 0 selects the one-tile-per-workgroup form, 1/2/4/8 the grid-stride form.
 int launch_plain_copy(void* dst, const void* src, uint64_t bytes, int unroll, hipStream_t s);
 
 }  // namespace pf

@@ -27,10 +27,19 @@ namespace pf {
 
 namespace {
 
-constexpr uint64_t kDefaultSlotBytes = 64ull << 20;
-constexpr uint32_t kDefaultSlots = 3;
+// Measured on MI355X (Llama-3.1-8B shape, 327 MB per layer): slots smaller than
+// a layer cost cross-stream hand-offs between DMA copies (16 MiB slots reach
+// ~25 GB/s on saves, 64 MiB ~40-55 GB/s and unstable, 256 MiB 56.3 GB/s,
+// 512 MiB 56.7 GB/s of a 57.3 GB/s link), so a slot holds a whole layer.
+constexpr uint64_t kDefaultSlotBytes = 512ull << 20;
+constexpr uint32_t kDefaultSlots = 2;
 constexpr uint64_t kDefaultAutoStagedMin = 4ull << 20;
 constexpr int kDefaultUnroll = 4;
+// Zero-copy launches are capped to a few workgroups: the host link, not the
+// GPU, is the bound, and fewer in-flight requests use it better.  Measured on
+// MI355X (Llama shape, 16 layers per launch): 64 workgroups load at 57.4 GB/s
+// and save at 55.0-55.8 GB/s; 2048 and more give 56.0 and 54.5 GB/s.
+constexpr uint32_t kDefaultZeroCopyWorkgroups = 64;
 
 bool aligned16(uint64_t v) { return (v & 15ull) == 0; }
 
@@ -62,7 +71,7 @@ class Xfer {
     if (cfg) {
       if (cfg->staging_slot_bytes) slot_bytes_ = cfg->staging_slot_bytes;
       if (cfg->staging_slots) n_slots_ = cfg->staging_slots;
-      zc_max_wg_ = cfg->zerocopy_max_workgroups;
+      if (cfg->zerocopy_max_workgroups) zc_max_wg_ = cfg->zerocopy_max_workgroups;
       if (cfg->auto_staged_min_bytes) auto_min_ = cfg->auto_staged_min_bytes;
       if (cfg->tile_unroll) unroll_ = static_cast<int>(cfg->tile_unroll);
     }
@@ -133,13 +142,19 @@ class Xfer {
 
   int plan_layer(const pf_layer_blocks& in, size_t index, int path, LayerPlan* out, bool* skip);
   int ensure_slot(Slot& sl, uint64_t bytes);
-  int launch(const BlockUnit* dev_units, uint32_t n_units, uint64_t max_tiles, bool to_far,
-             uint32_t max_wg, hipStream_t s);
+  // Zero-copy form: grid-stride kernel over `n_units` units, capped grid.
+  int launch_strided(const BlockUnit* dev_units, uint32_t n_units, uint64_t max_tiles, bool to_far,
+                     hipStream_t s);
+  // Staged form: one tile per workgroup over one unit.
+  int launch_tiles(const BlockUnit* dev_unit, const BlockUnit& host_unit, bool to_far,
+                   hipStream_t s);
+  int timing_begin(hipStream_t s);
+  int timing_end(hipStream_t s);
 
   int device_ = 0;
   uint64_t slot_bytes_ = kDefaultSlotBytes;
   uint32_t n_slots_ = kDefaultSlots;
-  uint32_t zc_max_wg_ = 0;
+  uint32_t zc_max_wg_ = kDefaultZeroCopyWorkgroups;
   uint64_t auto_min_ = kDefaultAutoStagedMin;
   int unroll_ = kDefaultUnroll;
 
@@ -173,24 +188,41 @@ int Xfer::ensure_slot(Slot& sl, uint64_t bytes) {
   return PF_OK;
 }
 
-int Xfer::launch(const BlockUnit* dev_units, uint32_t n_units, uint64_t max_tiles, bool to_far,
-                 uint32_t max_wg, hipStream_t s) {
-  if (timing_) {
-    if (timing_used_ == timing_pool_.size()) {
-      hipEvent_t a = nullptr, b = nullptr;
-      PF_HIP(hipEventCreate(&a));
-      PF_HIP(hipEventCreate(&b));
-      timing_pool_.emplace_back(a, b);
-    }
-    PF_HIP(hipEventRecord(timing_pool_[timing_used_].first, s));
+int Xfer::timing_begin(hipStream_t s) {
+  if (!timing_) return PF_OK;
+  if (timing_used_ == timing_pool_.size()) {
+    hipEvent_t a = nullptr, b = nullptr;
+    PF_HIP(hipEventCreate(&a));
+    PF_HIP(hipEventCreate(&b));
+    timing_pool_.emplace_back(a, b);
   }
-  int st = launch_block_units(dev_units, n_units, max_tiles, to_far, unroll_, max_wg, s);
-  if (st != PF_OK) return st;
-  if (timing_) {
-    PF_HIP(hipEventRecord(timing_pool_[timing_used_].second, s));
-    ++timing_used_;
-  }
+  PF_HIP(hipEventRecord(timing_pool_[timing_used_].first, s));
   return PF_OK;
+}
+
+int Xfer::timing_end(hipStream_t s) {
+  if (!timing_) return PF_OK;
+  PF_HIP(hipEventRecord(timing_pool_[timing_used_].second, s));
+  ++timing_used_;
+  return PF_OK;
+}
+
+int Xfer::launch_strided(const BlockUnit* dev_units, uint32_t n_units, uint64_t max_tiles,
+                         bool to_far, hipStream_t s) {
+  int st = timing_begin(s);
+  if (st != PF_OK) return st;
+  st = launch_block_units(dev_units, n_units, max_tiles, to_far, unroll_, zc_max_wg_, s);
+  if (st != PF_OK) return st;
+  return timing_end(s);
+}
+
+int Xfer::launch_tiles(const BlockUnit* dev_unit, const BlockUnit& host_unit, bool to_far,
+                       hipStream_t s) {
+  int st = timing_begin(s);
+  if (st != PF_OK) return st;
+  st = launch_block_tiles(dev_unit, 1, host_unit.n_blocks, host_unit.frag_bytes, to_far, s);
+  if (st != PF_OK) return st;
+  return timing_end(s);
 }
 
 int Xfer::last_kernel_ms(float* out_ms, uint32_t* out_launches) {
@@ -372,6 +404,7 @@ int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool s
     }
     const uint64_t block_bytes = p.frag_bytes * p.n_seg;
     uint64_t per_unit = std::max<uint64_t>(slot_bytes_ / block_bytes, 1);
+    per_unit = std::min<uint64_t>(per_unit, kMaxTileBlocks);
     for (uint64_t first = 0; first < p.n_blocks; first += per_unit) {
       uint64_t count = std::min(per_unit, p.n_blocks - first);
       unit_refs.push_back({pi, first, count});
@@ -475,11 +508,14 @@ int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool s
 
   // ---- 4. enqueue ---------------------------------------------------------
   PF_HIP(hipMemcpyAsync(slab->dev, slab->host, slab_bytes, hipMemcpyHostToDevice, s));
+  // With kernel timing on, the DMA copies run on the caller's stream too, so
+  // that every timed kernel executes alone (a measurement mode: no overlap).
+  hipStream_t side = timing_ ? s : side_;
   bool side_used = false;
   auto fork_side = [&]() -> int {
-    if (side_used) return PF_OK;
+    if (side_used || side == s) return PF_OK;
     PF_HIP(hipEventRecord(fork_, s));
-    PF_HIP(hipStreamWaitEvent(side_, fork_, 0));
+    PF_HIP(hipStreamWaitEvent(side, fork_, 0));
     side_used = true;
     return PF_OK;
   };
@@ -511,7 +547,7 @@ int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool s
           ++uj;
         }
       }
-      st = launch(units_dev + ui, static_cast<uint32_t>(uj - ui), max_tiles, save, zc_max_wg_, s);
+      st = launch_strided(units_dev + ui, static_cast<uint32_t>(uj - ui), max_tiles, save, s);
       if (st != PF_OK) return st;
       st = fire_events_through(plans[unit_refs[uj - 1].plan].src_index, s);
       if (st != PF_OK) return st;
@@ -529,31 +565,31 @@ int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool s
         ui + 1 == unit_refs.size() || unit_refs[ui + 1].plan != unit_refs[ui].plan;
     if (save) {
       if (sl.used) PF_HIP(hipStreamWaitEvent(s, sl.freed, 0));
-      st = launch(units_dev + ui, 1, tiles_of(u), true, 0, s);
+      st = launch_tiles(units_dev + ui, u, true, s);
       if (st != PF_OK) return st;
       PF_HIP(hipEventRecord(sl.ready, s));
-      PF_HIP(hipStreamWaitEvent(side_, sl.ready, 0));
+      PF_HIP(hipStreamWaitEvent(side, sl.ready, 0));
       for (uint32_t sgm = 0; sgm < p.n_seg; ++sgm) {
         PF_HIP(hipMemcpyAsync(p.host[sgm] + r.first * p.host_stride,
                               reinterpret_cast<const void*>(u.far_base[sgm]),
-                              r.count * p.frag_bytes, hipMemcpyDeviceToHost, side_));
+                              r.count * p.frag_bytes, hipMemcpyDeviceToHost, side));
       }
-      PF_HIP(hipEventRecord(sl.freed, side_));
+      PF_HIP(hipEventRecord(sl.freed, side));
       sl.used = true;
       if (last_of_layer) {
-        st = fire_events_through(p.src_index, side_);
+        st = fire_events_through(p.src_index, side);
         if (st != PF_OK) return st;
       }
     } else {
-      if (sl.used) PF_HIP(hipStreamWaitEvent(side_, sl.freed, 0));
+      if (sl.used) PF_HIP(hipStreamWaitEvent(side, sl.freed, 0));
       for (uint32_t sgm = 0; sgm < p.n_seg; ++sgm) {
         PF_HIP(hipMemcpyAsync(reinterpret_cast<void*>(u.far_base[sgm]),
                               p.host[sgm] + r.first * p.host_stride, r.count * p.frag_bytes,
-                              hipMemcpyHostToDevice, side_));
+                              hipMemcpyHostToDevice, side));
       }
-      PF_HIP(hipEventRecord(sl.ready, side_));
+      PF_HIP(hipEventRecord(sl.ready, side));
       PF_HIP(hipStreamWaitEvent(s, sl.ready, 0));
-      st = launch(units_dev + ui, 1, tiles_of(u), false, 0, s);
+      st = launch_tiles(units_dev + ui, u, false, s);
       if (st != PF_OK) return st;
       PF_HIP(hipEventRecord(sl.freed, s));
       sl.used = true;
@@ -567,7 +603,7 @@ int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool s
   if (side_used && save) {
     // Join: everything the side stream drained is ordered before whatever the
     // caller enqueues (or records) next on its stream.
-    PF_HIP(hipEventRecord(join_, side_));
+    PF_HIP(hipEventRecord(join_, side));
     PF_HIP(hipStreamWaitEvent(s, join_, 0));
   }
   // Trailing empty layers.
@@ -625,7 +661,8 @@ int pf_xfer_last_kernel_ms(pf_xfer_t x, float* out_ms, uint32_t* out_launches) {
 
 int pf_plain_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t tile_unroll,
                   pf_stream_t s) {
-  int unroll = tile_unroll ? static_cast<int>(tile_unroll) : 4;
+  // 0 selects the one-tile-per-workgroup form the staged path uses.
+  int unroll = static_cast<int>(tile_unroll);
   return pf::launch_plain_copy(reinterpret_cast<void*>(dst), reinterpret_cast<const void*>(src),
                                bytes, unroll, pf::native(s));
 }

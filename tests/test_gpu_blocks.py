@@ -143,6 +143,8 @@ LAYOUTS = {
     "tiny_528": dict(num_blocks=300, seg=528, segments=1, n_ids=300),
     "odd_size_1000": dict(num_blocks=50, seg=1000, segments=2),
     "misaligned_base": dict(num_blocks=50, seg=4096, segments=2, base_off=4),
+    # more list positions than one tile launch can index (65535): the staged path splits units
+    "many_tiny_64": dict(num_blocks=70000, seg=64, segments=1, n_ids=70000),
 }
 
 
