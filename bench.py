@@ -30,6 +30,11 @@ if ROOT not in sys.path:
 
 PCIE_GEN5_X16_GBPS = 63.0   # 32 GT/s x 16 lanes x 128/130 / 8
 HBM_PEAK_GBPS = 8000.0      # MI355X published HBM3E bandwidth
+# HBM bytes one staged gather/scatter launch moves at the default workload
+# (5000 blocks x 2 x 32 KiB), from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
+# of this script: 160191.7 and 320043.6 KiB per dispatch, scaled by what a plain
+# copy of exactly 1 GiB reads on the same counters (x2.000 and x1.000).
+MEASURED_TRAFFIC_DEFAULT_STAGED = int((160191.7 * 2.000 + 320043.6 * 1.000) * 1024)
 
 LLAMA = dict(layers=32, num_blocks=8192, block_tokens=16, kv_heads=8, head_dim=128, elem=2,
              n_save=5000)
@@ -212,8 +217,10 @@ def main():
         # once in HBM -> 2 x payload algorithmic bytes per launch
         alg_bytes = 2 * bytes_per_launch
         achieved = alg_bytes / (avg_launch_ms / 1e3) / 1e9
+        default_shape = (n_layers == LLAMA["layers"] and not args.slot_mb)
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                    "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                    "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                    "traffic": MEASURED_TRAFFIC_DEFAULT_STAGED if default_shape else None,
                     "kernel": "block_tiles_kernel (staged gather/scatter)",
                     "launches": launches, "avg_launch_us": round(avg_launch_ms * 1e3, 2),
                     "alg_bytes_per_launch": int(alg_bytes),
