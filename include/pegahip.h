@@ -311,6 +311,246 @@ int pf_xfer_set_kernel_timing(pf_xfer_t x, int enable);
 int pf_plain_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t tile_unroll,
                   pf_stream_t s);
 
+/* ------------------------------------------------------------------------ */
+/* Offset allocator (pure host arithmetic)                                   */
+/* Replaces ScaledOffsetAllocator (pegaflow-core/src/allocator.rs:63-142)    */
+/* over the `offset-allocator` crate.                                        */
+/* ------------------------------------------------------------------------ */
+
+typedef struct pf_allocator_s* pf_allocator_t;
+
+typedef struct pf_alloc_region {
+  uint64_t offset_bytes;
+  uint64_t size_bytes; /* rounded up to the unit; 0 = no space */
+  uint64_t token;      /* pass back to pf_allocator_free */
+} pf_alloc_region;
+
+/* new_with_unit_size_and_max_allocs, allocator.rs:73-92. */
+int pf_allocator_create(uint64_t total_bytes, uint64_t unit_size, uint32_t max_allocs,
+                        pf_allocator_t* out);
+int pf_allocator_destroy(pf_allocator_t a);
+/* allocate, allocator.rs:95-123: PF_OK with size_bytes == 0 when nothing fits
+ * (or size is 0); PF_ERR_INVALID_ARGUMENT when the request overflows u32 units. */
+int pf_allocator_allocate(pf_allocator_t a, uint64_t size_bytes, pf_alloc_region* out);
+int pf_allocator_free(pf_allocator_t a, const pf_alloc_region* region);
+/* total_bytes + storage_report, allocator.rs:131-142. */
+int pf_allocator_report(pf_allocator_t a, uint64_t* out_total_bytes, uint64_t* out_free_bytes,
+                        uint64_t* out_largest_free_bytes, uint64_t* out_total_units);
+
+/* ------------------------------------------------------------------------ */
+/* Pinned pool                                                               */
+/* Replaces PinnedAllocator / ShardedPinnedPool / NumaAwarePinnedPools /     */
+/* PinnedMemoryPool / PinnedAllocation                                       */
+/* (pegaflow-core/src/pinned_pool.rs:56-715).                                */
+/* ------------------------------------------------------------------------ */
+
+typedef struct pf_pool_s* pf_pool_t;
+
+typedef struct pf_pool_config {
+  uint64_t capacity;        /* total bytes, split evenly over NUMA nodes and shards */
+  uint32_t num_shards;      /* per node; 0 or 1 = one pool */
+  uint32_t use_hugepages;   /* MAP_HUGETLB backing */
+  uint32_t ssd_enabled;     /* regular (CPU-readable) backing instead of hipHostMalloc */
+  uint32_t n_numa_nodes;    /* 0 = one global pool */
+  const int32_t* numa_nodes;
+  uint64_t unit_size_hint;  /* 0 = 512 */
+} pf_pool_config;
+
+typedef struct pf_allocation {
+  uint64_t handle;  /* owning handle; 0 when the pool is exhausted */
+  void* host;
+  uint64_t device;
+  uint64_t size;    /* bytes actually reserved (unit-rounded) */
+} pf_allocation;
+
+/* compute_unit_size, pinned_pool.rs:135-141. */
+uint64_t pf_pool_compute_unit_size(uint64_t pool_size, uint64_t unit_size_hint);
+/* PinnedAllocator::new_global / new_numa, pinned_pool.rs:616-660. */
+int pf_pool_create(const pf_pool_config* cfg, pf_pool_t* out);
+int pf_pool_destroy(pf_pool_t p);
+/* allocate, pinned_pool.rs:666-675.  numa_node is ignored by a global pool.
+ * PF_OK with handle == 0 when nothing fits (the reference's `None`). */
+int pf_pool_allocate(pf_pool_t p, uint64_t size, int numa_node, pf_allocation* out);
+/* Drop of the PinnedAllocation guard, pinned_pool.rs:112-117. */
+int pf_pool_free(pf_allocation* a);
+int pf_pool_usage(pf_pool_t p, uint64_t* out_used, uint64_t* out_total);
+int pf_pool_largest_free(pf_pool_t p, int numa_node, uint64_t* out_bytes);
+int pf_pool_is_numa(pf_pool_t p);
+
+/* ------------------------------------------------------------------------ */
+/* NUMA helpers (pegaflow-common/src/numa.rs:49-257)                         */
+/* ------------------------------------------------------------------------ */
+
+/* format_cpu_list: [0,1,2,4] -> "0-2,4". */
+int pf_numa_format_cpu_list(const uint64_t* cpus, uint64_t n, char* buf, size_t cap);
+/* parse_cpulist: "0-3,8" -> sorted unique ids; *out_n = count needed. */
+int pf_numa_parse_cpulist(const char* cpulist, uint64_t* out, uint64_t cap, uint64_t* out_n);
+/* pin_thread_to_numa_node for the calling thread. */
+int pf_numa_pin_thread(int numa_node);
+/* Number of NUMA nodes with CPUs (1 when sysfs has none). */
+int pf_numa_node_count(void);
+/* NUMA node of a PCI device under `sysfs_root` (NULL = /sys/bus/pci/devices). */
+int pf_numa_node_of_pci(const char* bdf, const char* sysfs_root);
+
+/* ------------------------------------------------------------------------ */
+/* Layer topology and page-first placement                                   */
+/* Replaces build_page_layout / LayerTopology                                */
+/* (pegaflow-core/src/instance.rs:46-269,488-672).                           */
+/* ------------------------------------------------------------------------ */
+
+/* build_page_layout, instance.rs:107-162.  Worker w registered the layer ids
+ * set_ids[set_off[w] .. set_off[w+1]).  Outputs are indexed by layer id
+ * (n_layers entries) and by shard (*out_n_shards <= n_sets entries). */
+int pf_build_page_layout(const uint64_t* set_ids, const uint64_t* set_off, uint64_t n_sets,
+                         uint64_t n_layers, const uint64_t* padded_bytes,
+                         uint64_t* out_layer_shard, uint64_t* out_layer_offsets,
+                         uint64_t* out_layer_bytes, uint64_t* out_shard_page_sizes,
+                         uint64_t* out_n_shards);
+
+typedef struct pf_topology_s* pf_topology_t;
+
+typedef struct pf_worker_layers {
+  int32_t device_id;
+  uint32_t tp_rank;
+  uint32_t pp_rank;
+  uint32_t n_layers;
+  const char* const* layer_names;
+  const pf_kv_layout* layouts;
+  const uint32_t* group_ids; /* NULL = all group 0 */
+} pf_worker_layers;
+
+/* seal_topology, instance.rs:488-672. */
+int pf_topology_seal(const pf_worker_layers* workers, uint32_t n_workers, uint32_t tp_size,
+                     int page_first, pf_topology_t* out);
+int pf_topology_destroy(pf_topology_t t);
+uint64_t pf_topology_num_layers(pf_topology_t t);
+uint64_t pf_topology_total_slots(pf_topology_t t);
+int pf_topology_is_page_first(pf_topology_t t);
+/* Layer ids are ranks of the byte-wise sorted layer names. */
+int pf_topology_layer_id(pf_topology_t t, const char* layer_name, uint64_t* out_id);
+int pf_topology_slot_index(pf_topology_t t, uint64_t layer_id, uint64_t tp_rank, uint64_t* out);
+int pf_topology_page_placement(pf_topology_t t, uint64_t layer_id, uint64_t* out_offset,
+                               uint64_t* out_bytes);
+int pf_topology_shard_page_size(pf_topology_t t, uint64_t shard, uint64_t* out);
+int pf_topology_shard_layer_count(pf_topology_t t, uint64_t shard, uint64_t* out);
+
+/* ------------------------------------------------------------------------ */
+/* Load completion flag in shared memory                                     */
+/* Replaces LoadState (pegaflow-core/src/sync_state.rs:23-300): POSIX shm    */
+/* object "pega_load_<hex>", magic 'PFLD', version 1, i64 state              */
+/* (0 pending, 1 success, -1 error).                                         */
+/* ------------------------------------------------------------------------ */
+
+typedef struct pf_load_state_s* pf_load_state_t;
+
+int pf_load_state_create(pf_load_state_t* out);
+int pf_load_state_attach(const char* shm_name, pf_load_state_t* out);
+int pf_load_state_destroy(pf_load_state_t s);
+const char* pf_load_state_name(pf_load_state_t s);
+int64_t pf_load_state_get(pf_load_state_t s);
+int pf_load_state_set(pf_load_state_t s, int64_t state); /* 1 or -1 */
+
+/* ------------------------------------------------------------------------ */
+/* Per-GPU worker pair                                                       */
+/* Replaces GpuWorkerPool / LoadTask / SaveTask / LoadCompletion             */
+/* (pegaflow-core/src/gpu_worker.rs:15-345,428-523).                         */
+/* ------------------------------------------------------------------------ */
+
+typedef struct pf_worker_pool_s* pf_worker_pool_t;
+typedef struct pf_task_s* pf_task_t;
+
+typedef struct pf_task_result {
+  int32_t status;      /* PF_OK or an error status */
+  int32_t done;        /* 0 while pending (only from pf_task_wait with a timeout) */
+  uint64_t bytes;      /* payload bytes moved */
+  double elapsed_ms;   /* descriptor/plan construction + enqueue + synchronise */
+} pf_task_result;
+
+/* GpuWorkerPool::spawn, gpu_worker.rs:131-201: a load thread and a save thread
+ * pinned to `numa_node` (< 0 = no pinning), each with its own stream.
+ * use_descriptor_backends != 0: per-fragment descriptors through the backend of
+ * `transfer_mode`, exactly as the reference; 0: the block-ID engine, with
+ * PF_MODE_DIRECT = PF_PATH_AUTO and PF_MODE_KERNEL = PF_PATH_ZEROCOPY.
+ * Initialisation errors are returned here, synchronously. */
+int pf_worker_pool_spawn(int device_id, int numa_node, int transfer_mode,
+                         int use_descriptor_backends, pf_worker_pool_t* out);
+int pf_worker_pool_destroy(pf_worker_pool_t p);
+/* submit_load, gpu_worker.rs:204-212.  The layers are copied; host memory they
+ * point to must stay valid until the task settles.  load_state_shm (may be NULL)
+ * names a LoadState to signal. */
+int pf_worker_submit_load(pf_worker_pool_t p, const pf_layer_transfer* layers, uint64_t n_layers,
+                          const char* load_state_shm, pf_task_t* out_task);
+/* batch_save, gpu_worker.rs:216-243. */
+int pf_worker_submit_save(pf_worker_pool_t p, const pf_layer_transfer* layers, uint64_t n_layers,
+                          pf_task_t* out_task);
+/* Wait up to timeout_ms (< 0 = forever) for the task to settle.  Returns the
+ * task's status once done (message via pf_last_error), PF_OK while pending. */
+int pf_task_wait(pf_task_t t, int timeout_ms, pf_task_result* out);
+int pf_task_destroy(pf_task_t t);
+
+/* ------------------------------------------------------------------------ */
+/* Save / load by block ID                                                   */
+/* Replaces the parts of PegaEngine on the path: register_context_layer_     */
+/* batch[_strided] (pegaflow-core/src/lib.rs:228-440), batch_save_kv_blocks_ */
+/* from_ipc (offload.rs:293-659), prefix query + lease (lib.rs:506-546,      */
+/* 614-634), batch_load_kv_blocks_multi_layer[_inproc] (lib.rs:654-898).     */
+/* ------------------------------------------------------------------------ */
+
+typedef struct pf_engine_s* pf_engine_t;
+
+typedef struct pf_engine_config {
+  uint64_t pool_size;
+  uint32_t use_hugepages;
+  uint32_t numa_aware;
+  uint32_t pool_shards;
+  uint32_t blockwise_alloc;          /* one pinned allocation per block */
+  uint32_t ssd_enabled;              /* 512-byte host padding + CPU-readable backing */
+  uint32_t use_descriptor_backends;  /* see pf_worker_pool_spawn */
+  uint64_t unit_size_hint;
+} pf_engine_config;
+
+typedef struct pf_layer_save {       /* LayerSave, block.rs:20-25 */
+  const char* layer_name;
+  const uint64_t* block_ids;
+  const uint8_t* const* block_hashes;
+  const uint32_t* block_hash_lens;
+  uint64_t n_blocks;
+} pf_layer_save;
+
+int pf_engine_create(const pf_engine_config* cfg, pf_engine_t* out);
+int pf_engine_destroy(pf_engine_t e);
+/* block_stride_bytes and layer_group_ids may be NULL. */
+int pf_engine_register_context_layer_batch(
+    pf_engine_t e, const char* instance_id, const char* namespace_, int device_id,
+    uint64_t tp_rank, uint64_t pp_rank, uint64_t tp_size, uint64_t world_size, uint64_t n_layers,
+    const char* const* layer_names, const uint64_t* data_ptrs, const uint64_t* size_bytes,
+    const uint64_t* num_blocks, const uint64_t* bytes_per_block, const uint64_t* kv_stride_bytes,
+    const uint64_t* segments, const uint64_t* block_stride_bytes, const uint32_t* layer_group_ids,
+    int transfer_mode, int page_first);
+int pf_engine_unregister_instance(pf_engine_t e, const char* instance_id);
+/* Returns when the blocks are in host memory and queryable. */
+int pf_engine_batch_save(pf_engine_t e, const char* instance_id, uint64_t tp_rank,
+                         uint64_t pp_rank, int device_id, const pf_layer_save* saves,
+                         uint64_t n_saves);
+/* Longest cached prefix of the hashes and a lease over those blocks (0 = none). */
+int pf_engine_query_prefix(pf_engine_t e, const char* instance_id,
+                           const uint8_t* const* hashes, const uint32_t* hash_lens, uint64_t n,
+                           uint64_t* out_hits, uint64_t* out_lease);
+int pf_engine_release_lease(pf_engine_t e, uint64_t lease);
+/* One lease loaded into n_groups load groups.  group_layer_names[g] is an array
+ * of group_sizes[g] layer names; dest_block_ids[g] holds one destination per
+ * leased block (-1 = skip).  load_state_shm may be NULL.  *out_task settles when
+ * the load does. */
+int pf_engine_batch_load(pf_engine_t e, const char* instance_id, uint64_t tp_rank, int device_id,
+                         uint64_t n_groups, const char* const* const* group_layer_names,
+                         const uint64_t* group_sizes, uint64_t lease,
+                         const int64_t* const* dest_block_ids, uint64_t n_blocks,
+                         const char* load_state_shm, pf_task_t* out_task);
+int pf_engine_pool_usage(pf_engine_t e, uint64_t* out_used, uint64_t* out_total);
+uint64_t pf_engine_cached_blocks(pf_engine_t e);
+/* Drop every cached block that is not leased; returns how many. */
+uint64_t pf_engine_evict_all(pf_engine_t e);
+
 #ifdef __cplusplus
 } /* extern "C" */
 #endif

@@ -89,6 +89,43 @@ class PfXferConfig(C.Structure):
                 ("tile_unroll", u32), ("reserved", u32)]
 
 
+class PfAllocRegion(C.Structure):
+    _fields_ = [("offset_bytes", u64), ("size_bytes", u64), ("token", u64)]
+
+
+class PfPoolConfig(C.Structure):
+    _fields_ = [("capacity", u64), ("num_shards", u32), ("use_hugepages", u32),
+                ("ssd_enabled", u32), ("n_numa_nodes", u32), ("numa_nodes", C.POINTER(C.c_int32)),
+                ("unit_size_hint", u64)]
+
+
+class PfAllocation(C.Structure):
+    _fields_ = [("handle", u64), ("host", vp), ("device", u64), ("size", u64)]
+
+
+class PfWorkerLayers(C.Structure):
+    _fields_ = [("device_id", C.c_int32), ("tp_rank", u32), ("pp_rank", u32), ("n_layers", u32),
+                ("layer_names", C.POINTER(C.c_char_p)), ("layouts", C.POINTER(PfKvLayout)),
+                ("group_ids", C.POINTER(u32))]
+
+
+class PfTaskResult(C.Structure):
+    _fields_ = [("status", C.c_int32), ("done", C.c_int32), ("bytes", u64),
+                ("elapsed_ms", C.c_double)]
+
+
+class PfEngineConfig(C.Structure):
+    _fields_ = [("pool_size", u64), ("use_hugepages", u32), ("numa_aware", u32),
+                ("pool_shards", u32), ("blockwise_alloc", u32), ("ssd_enabled", u32),
+                ("use_descriptor_backends", u32), ("unit_size_hint", u64)]
+
+
+class PfLayerSave(C.Structure):
+    _fields_ = [("layer_name", C.c_char_p), ("block_ids", C.POINTER(u64)),
+                ("block_hashes", C.POINTER(C.POINTER(C.c_uint8))),
+                ("block_hash_lens", C.POINTER(u32)), ("n_blocks", u64)]
+
+
 # name -> (restype, argtypes).  Every symbol include/pegahip.h declares.
 PROTOTYPES = {
     "pf_last_error": (C.c_char_p, []),
@@ -148,6 +185,70 @@ PROTOTYPES = {
     "pf_xfer_last_kernel_ms": (C.c_int, [vp, C.POINTER(C.c_float), C.POINTER(u32)]),
     "pf_xfer_set_kernel_timing": (C.c_int, [vp, C.c_int]),
     "pf_plain_copy": (C.c_int, [u64, u64, u64, u32, vp]),
+    "pf_allocator_create": (C.c_int, [u64, u64, u32, C.POINTER(vp)]),
+    "pf_allocator_destroy": (C.c_int, [vp]),
+    "pf_allocator_allocate": (C.c_int, [vp, u64, C.POINTER(PfAllocRegion)]),
+    "pf_allocator_free": (C.c_int, [vp, C.POINTER(PfAllocRegion)]),
+    "pf_allocator_report": (C.c_int, [vp, C.POINTER(u64), C.POINTER(u64), C.POINTER(u64),
+                                      C.POINTER(u64)]),
+    "pf_pool_compute_unit_size": (u64, [u64, u64]),
+    "pf_pool_create": (C.c_int, [C.POINTER(PfPoolConfig), C.POINTER(vp)]),
+    "pf_pool_destroy": (C.c_int, [vp]),
+    "pf_pool_allocate": (C.c_int, [vp, u64, C.c_int, C.POINTER(PfAllocation)]),
+    "pf_pool_free": (C.c_int, [C.POINTER(PfAllocation)]),
+    "pf_pool_usage": (C.c_int, [vp, C.POINTER(u64), C.POINTER(u64)]),
+    "pf_pool_largest_free": (C.c_int, [vp, C.c_int, C.POINTER(u64)]),
+    "pf_pool_is_numa": (C.c_int, [vp]),
+    "pf_numa_format_cpu_list": (C.c_int, [C.POINTER(u64), u64, C.c_char_p, C.c_size_t]),
+    "pf_numa_parse_cpulist": (C.c_int, [C.c_char_p, C.POINTER(u64), u64, C.POINTER(u64)]),
+    "pf_numa_pin_thread": (C.c_int, [C.c_int]),
+    "pf_numa_node_count": (C.c_int, []),
+    "pf_numa_node_of_pci": (C.c_int, [C.c_char_p, C.c_char_p]),
+    "pf_build_page_layout": (C.c_int, [C.POINTER(u64), C.POINTER(u64), u64, u64, C.POINTER(u64),
+                                       C.POINTER(u64), C.POINTER(u64), C.POINTER(u64),
+                                       C.POINTER(u64), C.POINTER(u64)]),
+    "pf_topology_seal": (C.c_int, [C.POINTER(PfWorkerLayers), u32, u32, C.c_int, C.POINTER(vp)]),
+    "pf_topology_destroy": (C.c_int, [vp]),
+    "pf_topology_num_layers": (u64, [vp]),
+    "pf_topology_total_slots": (u64, [vp]),
+    "pf_topology_is_page_first": (C.c_int, [vp]),
+    "pf_topology_layer_id": (C.c_int, [vp, C.c_char_p, C.POINTER(u64)]),
+    "pf_topology_slot_index": (C.c_int, [vp, u64, u64, C.POINTER(u64)]),
+    "pf_topology_page_placement": (C.c_int, [vp, u64, C.POINTER(u64), C.POINTER(u64)]),
+    "pf_topology_shard_page_size": (C.c_int, [vp, u64, C.POINTER(u64)]),
+    "pf_topology_shard_layer_count": (C.c_int, [vp, u64, C.POINTER(u64)]),
+    "pf_load_state_create": (C.c_int, [C.POINTER(vp)]),
+    "pf_load_state_attach": (C.c_int, [C.c_char_p, C.POINTER(vp)]),
+    "pf_load_state_destroy": (C.c_int, [vp]),
+    "pf_load_state_name": (C.c_char_p, [vp]),
+    "pf_load_state_get": (C.c_int64, [vp]),
+    "pf_load_state_set": (C.c_int, [vp, C.c_int64]),
+    "pf_worker_pool_spawn": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(vp)]),
+    "pf_worker_pool_destroy": (C.c_int, [vp]),
+    "pf_worker_submit_load": (C.c_int, [vp, C.POINTER(PfLayerTransfer), u64, C.c_char_p,
+                                        C.POINTER(vp)]),
+    "pf_worker_submit_save": (C.c_int, [vp, C.POINTER(PfLayerTransfer), u64, C.POINTER(vp)]),
+    "pf_task_wait": (C.c_int, [vp, C.c_int, C.POINTER(PfTaskResult)]),
+    "pf_task_destroy": (C.c_int, [vp]),
+    "pf_engine_create": (C.c_int, [C.POINTER(PfEngineConfig), C.POINTER(vp)]),
+    "pf_engine_destroy": (C.c_int, [vp]),
+    "pf_engine_register_context_layer_batch": (C.c_int, [
+        vp, C.c_char_p, C.c_char_p, C.c_int, u64, u64, u64, u64, u64, C.POINTER(C.c_char_p),
+        C.POINTER(u64), C.POINTER(u64), C.POINTER(u64), C.POINTER(u64), C.POINTER(u64),
+        C.POINTER(u64), C.POINTER(u64), C.POINTER(u32), C.c_int, C.c_int]),
+    "pf_engine_unregister_instance": (C.c_int, [vp, C.c_char_p]),
+    "pf_engine_batch_save": (C.c_int, [vp, C.c_char_p, u64, u64, C.c_int, C.POINTER(PfLayerSave),
+                                       u64]),
+    "pf_engine_query_prefix": (C.c_int, [vp, C.c_char_p, C.POINTER(C.POINTER(C.c_uint8)),
+                                         C.POINTER(u32), u64, C.POINTER(u64), C.POINTER(u64)]),
+    "pf_engine_release_lease": (C.c_int, [vp, u64]),
+    "pf_engine_batch_load": (C.c_int, [vp, C.c_char_p, u64, C.c_int, u64,
+                                       C.POINTER(C.POINTER(C.c_char_p)), C.POINTER(u64), u64,
+                                       C.POINTER(C.POINTER(C.c_int64)), u64, C.c_char_p,
+                                       C.POINTER(vp)]),
+    "pf_engine_pool_usage": (C.c_int, [vp, C.POINTER(u64), C.POINTER(u64)]),
+    "pf_engine_cached_blocks": (u64, [vp]),
+    "pf_engine_evict_all": (u64, [vp]),
 }
 
 
@@ -165,6 +266,14 @@ class InvalidArgument(PegaHipError, ValueError):
 
 
 class StorageError(PegaHipError):
+    pass
+
+
+class InstanceMissing(PegaHipError):
+    pass
+
+
+class WorkerMissing(PegaHipError):
     pass
 
 
@@ -198,4 +307,8 @@ def check(status: int) -> None:
         raise InvalidArgument(status, msg)
     if status == PF_ERR_STORAGE:
         raise StorageError(status, msg)
+    if status == PF_ERR_INSTANCE_MISSING:
+        raise InstanceMissing(status, msg)
+    if status == PF_ERR_WORKER_MISSING:
+        raise WorkerMissing(status, msg)
     raise PegaHipError(status, msg)

@@ -1,0 +1,125 @@
+// Host-side images of saved blocks.  Follows pegaflow-core/src/block.rs:62-454
+// and pegaflow-common/src/block.rs:1-43 of the reference.
+#pragma once
+
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "pf_pool.hpp"
+
+namespace pf {
+
+// pegaflow-common/src/block.rs:5-21.
+struct BlockKey {
+  std::string ns;
+  std::string hash;  // raw bytes
+  bool operator<(const BlockKey& o) const { return ns != o.ns ? ns < o.ns : hash < o.hash; }
+  bool operator==(const BlockKey& o) const { return ns == o.ns && hash == o.hash; }
+};
+
+// pegaflow-common/src/block.rs:30-43: group 0 keeps the raw hash, groups >= 1
+// append the big-endian group id.
+inline std::string group_hash(const std::string& hash, uint32_t group_id) {
+  if (group_id == 0) return hash;
+  std::string out = hash;
+  out.push_back(static_cast<char>((group_id >> 24) & 0xFF));
+  out.push_back(static_cast<char>((group_id >> 16) & 0xFF));
+  out.push_back(static_cast<char>((group_id >> 8) & 0xFF));
+  out.push_back(static_cast<char>(group_id & 0xFF));
+  return out;
+}
+
+// block.rs:62-88: one contiguous range of pinned memory; keeps its allocation alive.
+class Segment {
+ public:
+  // False when [host_ptr, host_ptr + size) is not inside `allocation`.
+  static bool create(uint8_t* host_ptr, uint64_t size, std::shared_ptr<PinnedAllocation> allocation,
+                     Segment* out) {
+    MappedPinnedPtr p;
+    if (!allocation || !allocation->mapped_ptr_for_host_range(host_ptr, size, &p)) return false;
+    out->ptr_ = p;
+    out->size_ = size;
+    out->allocation_ = std::move(allocation);
+    return true;
+  }
+  MappedPinnedPtr ptr() const { return ptr_; }
+  uint64_t size() const { return size_; }
+  uint64_t allocation_id() const { return allocation_ ? allocation_->allocation_id() : 0; }
+
+ private:
+  MappedPinnedPtr ptr_;
+  uint64_t size_ = 0;
+  std::shared_ptr<PinnedAllocation> allocation_;
+};
+
+// block.rs:90-199: an ordered list of segments, layout-agnostic.
+class RawBlock {
+ public:
+  RawBlock() = default;
+  explicit RawBlock(std::vector<Segment> segments) : segments_(std::move(segments)) {
+    for (const auto& s : segments_) total_size_ += s.size();
+  }
+  static RawBlock single_segment(Segment s) { return RawBlock(std::vector<Segment>{std::move(s)}); }
+  static RawBlock two_segments(Segment k, Segment v) {
+    return RawBlock(std::vector<Segment>{std::move(k), std::move(v)});
+  }
+  size_t num_segments() const { return segments_.size(); }
+  bool segment_mapped_ptr(size_t i, MappedPinnedPtr* out) const {
+    if (i >= segments_.size()) return false;
+    *out = segments_[i].ptr();
+    return true;
+  }
+  uint64_t segment_allocation_id(size_t i) const {
+    return i < segments_.size() ? segments_[i].allocation_id() : 0;
+  }
+  uint64_t segment_size(size_t i) const { return i < segments_.size() ? segments_[i].size() : 0; }
+  uint64_t memory_footprint() const { return total_size_; }
+
+ private:
+  std::vector<Segment> segments_;
+  uint64_t total_size_ = 0;
+};
+
+// block.rs:255-330: immutable once every slot is filled.
+class SealedBlock {
+ public:
+  explicit SealedBlock(std::vector<RawBlock> slots) : slots_(std::move(slots)) {
+    for (const auto& b : slots_) footprint_ += b.memory_footprint();
+  }
+  const RawBlock* get_slot(size_t slot_id) const {
+    return slot_id < slots_.size() ? &slots_[slot_id] : nullptr;
+  }
+  size_t num_slots() const { return slots_.size(); }
+  uint64_t memory_footprint() const { return footprint_; }
+
+ private:
+  std::vector<RawBlock> slots_;
+  uint64_t footprint_ = 0;
+};
+
+// block.rs:346-454: slots arrive one by one; seals when none remain.
+class InflightBlock {
+ public:
+  explicit InflightBlock(size_t total_slots)
+      : slots_(total_slots), filled_(total_slots, false), remaining_(total_slots) {}
+  enum class Insert { Inserted, Completed, Duplicate };
+  Insert insert_slot(size_t slot_id, RawBlock block) {
+    if (slot_id >= slots_.size() || filled_[slot_id]) return Insert::Duplicate;
+    slots_[slot_id] = std::move(block);
+    filled_[slot_id] = true;
+    --remaining_;
+    return remaining_ == 0 ? Insert::Completed : Insert::Inserted;
+  }
+  size_t total_slots() const { return slots_.size(); }
+  size_t filled_count() const { return slots_.size() - remaining_; }
+  std::shared_ptr<SealedBlock> seal() { return std::make_shared<SealedBlock>(std::move(slots_)); }
+
+ private:
+  std::vector<RawBlock> slots_;
+  std::vector<bool> filled_;
+  size_t remaining_;
+};
+
+}  // namespace pf

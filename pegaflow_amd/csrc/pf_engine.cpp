@@ -1,0 +1,754 @@
+#include "pf_engine.hpp"
+
+#include <algorithm>
+#include <set>
+
+#include "pf_common.hpp"
+#include "pf_sync_state.hpp"
+
+namespace pf {
+
+namespace {
+
+constexpr uint64_t kSsdAlignment = 512;
+
+int bad(std::string* err, int code, std::string msg) {
+  if (err) *err = std::move(msg);
+  return code;
+}
+
+}  // namespace
+
+// Per-layer state of one save (offload.rs:52-66).
+struct SaveLayerCtx {
+  std::string layer_name;
+  KVCacheLayout layout;
+  size_t slot_id = 0;
+  uint32_t group = 0;
+  std::vector<std::pair<uint64_t, std::string>> blocks_to_save;  // (block_idx, raw hash)
+  std::vector<std::shared_ptr<RawBlock>> raw_blocks;             // parallel to blocks_to_save
+};
+
+// ---------------------------------------------------------------------------
+// InstanceContext
+// ---------------------------------------------------------------------------
+
+int InstanceContext::check_accepting(int device_id, size_t tp_rank, std::string* err) {
+  if (tp_rank >= tp_size_) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT, "tp_rank " + std::to_string(tp_rank) +
+                                                 " out of range (tp_size " +
+                                                 std::to_string(tp_size_) + ")");
+  }
+  std::lock_guard<std::mutex> lock(mu_);
+  // Duplicate device first: a restarted worker must hear that its device
+  // still exists, not a generic "fully registered" (instance.rs:455-470).
+  if (gpus_.count(device_id)) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT,
+               "GPU context for device " + std::to_string(device_id) + " already exists");
+  }
+  if (topology_) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT,
+               "instance " + id_ + " is already fully registered (" + std::to_string(world_size_) +
+                   " workers); device " + std::to_string(device_id) + " cannot join");
+  }
+  return PF_OK;
+}
+
+int InstanceContext::register_new_gpu(std::shared_ptr<GpuContext> ctx, std::string* err) {
+  std::lock_guard<std::mutex> lock(mu_);
+  const int device_id = ctx->reg.device_id;
+  if (gpus_.count(device_id)) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT,
+               "GPU context for device " + std::to_string(device_id) + " already exists");
+  }
+  if (topology_) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT,
+               "instance " + id_ + " is already fully registered (" + std::to_string(world_size_) +
+                   " workers); device " + std::to_string(device_id) + " cannot join");
+  }
+  std::shared_ptr<LayerTopology> sealed;
+  if (gpus_.size() + 1 == world_size_) {
+    // The registration that completes the worker set seals the topology; if
+    // that fails the registration is rejected as a whole.
+    std::vector<const WorkerRegistration*> workers;
+    for (auto& kv : gpus_) workers.push_back(&kv.second->reg);
+    workers.push_back(&ctx->reg);
+    sealed = std::make_shared<LayerTopology>();
+    std::string cause;
+    if (!LayerTopology::seal(workers, tp_size_, page_first_, id_, world_size_, sealed.get(),
+                             &cause)) {
+      return bad(err, PF_ERR_INVALID_ARGUMENT, cause);
+    }
+  }
+  gpus_[device_id] = std::move(ctx);
+  if (sealed) topology_ = std::move(sealed);
+  return PF_OK;
+}
+
+std::shared_ptr<LayerTopology> InstanceContext::sealed_topology(std::string* err) {
+  std::lock_guard<std::mutex> lock(mu_);
+  if (!topology_ && err) {
+    *err = "instance " + id_ + " registration incomplete: " + std::to_string(gpus_.size()) + "/" +
+           std::to_string(world_size_) + " workers registered";
+  }
+  return topology_;
+}
+
+std::shared_ptr<GpuContext> InstanceContext::get_gpu(int device_id) {
+  std::lock_guard<std::mutex> lock(mu_);
+  auto it = gpus_.find(device_id);
+  return it == gpus_.end() ? nullptr : it->second;
+}
+
+std::string InstanceContext::verify_topology(size_t tp_size, size_t world_size,
+                                             bool page_first) const {
+  if (tp_size_ == tp_size && world_size_ == world_size && page_first_ == page_first) return "";
+  auto b = [](bool v) { return v ? "true" : "false"; };
+  return "exists with tp=" + std::to_string(tp_size_) + ", world=" + std::to_string(world_size_) +
+         ", page_first=" + b(page_first_) + "; requested tp=" + std::to_string(tp_size) +
+         ", world=" + std::to_string(world_size) + ", page_first=" + b(page_first);
+}
+
+// ---------------------------------------------------------------------------
+// Engine
+// ---------------------------------------------------------------------------
+
+std::unique_ptr<Engine> Engine::create(const EngineConfig& cfg, std::string* err, int* status) {
+  std::unique_ptr<Engine> e(new Engine());
+  e->cfg_ = cfg;
+  e->numa_ = NumaTopology::detect();
+  std::string perr;
+  int pstatus = PF_ERR_STORAGE;
+  if (cfg.numa_aware) {
+    e->pool_ = PinnedAllocator::new_numa(cfg.pool_size, e->numa_.gpu_numa_nodes(), cfg.pool_shards,
+                                         cfg.use_hugepages, cfg.ssd_enabled, cfg.unit_size_hint,
+                                         &perr, &pstatus);
+  } else {
+    e->pool_ = PinnedAllocator::new_global(cfg.pool_size, cfg.pool_shards, cfg.use_hugepages,
+                                           cfg.ssd_enabled, cfg.unit_size_hint, &perr, &pstatus);
+  }
+  if (!e->pool_) {
+    if (err) *err = perr;
+    if (status) *status = pstatus;
+    return nullptr;
+  }
+  return e;
+}
+
+Engine::~Engine() {
+  // Workers first (they may still touch host blocks), then blocks, then the pool.
+  instances_.clear();
+  leases_.clear();
+  inflight_.clear();
+  sealed_.clear();
+}
+
+std::shared_ptr<InstanceContext> Engine::get_instance(const std::string& id, std::string* err) {
+  std::lock_guard<std::mutex> lock(mu_);
+  auto it = instances_.find(id);
+  if (it == instances_.end()) {
+    if (err) *err = "instance " + id + " not registered";
+    return nullptr;
+  }
+  return it->second;
+}
+
+int Engine::register_context_layer_batch_strided(
+    const std::string& instance_id, const std::string& ns, int device_id, size_t tp_rank,
+    size_t pp_rank, size_t tp_size, size_t world_size, const std::vector<std::string>& layer_names,
+    const std::vector<uint64_t>& data_ptrs, const std::vector<uint64_t>& size_bytes,
+    const std::vector<uint64_t>& num_blocks, const std::vector<uint64_t>& bytes_per_block,
+    const std::vector<uint64_t>& kv_stride_bytes, const std::vector<uint64_t>& segments,
+    const std::vector<uint64_t>* block_stride_bytes, const std::vector<uint32_t>* layer_group_ids,
+    TransferMode mode, bool page_first, std::string* err) {
+  const size_t n = layer_names.size();
+  if (data_ptrs.size() != n || size_bytes.size() != n || num_blocks.size() != n ||
+      bytes_per_block.size() != n || kv_stride_bytes.size() != n || segments.size() != n) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT,
+               "registration metadata length mismatch: layer_names=" + std::to_string(n) +
+                   ", data_ptrs=" + std::to_string(data_ptrs.size()) +
+                   ", size_bytes=" + std::to_string(size_bytes.size()) +
+                   ", num_blocks=" + std::to_string(num_blocks.size()) +
+                   ", bytes_per_block=" + std::to_string(bytes_per_block.size()) +
+                   ", kv_stride_bytes=" + std::to_string(kv_stride_bytes.size()) +
+                   ", segments=" + std::to_string(segments.size()));
+  }
+  if (block_stride_bytes && block_stride_bytes->size() != n) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT,
+               "registration metadata length mismatch: layer_names=" + std::to_string(n) +
+                   ", block_stride_bytes=" + std::to_string(block_stride_bytes->size()));
+  }
+  if (layer_group_ids && layer_group_ids->size() != n) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT,
+               "registration metadata length mismatch: layer_names=" + std::to_string(n) +
+                   ", layer_group_ids=" + std::to_string(layer_group_ids->size()));
+  }
+  if (device_id < 0) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT,
+               "device_id " + std::to_string(device_id) + " must be >= 0");
+  }
+  if (tp_size == 0 || world_size == 0) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT, "tp_size and world_size must be > 0");
+  }
+  auto ctx = std::make_shared<GpuContext>();
+  ctx->reg.device_id = device_id;
+  ctx->reg.tp_rank = tp_rank;
+  ctx->reg.pp_rank = pp_rank;
+  for (size_t i = 0; i < n; ++i) {
+    KVCacheLayout layout;
+    std::string cause;
+    if (!KVCacheLayout::create(data_ptrs[i], size_bytes[i], num_blocks[i], bytes_per_block[i],
+                               kv_stride_bytes[i], segments[i], &layout, &cause) ||
+        (block_stride_bytes && !layout.with_block_stride((*block_stride_bytes)[i], &cause))) {
+      return bad(err, PF_ERR_INVALID_ARGUMENT, "layer " + layer_names[i] + ": " + cause);
+    }
+    if (cfg_.ssd_enabled) layout.with_ssd_padding(kSsdAlignment);
+    if (!ctx->reg.kv_caches.emplace(layer_names[i], layout).second) {
+      return bad(err, PF_ERR_INVALID_ARGUMENT,
+                 "duplicate layer name in registration batch: " + layer_names[i]);
+    }
+    if (layer_group_ids) ctx->reg.layer_groups[layer_names[i]] = (*layer_group_ids)[i];
+  }
+  if (ctx->reg.kv_caches.empty()) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT,
+               "device " + std::to_string(device_id) + " registered no KV cache layers");
+  }
+
+  // get_or_create_instance (lib.rs:196-222).
+  std::shared_ptr<InstanceContext> instance;
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    auto it = instances_.find(instance_id);
+    if (it != instances_.end()) {
+      std::string mismatch = it->second->verify_topology(tp_size, world_size, page_first);
+      if (!mismatch.empty()) {
+        return bad(err, PF_ERR_INVALID_ARGUMENT, "instance " + instance_id + " " + mismatch);
+      }
+      instance = it->second;
+    } else {
+      instance = std::make_shared<InstanceContext>(instance_id, ns, tp_size, world_size, page_first);
+      instances_[instance_id] = instance;
+    }
+  }
+  ctx->preferred_numa = numa_.numa_for_gpu(device_id);
+  if (pool_->is_numa() && ctx->preferred_numa.is_unknown()) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT,
+               "NUMA-aware allocation is enabled, but GPU " + std::to_string(device_id) +
+                   " NUMA affinity is unknown. Please ensure the GPU's PCI NUMA node is "
+                   "detectable, or disable NUMA-aware allocation.");
+  }
+  int st = instance->check_accepting(device_id, tp_rank, err);
+  if (st != PF_OK) return st;
+  std::string werr;
+  int wstatus = PF_ERR_DEVICE_INIT;
+  ctx->worker_pool = GpuWorkerPool::spawn(device_id, ctx->preferred_numa, mode,
+                                          cfg_.use_descriptor_backends, &werr, &wstatus);
+  if (!ctx->worker_pool) return bad(err, wstatus, werr);
+  return instance->register_new_gpu(std::move(ctx), err);
+}
+
+int Engine::unregister_instance(const std::string& instance_id, std::string* err) {
+  std::shared_ptr<InstanceContext> removed;
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    auto it = instances_.find(instance_id);
+    if (it == instances_.end()) {
+      return bad(err, PF_ERR_INSTANCE_MISSING, "instance " + instance_id + " not registered");
+    }
+    removed = it->second;
+    instances_.erase(it);
+    for (auto lit = leases_.begin(); lit != leases_.end();) {
+      lit = lit->second.instance_id == instance_id ? leases_.erase(lit) : std::next(lit);
+    }
+  }
+  removed.reset();  // joins the worker threads outside the lock
+  return PF_OK;
+}
+
+bool Engine::evict_one() {
+  // mu_ held by the caller.  Oldest first; blocks that are leased or being
+  // loaded (someone else holds a reference) stay.
+  for (size_t i = 0; i < sealed_order_.size();) {
+    auto sit = sealed_.find(sealed_order_[i]);
+    if (sit == sealed_.end()) {
+      sealed_order_.erase(sealed_order_.begin() + static_cast<std::ptrdiff_t>(i));
+      continue;
+    }
+    if (sit->second.use_count() > 1) {
+      ++i;
+      continue;
+    }
+    sealed_.erase(sit);
+    sealed_order_.erase(sealed_order_.begin() + static_cast<std::ptrdiff_t>(i));
+    return true;
+  }
+  return false;
+}
+
+std::shared_ptr<PinnedAllocation> Engine::allocate(uint64_t size, NumaNode numa) {
+  for (;;) {
+    if (auto a = pool_->allocate(size, numa)) return a;
+    std::lock_guard<std::mutex> lock(mu_);
+    if (!evict_one()) return nullptr;
+  }
+}
+
+size_t Engine::cached_blocks() {
+  std::lock_guard<std::mutex> lock(mu_);
+  return sealed_.size();
+}
+
+size_t Engine::evict_all() {
+  std::lock_guard<std::mutex> lock(mu_);
+  size_t n = 0;
+  while (evict_one()) ++n;
+  return n;
+}
+
+// offload.rs:182-282.
+int Engine::alloc_page_first_targets(const LayerTopology& topo, SaveLayerCtx* ctxs, size_t n,
+                                     NumaNode numa,
+                                     std::vector<std::shared_ptr<PinnedAllocation>>* pages,
+                                     std::vector<LayerTransferData>* out, std::string* err) {
+  const size_t shard = ctxs[0].slot_id;
+  size_t page_size = 0;
+  topo.shard_page_size(shard, &page_size);
+  const auto& reference = ctxs[0].blocks_to_save;
+  std::set<size_t> layer_ids;
+  for (size_t i = 0; i < n; ++i) {
+    if (ctxs[i].layout.is_split()) {
+      return bad(err, PF_ERR_INVALID_ARGUMENT,
+                 "page-first save does not support split K/V (layer " + ctxs[i].layer_name + ")");
+    }
+    if (ctxs[i].slot_id != shard) {
+      return bad(err, PF_ERR_INVALID_ARGUMENT,
+                 "page-first save spans multiple shards (one writer must save one shard)");
+    }
+    if (ctxs[i].blocks_to_save != reference) {
+      return bad(err, PF_ERR_INVALID_ARGUMENT,
+                 "page-first save requires the same block set across all layers");
+    }
+    size_t id = 0;
+    std::string cause;
+    if (!topo.layer_id(ctxs[i].layer_name, &id, &cause)) {
+      return bad(err, PF_ERR_INVALID_ARGUMENT, cause);
+    }
+    layer_ids.insert(id);
+  }
+  size_t shard_layers = 0;
+  topo.shard_layer_count(shard, &shard_layers);
+  if (layer_ids.size() != shard_layers) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT,
+               "page-first save must cover all " + std::to_string(shard_layers) +
+                   " layers of shard " + std::to_string(shard) + ", got " +
+                   std::to_string(layer_ids.size()) +
+                   " distinct (one worker must write a shard's entire page)");
+  }
+  if (page_size == 0) return bad(err, PF_ERR_STORAGE, "page size is zero");
+  for (size_t b = 0; b < reference.size(); ++b) {
+    auto page = allocate(page_size, numa);
+    if (!page) return bad(err, PF_ERR_STORAGE, "pinned pool exhausted while allocating page");
+    pages->push_back(std::move(page));
+  }
+  for (size_t i = 0; i < n; ++i) {
+    size_t id = 0, offset = 0, layer_bytes = 0;
+    topo.layer_id(ctxs[i].layer_name, &id, nullptr);
+    topo.page_placement(id, &offset, &layer_bytes);
+    LayerTransferData ltd;
+    ltd.layer_name = ctxs[i].layer_name;
+    ltd.layout = ctxs[i].layout;
+    for (size_t b = 0; b < reference.size(); ++b) {
+      Segment seg;
+      const auto& page = (*pages)[b];
+      if (!Segment::create(page->as_ptr() + offset, layer_bytes, page, &seg)) {
+        return bad(err, PF_ERR_STORAGE, "page slice exceeds its pinned allocation");
+      }
+      auto raw = std::make_shared<RawBlock>(RawBlock::single_segment(std::move(seg)));
+      TransferBlock tb;
+      tb.block_idx = reference[b].first;
+      tb.block.raw = raw.get();
+      tb.block.keep = raw;
+      ltd.blocks.push_back(std::move(tb));
+    }
+    out->push_back(std::move(ltd));
+  }
+  return PF_OK;
+}
+
+int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank, size_t pp_rank,
+                                 int device_id, const std::vector<LayerSave>& saves,
+                                 std::string* err) {
+  auto instance = get_instance(instance_id, err);
+  if (!instance) return PF_ERR_INSTANCE_MISSING;
+  auto topo = instance->sealed_topology(err);
+  if (!topo) return PF_ERR_INVALID_ARGUMENT;
+  const std::string ns = instance->ns();
+
+  // ---- Phase 0: resolve metadata, bounds-check block ids ------------------
+  auto gpu = instance->get_gpu(device_id);
+  if (!gpu) {
+    return bad(err, PF_ERR_WORKER_MISSING,
+               "instance " + instance_id + " has no worker for device " + std::to_string(device_id));
+  }
+  if (gpu->reg.tp_rank != tp_rank || gpu->reg.pp_rank != pp_rank) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT,
+               "device_id " + std::to_string(device_id) + " is registered for tp_rank " +
+                   std::to_string(gpu->reg.tp_rank) + ", pp_rank " +
+                   std::to_string(gpu->reg.pp_rank) + ", but save requested tp_rank " +
+                   std::to_string(tp_rank) + ", pp_rank " + std::to_string(pp_rank));
+  }
+  std::vector<SaveLayerCtx> ctxs;
+  std::set<std::pair<uint32_t, std::string>> hashes_to_save;
+  for (const LayerSave& s : saves) {
+    if (s.block_ids.size() != s.block_hashes.size()) {
+      return bad(err, PF_ERR_INVALID_ARGUMENT,
+                 "block_ids length " + std::to_string(s.block_ids.size()) +
+                     " does not match block_hashes " + std::to_string(s.block_hashes.size()) +
+                     " for layer " + s.layer_name);
+    }
+    size_t layer_id = 0;
+    std::string cause;
+    if (!topo->layer_id(s.layer_name, &layer_id, &cause)) {
+      return bad(err, PF_ERR_INVALID_ARGUMENT, cause);
+    }
+    auto lit = gpu->reg.kv_caches.find(s.layer_name);
+    if (lit == gpu->reg.kv_caches.end()) {
+      return bad(err, PF_ERR_INVALID_ARGUMENT,
+                 "layer " + s.layer_name + " not registered on device");
+    }
+    SaveLayerCtx ctx;
+    ctx.layer_name = s.layer_name;
+    ctx.layout = lit->second;
+    if (!topo->slot_index(layer_id, tp_rank, &ctx.slot_id, &cause)) {
+      return bad(err, PF_ERR_INVALID_ARGUMENT, cause);
+    }
+    ctx.group = topo->group_of_layer(layer_id);
+    const uint64_t nb = ctx.layout.num_blocks();
+    for (size_t i = 0; i < s.block_ids.size(); ++i) {
+      if (s.block_ids[i] >= nb) {
+        return bad(err, PF_ERR_INVALID_ARGUMENT,
+                   "block_id " + std::to_string(s.block_ids[i]) + " out of range (num_blocks=" +
+                       std::to_string(nb) + ") for layer " + s.layer_name);
+      }
+      ctx.blocks_to_save.emplace_back(s.block_ids[i], s.block_hashes[i]);
+    }
+    if (ctx.blocks_to_save.empty()) continue;
+    for (auto& b : ctx.blocks_to_save) hashes_to_save.emplace(ctx.group, b.second);
+    ctxs.push_back(std::move(ctx));
+  }
+  if (ctxs.empty()) return PF_OK;
+
+  // ---- Phase 1: drop hashes whose group-encoded key is already cached -----
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    for (auto it = hashes_to_save.begin(); it != hashes_to_save.end();) {
+      BlockKey key{ns, group_hash(it->second, it->first)};
+      it = sealed_.count(key) ? hashes_to_save.erase(it) : std::next(it);
+    }
+  }
+  if (hashes_to_save.empty()) return PF_OK;
+  for (auto& ctx : ctxs) {
+    auto& v = ctx.blocks_to_save;
+    v.erase(std::remove_if(v.begin(), v.end(),
+                           [&](const std::pair<uint64_t, std::string>& b) {
+                             return !hashes_to_save.count({ctx.group, b.second});
+                           }),
+            v.end());
+  }
+  ctxs.erase(std::remove_if(ctxs.begin(), ctxs.end(),
+                            [](const SaveLayerCtx& c) { return c.blocks_to_save.empty(); }),
+             ctxs.end());
+  if (ctxs.empty()) return PF_OK;
+
+  // ---- Phase 2: pinned allocation + host images ----------------------------
+  const NumaNode numa = gpu->preferred_numa;
+  const bool page_first = topo->is_page_first();
+  std::vector<LayerTransferData> gpu_layers;
+  std::vector<std::shared_ptr<PinnedAllocation>> pages;
+  if (page_first) {
+    int st = alloc_page_first_targets(*topo, ctxs.data(), ctxs.size(), numa, &pages, &gpu_layers,
+                                      err);
+    if (st != PF_OK) return st;
+  } else {
+    for (auto& ctx : ctxs) {
+      const KVCacheLayout& layout = ctx.layout;
+      const size_t num = ctx.blocks_to_save.size();
+      const size_t alloc_count = cfg_.blockwise_alloc ? num : 1;
+      const size_t per_alloc = cfg_.blockwise_alloc ? 1 : num;
+      auto alloc_pinned = [&](uint64_t stride, const char* what,
+                              std::shared_ptr<PinnedAllocation>* out) -> int {
+        uint64_t size = 0;
+        if (__builtin_mul_overflow(stride, static_cast<uint64_t>(per_alloc), &size) || size == 0) {
+          return bad(err, PF_ERR_STORAGE, std::string("allocation size overflow for ") + what);
+        }
+        *out = allocate(size, numa);
+        if (!*out) {
+          return bad(err, PF_ERR_STORAGE,
+                     std::string("pinned pool exhausted while allocating ") + what);
+        }
+        return PF_OK;
+      };
+      for (size_t a = 0; a < alloc_count; ++a) {
+        if (layout.is_split()) {
+          const uint64_t stride = layout.padded_segment_bytes();
+          std::shared_ptr<PinnedAllocation> k_alloc, v_alloc;
+          int st = alloc_pinned(stride, "K segment buffer", &k_alloc);
+          if (st == PF_OK) st = alloc_pinned(stride, "V segment buffer", &v_alloc);
+          if (st != PF_OK) return st;
+          for (size_t i = 0; i < per_alloc; ++i) {
+            Segment k, v;
+            if (!Segment::create(k_alloc->as_ptr() + i * stride, stride, k_alloc, &k) ||
+                !Segment::create(v_alloc->as_ptr() + i * stride, stride, v_alloc, &v)) {
+              return bad(err, PF_ERR_STORAGE, "segment exceeds its pinned allocation");
+            }
+            ctx.raw_blocks.push_back(
+                std::make_shared<RawBlock>(RawBlock::two_segments(std::move(k), std::move(v))));
+          }
+        } else {
+          const uint64_t stride = layout.padded_block_bytes();
+          std::shared_ptr<PinnedAllocation> alloc;
+          int st = alloc_pinned(stride, "block buffer", &alloc);
+          if (st != PF_OK) return st;
+          for (size_t i = 0; i < per_alloc; ++i) {
+            Segment s;
+            if (!Segment::create(alloc->as_ptr() + i * stride, stride, alloc, &s)) {
+              return bad(err, PF_ERR_STORAGE, "segment exceeds its pinned allocation");
+            }
+            ctx.raw_blocks.push_back(
+                std::make_shared<RawBlock>(RawBlock::single_segment(std::move(s))));
+          }
+        }
+      }
+      LayerTransferData ltd;
+      ltd.layer_name = ctx.layer_name;
+      ltd.layout = layout;
+      for (size_t i = 0; i < num; ++i) {
+        TransferBlock tb;
+        tb.block_idx = ctx.blocks_to_save[i].first;
+        tb.block.raw = ctx.raw_blocks[i].get();
+        tb.block.keep = ctx.raw_blocks[i];
+        ltd.blocks.push_back(std::move(tb));
+      }
+      gpu_layers.push_back(std::move(ltd));
+    }
+  }
+
+  // ---- Phase 3: one GPU copy task, one synchronisation ---------------------
+  TaskResult res = gpu->worker_pool->batch_save(std::move(gpu_layers)).get();
+  if (res.status != PF_OK) return bad(err, res.status, res.message);
+
+  // ---- Phase 4: insert into the store --------------------------------------
+  std::lock_guard<std::mutex> lock(mu_);
+  auto insert = [&](const BlockKey& key, size_t total_slots, size_t slot_id, RawBlock block) {
+    if (sealed_.count(key)) return;
+    auto it = inflight_.find(key);
+    if (it == inflight_.end()) it = inflight_.emplace(key, InflightBlock(total_slots)).first;
+    if (it->second.insert_slot(slot_id, std::move(block)) == InflightBlock::Insert::Completed) {
+      sealed_[key] = it->second.seal();
+      sealed_order_.push_back(key);
+      inflight_.erase(it);
+    }
+  };
+  if (page_first) {
+    const size_t slot_id = ctxs[0].slot_id;
+    size_t page_size = 0;
+    topo->shard_page_size(slot_id, &page_size);
+    for (size_t b = 0; b < pages.size(); ++b) {
+      Segment seg;
+      Segment::create(pages[b]->as_ptr(), page_size, pages[b], &seg);
+      insert(BlockKey{ns, ctxs[0].blocks_to_save[b].second}, topo->total_slots(), slot_id,
+             RawBlock::single_segment(std::move(seg)));
+    }
+  } else {
+    for (auto& ctx : ctxs) {
+      size_t total_slots = 0;
+      std::string cause;
+      if (!topo->group_total_slots(ctx.group, &total_slots, &cause)) {
+        return bad(err, PF_ERR_INVALID_ARGUMENT, cause);
+      }
+      for (size_t i = 0; i < ctx.blocks_to_save.size(); ++i) {
+        insert(BlockKey{ns, group_hash(ctx.blocks_to_save[i].second, ctx.group)}, total_slots,
+               ctx.slot_id, std::move(*ctx.raw_blocks[i]));
+      }
+    }
+  }
+  return PF_OK;
+}
+
+int Engine::query_prefix(const std::string& instance_id, const std::vector<std::string>& hashes,
+                         uint64_t* out_hits, uint64_t* out_lease, std::string* err) {
+  auto instance = get_instance(instance_id, err);
+  if (!instance) return PF_ERR_INSTANCE_MISSING;
+  std::lock_guard<std::mutex> lock(mu_);
+  Lease lease;
+  lease.instance_id = instance_id;
+  for (const std::string& h : hashes) {
+    auto it = sealed_.find(BlockKey{instance->ns(), h});
+    if (it == sealed_.end()) break;
+    lease.blocks.push_back(it->second);
+  }
+  *out_hits = lease.blocks.size();
+  *out_lease = 0;
+  if (!lease.blocks.empty()) {
+    *out_lease = next_lease_++;
+    leases_[*out_lease] = std::move(lease);
+  }
+  return PF_OK;
+}
+
+bool Engine::release_query_lease(uint64_t lease) {
+  std::lock_guard<std::mutex> lock(mu_);
+  return leases_.erase(lease) > 0;
+}
+
+int Engine::batch_load_kv_blocks_multi_layer(
+    const std::string& instance_id, size_t tp_rank, int device_id,
+    const std::vector<std::vector<std::string>>& layer_groups,
+    const std::vector<LoadRequest>& loads, const std::string& load_state_shm,
+    std::future<TaskResult>* out, std::string* err) {
+  auto instance = get_instance(instance_id, err);
+  if (!instance) return PF_ERR_INSTANCE_MISSING;
+  auto topo = instance->sealed_topology(err);
+  if (!topo) return PF_ERR_INVALID_ARGUMENT;
+  auto gpu = instance->get_gpu(device_id);
+  if (!gpu) {
+    return bad(err, PF_ERR_WORKER_MISSING,
+               "instance " + instance_id + " has no worker for device " + std::to_string(device_id));
+  }
+  if (layer_groups.empty()) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT, "load requires at least one layer group");
+  }
+  size_t layer_count = 0;
+  std::set<std::string> unique;
+  for (auto& g : layer_groups) {
+    layer_count += g.size();
+    unique.insert(g.begin(), g.end());
+  }
+  if (unique.size() != layer_count) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT, "load layer names must be unique across groups");
+  }
+  // Each load group maps to exactly one storage group (lib.rs:748-770).
+  std::vector<int64_t> storage_group(layer_groups.size(), -1);
+  for (size_t gi = 0; gi < layer_groups.size(); ++gi) {
+    for (const std::string& name : layer_groups[gi]) {
+      size_t id = 0;
+      std::string cause;
+      if (!topo->layer_id(name, &id, &cause)) return bad(err, PF_ERR_INVALID_ARGUMENT, cause);
+      int64_t g = topo->group_of_layer(id);
+      if (storage_group[gi] >= 0 && storage_group[gi] != g) {
+        return bad(err, PF_ERR_INVALID_ARGUMENT,
+                   "load group mixes storage groups " + std::to_string(storage_group[gi]) +
+                       " and " + std::to_string(g) + " (layer " + name + ")");
+      }
+      storage_group[gi] = g;
+    }
+  }
+  // Consume the leases.
+  std::vector<std::vector<std::pair<uint64_t, size_t>>> targets(layer_groups.size());
+  std::vector<std::shared_ptr<SealedBlock>> block_cache;
+  for (const LoadRequest& lr : loads) {
+    std::vector<std::shared_ptr<SealedBlock>> blocks;
+    {
+      std::lock_guard<std::mutex> lock(mu_);
+      auto it = leases_.find(lr.lease);
+      if (it == leases_.end() || it->second.instance_id != instance_id) {
+        return bad(err, PF_ERR_STORAGE,
+                   "query lease " + std::to_string(lr.lease) + " not found for instance " +
+                       instance_id);
+      }
+      blocks = std::move(it->second.blocks);
+      leases_.erase(it);
+    }
+    if (lr.block_ids_by_group.size() != layer_groups.size()) {
+      return bad(err, PF_ERR_INVALID_ARGUMENT,
+                 "load group count " + std::to_string(lr.block_ids_by_group.size()) +
+                     " does not match layer group count " + std::to_string(layer_groups.size()));
+    }
+    const size_t start = block_cache.size();
+    for (size_t gi = 0; gi < layer_groups.size(); ++gi) {
+      const auto& ids = lr.block_ids_by_group[gi];
+      if (blocks.size() != ids.size()) {
+        return bad(err, PF_ERR_INVALID_ARGUMENT,
+                   "query lease block count " + std::to_string(blocks.size()) +
+                       " does not match destination block count " + std::to_string(ids.size()) +
+                       " for group " + std::to_string(gi));
+      }
+      if (storage_group[gi] >= 0) {
+        size_t expected = 0;
+        std::string cause;
+        if (!topo->group_total_slots(static_cast<uint32_t>(storage_group[gi]), &expected, &cause)) {
+          return bad(err, PF_ERR_INVALID_ARGUMENT, cause);
+        }
+        for (size_t si = 0; si < ids.size(); ++si) {
+          if (ids[si] >= 0 && blocks[si]->num_slots() != expected) {
+            return bad(err, PF_ERR_INVALID_ARGUMENT,
+                       "stored block has " + std::to_string(blocks[si]->num_slots()) +
+                           " slots but storage group " + std::to_string(storage_group[gi]) +
+                           " of instance " + instance_id + " expects " + std::to_string(expected) +
+                           ": namespace is shared by incompatible KV layouts");
+          }
+        }
+      }
+      for (size_t si = 0; si < ids.size(); ++si) {
+        if (ids[si] >= 0) targets[gi].emplace_back(static_cast<uint64_t>(ids[si]), start + si);
+      }
+    }
+    block_cache.insert(block_cache.end(), blocks.begin(), blocks.end());
+  }
+  // One LayerTransferData per layer.
+  std::vector<LayerTransferData> layers;
+  for (size_t gi = 0; gi < layer_groups.size(); ++gi) {
+    for (const std::string& name : layer_groups[gi]) {
+      size_t layer_id = 0;
+      topo->layer_id(name, &layer_id, nullptr);
+      auto lit = gpu->reg.kv_caches.find(name);
+      if (lit == gpu->reg.kv_caches.end()) {
+        return bad(err, PF_ERR_INVALID_ARGUMENT,
+                   "layer " + name + " not registered on device " + std::to_string(device_id));
+      }
+      size_t slot_id = 0;
+      std::string cause;
+      if (!topo->slot_index(layer_id, tp_rank, &slot_id, &cause)) {
+        return bad(err, PF_ERR_INVALID_ARGUMENT, cause);
+      }
+      size_t host_offset = 0, unused = 0;
+      if (!topo->page_placement(layer_id, &host_offset, &unused)) host_offset = 0;
+      LayerTransferData ltd;
+      ltd.layer_name = name;
+      ltd.layout = lit->second;
+      for (auto& t : targets[gi]) {
+        const auto& sealed = block_cache[t.second];
+        const RawBlock* raw = sealed->get_slot(slot_id);
+        if (!raw) {
+          return bad(err, PF_ERR_INVALID_ARGUMENT,
+                     "stored block is missing slot " + std::to_string(slot_id) + " for layer " +
+                         name);
+        }
+        TransferBlock tb;
+        tb.block_idx = t.first;
+        tb.block.raw = raw;
+        tb.block.keep = sealed;
+        tb.block.offset = host_offset;
+        ltd.blocks.push_back(std::move(tb));
+      }
+      if (!ltd.blocks.empty()) layers.push_back(std::move(ltd));
+    }
+  }
+  if (layers.empty()) {
+    // Nothing to load: complete at once (lib.rs:885-890).
+    std::promise<TaskResult> p;
+    p.set_value(TaskResult());
+    *out = p.get_future();
+    if (!load_state_shm.empty()) {
+      std::string aerr;
+      if (auto ls = LoadState::attach(load_state_shm, &aerr)) ls->set_completed();
+    }
+    return PF_OK;
+  }
+  LoadCompletion completion;
+  completion.load_state_shm = load_state_shm;
+  *out = gpu->worker_pool->submit_load(std::move(layers), std::move(completion));
+  return PF_OK;
+}
+
+}  // namespace pf

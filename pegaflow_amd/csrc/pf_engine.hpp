@@ -1,0 +1,147 @@
+// Save / load by block ID over the transfer path: registration, host image
+// construction, submission to the per-GPU workers, and the minimal block
+// store the cycle needs.  Follows the parts of PegaEngine that sit on the
+// path (pegaflow-core/src/lib.rs:228-440,654-898, offload.rs:182-659,
+// instance.rs:293-478,680-860 of the reference).  The cache policy behind
+// the reference's StorageEngine (TinyLFU/LRU, SSD, RDMA, prefetch) is not
+// reproduced: blocks are kept until evicted oldest-first under pool pressure.
+#pragma once
+
+#include <cstdint>
+#include <future>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "pf_block.hpp"
+#include "pf_pool.hpp"
+#include "pf_topology.hpp"
+#include "pf_worker.hpp"
+
+namespace pf {
+
+struct EngineConfig {
+  uint64_t pool_size = 0;
+  bool use_hugepages = false;
+  bool numa_aware = false;        // one pool per NUMA node that has a GPU
+  uint32_t pool_shards = 1;
+  bool blockwise_alloc = false;   // one pinned allocation per block instead of per layer
+  bool ssd_enabled = false;       // pad host strides to 512 B; regular (CPU-readable) backing
+  bool use_descriptor_backends = false;  // workers use per-fragment descriptors + backends
+  uint64_t unit_size_hint = 0;
+};
+
+// block.rs:20-25.
+struct LayerSave {
+  std::string layer_name;
+  std::vector<uint64_t> block_ids;
+  std::vector<std::string> block_hashes;
+};
+
+// One lease's destinations: per load group, one entry per leased block; -1 = skip.
+struct LoadRequest {
+  uint64_t lease = 0;
+  std::vector<std::vector<int64_t>> block_ids_by_group;
+};
+
+// instance.rs:293-378.
+struct GpuContext {
+  WorkerRegistration reg;
+  NumaNode preferred_numa;
+  std::unique_ptr<GpuWorkerPool> worker_pool;
+};
+
+// instance.rs:380-478,680-860.
+class InstanceContext {
+ public:
+  InstanceContext(std::string id, std::string ns, size_t tp_size, size_t world_size,
+                  bool page_first)
+      : id_(std::move(id)), ns_(std::move(ns)), tp_size_(tp_size), world_size_(world_size),
+        page_first_(page_first) {}
+  int register_new_gpu(std::shared_ptr<GpuContext> ctx, std::string* err);
+  // Fails while workers are still registering.
+  std::shared_ptr<LayerTopology> sealed_topology(std::string* err);
+  std::shared_ptr<GpuContext> get_gpu(int device_id);
+  std::string verify_topology(size_t tp_size, size_t world_size, bool page_first) const;
+  const std::string& id() const { return id_; }
+  const std::string& ns() const { return ns_; }
+  size_t tp_size() const { return tp_size_; }
+  // Validation that must precede the (expensive) GPU context construction.
+  int check_accepting(int device_id, size_t tp_rank, std::string* err);
+
+ private:
+  std::string id_, ns_;
+  size_t tp_size_, world_size_;
+  bool page_first_;
+  std::mutex mu_;
+  std::map<int, std::shared_ptr<GpuContext>> gpus_;
+  std::shared_ptr<LayerTopology> topology_;
+};
+
+class Engine {
+ public:
+  static std::unique_ptr<Engine> create(const EngineConfig& cfg, std::string* err, int* status);
+  ~Engine();
+
+  // lib.rs:302-440.
+  int register_context_layer_batch_strided(
+      const std::string& instance_id, const std::string& ns, int device_id, size_t tp_rank,
+      size_t pp_rank, size_t tp_size, size_t world_size, const std::vector<std::string>& layer_names,
+      const std::vector<uint64_t>& data_ptrs, const std::vector<uint64_t>& size_bytes,
+      const std::vector<uint64_t>& num_blocks, const std::vector<uint64_t>& bytes_per_block,
+      const std::vector<uint64_t>& kv_stride_bytes, const std::vector<uint64_t>& segments,
+      const std::vector<uint64_t>* block_stride_bytes, const std::vector<uint32_t>* layer_group_ids,
+      TransferMode mode, bool page_first, std::string* err);
+  // lib.rs:443-457.
+  int unregister_instance(const std::string& instance_id, std::string* err);
+  // offload.rs:293-659.  Returns once the bytes are in host memory and the
+  // blocks are queryable.
+  int batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank, size_t pp_rank,
+                           int device_id, const std::vector<LayerSave>& saves, std::string* err);
+  // Longest cached prefix of `hashes` (group 0 keys) + a lease over those
+  // blocks (lib.rs:506-546,614-629).
+  int query_prefix(const std::string& instance_id, const std::vector<std::string>& hashes,
+                   uint64_t* out_hits, uint64_t* out_lease, std::string* err);
+  bool release_query_lease(uint64_t lease);
+  // lib.rs:654-898.  On success *out is fulfilled when the load settles (at
+  // once when nothing is to be loaded).
+  int batch_load_kv_blocks_multi_layer(const std::string& instance_id, size_t tp_rank,
+                                       int device_id,
+                                       const std::vector<std::vector<std::string>>& layer_groups,
+                                       const std::vector<LoadRequest>& loads,
+                                       const std::string& load_state_shm,
+                                       std::future<TaskResult>* out, std::string* err);
+  void pool_usage(uint64_t* used, uint64_t* total) { pool_->usage(used, total); }
+  size_t cached_blocks();
+  // Test hook / pressure valve: drop every sealed block that is not leased.
+  size_t evict_all();
+
+ private:
+  Engine() = default;
+  std::shared_ptr<InstanceContext> get_instance(const std::string& id, std::string* err);
+  // storage/mod.rs:294-330: allocate, evicting oldest sealed blocks on pressure.
+  std::shared_ptr<PinnedAllocation> allocate(uint64_t size, NumaNode numa);
+  bool evict_one();
+  int alloc_page_first_targets(const LayerTopology& topo, struct SaveLayerCtx* ctxs, size_t n,
+                               NumaNode numa, std::vector<std::shared_ptr<PinnedAllocation>>* pages,
+                               std::vector<LayerTransferData>* out, std::string* err);
+
+  EngineConfig cfg_;
+  std::unique_ptr<PinnedAllocator> pool_;
+  NumaTopology numa_;
+  std::mutex mu_;  // instances, store, leases
+  std::map<std::string, std::shared_ptr<InstanceContext>> instances_;
+  std::map<BlockKey, InflightBlock> inflight_;
+  std::map<BlockKey, std::shared_ptr<SealedBlock>> sealed_;
+  std::vector<BlockKey> sealed_order_;  // insertion order, for oldest-first eviction
+  struct Lease {
+    std::string instance_id;
+    std::vector<std::shared_ptr<SealedBlock>> blocks;
+  };
+  std::map<uint64_t, Lease> leases_;
+  uint64_t next_lease_ = 1;
+};
+
+}  // namespace pf

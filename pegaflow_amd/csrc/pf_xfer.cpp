@@ -22,26 +22,15 @@
 #include "pf_kernels.hpp"
 #include "pf_layout.hpp"
 #include "pf_transfer.hpp"
+#include "pf_xfer.hpp"
 
 namespace pf {
 
 namespace {
 
-// Measured on MI355X (Llama-3.1-8B shape, 327 MB per layer): slots smaller than
-// a layer cost cross-stream hand-offs between DMA copies (16 MiB slots reach
-// ~25 GB/s on saves, 64 MiB ~40-55 GB/s and unstable, 256 MiB 56.3 GB/s,
-// 512 MiB 56.7 GB/s of a 57.3 GB/s link), so a slot holds a whole layer.
-constexpr uint64_t kDefaultSlotBytes = 512ull << 20;
-constexpr uint32_t kDefaultSlots = 2;
-constexpr uint64_t kDefaultAutoStagedMin = 4ull << 20;
-constexpr int kDefaultUnroll = 4;
-// Zero-copy launches are capped to a few workgroups: the host link, not the
-// GPU, is the bound, and fewer in-flight requests use it better.  Measured on
-// MI355X (Llama shape, 16 layers per launch): 64 workgroups load at 57.4 GB/s
-// and save at 55.0-55.8 GB/s; 2048 and more give 56.0 and 54.5 GB/s.
-constexpr uint32_t kDefaultZeroCopyWorkgroups = 64;
-
 bool aligned16(uint64_t v) { return (v & 15ull) == 0; }
+
+}  // namespace
 
 struct LayerPlan {
   std::string name;
@@ -63,114 +52,6 @@ struct LayerPlan {
   size_t src_index = 0;         // index in the caller's layer array
 };
 
-}  // namespace
-
-class Xfer {
- public:
-  explicit Xfer(const pf_xfer_config* cfg) {
-    if (cfg) {
-      if (cfg->staging_slot_bytes) slot_bytes_ = cfg->staging_slot_bytes;
-      if (cfg->staging_slots) n_slots_ = cfg->staging_slots;
-      if (cfg->zerocopy_max_workgroups) zc_max_wg_ = cfg->zerocopy_max_workgroups;
-      if (cfg->auto_staged_min_bytes) auto_min_ = cfg->auto_staged_min_bytes;
-      if (cfg->tile_unroll) unroll_ = static_cast<int>(cfg->tile_unroll);
-    }
-  }
-
-  ~Xfer() {
-    if (side_) {
-      (void)hipStreamSynchronize(side_);
-      (void)hipStreamDestroy(side_);
-    }
-    for (auto& sl : slots_) {
-      if (sl.ready) (void)hipEventDestroy(sl.ready);
-      if (sl.freed) (void)hipEventDestroy(sl.freed);
-      if (sl.buf) (void)hipFree(sl.buf);
-    }
-    if (fork_) (void)hipEventDestroy(fork_);
-    if (join_) (void)hipEventDestroy(join_);
-    for (auto& p : timing_pool_) {
-      (void)hipEventDestroy(p.first);
-      (void)hipEventDestroy(p.second);
-    }
-    (void)hipGetLastError();
-  }
-
-  int init() {
-    if (!unroll_supported(unroll_)) {
-      return fail(PF_ERR_INVALID_ARGUMENT, "tile_unroll must be 1, 2, 4 or 8, got %d", unroll_);
-    }
-    if (n_slots_ < 2 || n_slots_ > 16) {
-      return fail(PF_ERR_INVALID_ARGUMENT, "staging_slots must be in [2, 16], got %u", n_slots_);
-    }
-    hipError_t e = hipGetDevice(&device_);
-    if (e != hipSuccess) {
-      fail_hip(e, "hipGetDevice");
-      return fail(PF_ERR_DEVICE_INIT, "transfer engine init failed: %s", last_error().c_str());
-    }
-    PF_HIP(hipStreamCreateWithFlags(&side_, hipStreamNonBlocking));
-    PF_HIP(hipEventCreateWithFlags(&fork_, hipEventDisableTiming));
-    PF_HIP(hipEventCreateWithFlags(&join_, hipEventDisableTiming));
-    slots_.resize(n_slots_);
-    for (auto& sl : slots_) {
-      PF_HIP(hipEventCreateWithFlags(&sl.ready, hipEventDisableTiming));
-      PF_HIP(hipEventCreateWithFlags(&sl.freed, hipEventDisableTiming));
-    }
-    return PF_OK;
-  }
-
-  int run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save, hipStream_t s);
-
-  void set_layer_events(pf_event_t* events, uint64_t n) {
-    layer_events_.clear();
-    if (events) {
-      for (uint64_t i = 0; i < n; ++i) layer_events_.push_back(native(events[i]));
-    }
-  }
-  int last_path() const { return last_path_; }
-  void set_timing(bool on) { timing_ = on; }
-  int last_kernel_ms(float* out_ms, uint32_t* out_launches);
-
- private:
-  struct Slot {
-    void* buf = nullptr;
-    uint64_t cap = 0;
-    hipEvent_t ready = nullptr;  // contents complete (gather done / fill done)
-    hipEvent_t freed = nullptr;  // contents consumed (drain done / scatter done)
-    bool used = false;
-  };
-
-  int plan_layer(const pf_layer_blocks& in, size_t index, int path, LayerPlan* out, bool* skip);
-  int ensure_slot(Slot& sl, uint64_t bytes);
-  // Zero-copy form: grid-stride kernel over `n_units` units, capped grid.
-  int launch_strided(const BlockUnit* dev_units, uint32_t n_units, uint64_t max_tiles, bool to_far,
-                     hipStream_t s);
-  // Staged form: one tile per workgroup over one unit.
-  int launch_tiles(const BlockUnit* dev_unit, const BlockUnit& host_unit, bool to_far,
-                   hipStream_t s);
-  int timing_begin(hipStream_t s);
-  int timing_end(hipStream_t s);
-
-  int device_ = 0;
-  uint64_t slot_bytes_ = kDefaultSlotBytes;
-  uint32_t n_slots_ = kDefaultSlots;
-  uint32_t zc_max_wg_ = kDefaultZeroCopyWorkgroups;
-  uint64_t auto_min_ = kDefaultAutoStagedMin;
-  int unroll_ = kDefaultUnroll;
-
-  hipStream_t side_ = nullptr;
-  hipEvent_t fork_ = nullptr;
-  hipEvent_t join_ = nullptr;
-  std::vector<Slot> slots_;
-  uint32_t next_slot_ = 0;
-  SlabPool slabs_;
-  std::vector<hipEvent_t> layer_events_;
-  int last_path_ = 0;
-
-  bool timing_ = false;
-  std::vector<std::pair<hipEvent_t, hipEvent_t>> timing_pool_;
-  size_t timing_used_ = 0;
-};
 
 int Xfer::ensure_slot(Slot& sl, uint64_t bytes) {
   if (sl.cap >= bytes) return PF_OK;

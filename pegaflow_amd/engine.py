@@ -1,0 +1,306 @@
+"""Worker pool, load-completion flag and the save/load-by-block-ID engine over
+the C ABI.  Mirrors the reference's GpuWorkerPool
+(pegaflow-core/src/gpu_worker.rs:116-243), LoadState (sync_state.rs:113-188)
+and the path-relevant surface of PegaEngine (lib.rs:228-440,506-546,654-709,
+offload.rs:293-659)."""
+
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Sequence
+
+from . import _lib
+from ._lib import check
+from .transfer import LayerTransferData, TransferMode
+
+LOAD_STATE_PENDING = 0
+LOAD_STATE_SUCCESS = 1
+LOAD_STATE_ERROR = -1
+
+
+class LoadState:
+    """Shared-memory completion flag a submitter polls."""
+
+    def __init__(self, attach_to: str | None = None):
+        self._lib = _lib.load()
+        h = C.c_void_p()
+        if attach_to is None:
+            check(self._lib.pf_load_state_create(C.byref(h)))
+        else:
+            check(self._lib.pf_load_state_attach(attach_to.encode(), C.byref(h)))
+        self.handle = h
+
+    @property
+    def shm_name(self) -> str:
+        return self._lib.pf_load_state_name(self.handle).decode()
+
+    def get(self) -> int:
+        return self._lib.pf_load_state_get(self.handle)
+
+    def set_completed(self) -> None:
+        check(self._lib.pf_load_state_set(self.handle, LOAD_STATE_SUCCESS))
+
+    def set_error(self) -> None:
+        check(self._lib.pf_load_state_set(self.handle, LOAD_STATE_ERROR))
+
+    def close(self) -> None:
+        if self.handle is not None:
+            self._lib.pf_load_state_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+@dataclass
+class TaskResult:
+    done: bool
+    bytes: int
+    elapsed_ms: float
+
+
+class Task:
+    """A submitted load or save; ``wait`` raises if the task failed."""
+
+    def __init__(self, handle, keep=None):
+        self._lib = _lib.load()
+        self.handle = handle
+        self._keep = keep
+
+    def wait(self, timeout_ms: int = -1) -> TaskResult:
+        r = _lib.PfTaskResult()
+        check(self._lib.pf_task_wait(self.handle, timeout_ms, C.byref(r)))
+        return TaskResult(bool(r.done), r.bytes, r.elapsed_ms)
+
+    def close(self) -> None:
+        if self.handle is not None:
+            self._lib.pf_task_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def _pack_layer_transfers(layers: Sequence[LayerTransferData]):
+    n_layers = len(layers)
+    arr = (_lib.PfLayerTransfer * max(n_layers, 1))()
+    keep = []
+    for i, layer in enumerate(layers):
+        nb = len(layer.blocks)
+        idx = (C.c_uint64 * max(nb, 1))(*[int(b) for b in layer.block_idx])
+        blocks = (_lib.PfHostBlock * max(nb, 1))()
+        for j, hb in enumerate(layer.blocks):
+            ns = len(hb.seg_host)
+            blocks[j].num_segments = ns
+            for s in range(ns):
+                blocks[j].seg_host[s] = hb.seg_host[s]
+                blocks[j].seg_device[s] = hb.seg_device[s]
+                blocks[j].seg_alloc[s] = hb.seg_alloc[s]
+                blocks[j].seg_size[s] = hb.seg_size[s] if s < len(hb.seg_size) else 0
+            blocks[j].host_offset = hb.host_offset
+        name = layer.layer_name.encode()
+        keep.append((idx, blocks, name))
+        arr[i].layer_name = name
+        arr[i].layout = layer.layout.c
+        arr[i].block_idx = idx
+        arr[i].blocks = blocks
+        arr[i].n_blocks = nb
+    return arr, n_layers, keep
+
+
+class GpuWorkerPool:
+    """One load thread and one save thread for a GPU, each with its own
+    stream; tasks run serially per thread with one synchronisation each."""
+
+    def __init__(self, device_id: int, numa_node: int = -1, transfer_mode: int = TransferMode.DIRECT,
+                 use_descriptor_backends: bool = False):
+        self._lib = _lib.load()
+        h = C.c_void_p()
+        check(self._lib.pf_worker_pool_spawn(device_id, numa_node, transfer_mode,
+                                             1 if use_descriptor_backends else 0, C.byref(h)))
+        self.handle = h
+
+    def submit_load(self, layers: Sequence[LayerTransferData],
+                    load_state: LoadState | None = None) -> Task:
+        arr, n, keep = _pack_layer_transfers(layers)
+        t = C.c_void_p()
+        shm = load_state.shm_name.encode() if load_state is not None else None
+        check(self._lib.pf_worker_submit_load(self.handle, arr, n, shm, C.byref(t)))
+        return Task(t)
+
+    def batch_save(self, layers: Sequence[LayerTransferData]) -> Task:
+        arr, n, keep = _pack_layer_transfers(layers)
+        t = C.c_void_p()
+        check(self._lib.pf_worker_submit_save(self.handle, arr, n, C.byref(t)))
+        return Task(t)
+
+    def close(self) -> None:
+        if self.handle is not None:
+            self._lib.pf_worker_pool_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+@dataclass
+class LayerSave:
+    """Per-layer save input: layer name, device block ids, content hashes."""
+    layer_name: str
+    block_ids: Sequence[int]
+    block_hashes: Sequence[bytes]
+
+
+def _pack_hashes(hashes: Sequence[bytes]):
+    n = len(hashes)
+    bufs = [(C.c_uint8 * max(len(h), 1)).from_buffer_copy(h if h else b"\0") for h in hashes]
+    ptrs = (C.POINTER(C.c_uint8) * max(n, 1))(*[C.cast(b, C.POINTER(C.c_uint8)) for b in bufs])
+    lens = (C.c_uint32 * max(n, 1))(*[len(h) for h in hashes])
+    return ptrs, lens, bufs
+
+
+class PegaEngine:
+    """Save / query / load by block ID on one node."""
+
+    def __init__(self, pool_size: int, use_hugepages: bool = False, numa_aware: bool = False,
+                 pool_shards: int = 1, blockwise_alloc: bool = False, ssd_enabled: bool = False,
+                 use_descriptor_backends: bool = False, unit_size_hint: int = 0):
+        self._lib = _lib.load()
+        cfg = _lib.PfEngineConfig(pool_size, int(use_hugepages), int(numa_aware), pool_shards,
+                                  int(blockwise_alloc), int(ssd_enabled),
+                                  int(use_descriptor_backends), unit_size_hint)
+        h = C.c_void_p()
+        check(self._lib.pf_engine_create(C.byref(cfg), C.byref(h)))
+        self.handle = h
+
+    def register_context_layer_batch(self, instance_id: str, namespace: str, device_id: int,
+                                     tp_rank: int, pp_rank: int, tp_size: int, world_size: int,
+                                     layer_names: Sequence[str], data_ptrs: Sequence[int],
+                                     size_bytes_list: Sequence[int], num_blocks_list: Sequence[int],
+                                     bytes_per_block_list: Sequence[int],
+                                     kv_stride_bytes_list: Sequence[int],
+                                     segments_list: Sequence[int],
+                                     transfer_mode: int = TransferMode.DIRECT,
+                                     page_first: bool = False,
+                                     block_stride_bytes_list: Sequence[int] | None = None,
+                                     layer_group_ids: Sequence[int] | None = None) -> None:
+        n = len(layer_names)
+        lists = (data_ptrs, size_bytes_list, num_blocks_list, bytes_per_block_list,
+                 kv_stride_bytes_list, segments_list)
+        if any(len(x) != n for x in lists):
+            raise _lib.InvalidArgument(
+                _lib.PF_ERR_INVALID_ARGUMENT,
+                f"registration metadata length mismatch: layer_names={n}, "
+                + ", ".join(f"{k}={len(v)}" for k, v in zip(
+                    ("data_ptrs", "size_bytes", "num_blocks", "bytes_per_block",
+                     "kv_stride_bytes", "segments"), lists)))
+        u64 = C.c_uint64
+        names = (C.c_char_p * max(n, 1))(*[s.encode() for s in layer_names])
+        arrs = [(u64 * max(n, 1))(*[int(v) for v in x]) for x in lists]
+        strides = (u64 * max(n, 1))(*block_stride_bytes_list) if block_stride_bytes_list else None
+        groups = (C.c_uint32 * max(n, 1))(*layer_group_ids) if layer_group_ids else None
+        check(self._lib.pf_engine_register_context_layer_batch(
+            self.handle, instance_id.encode(), namespace.encode(), device_id, tp_rank, pp_rank,
+            tp_size, world_size, n, names, *arrs, strides, groups, transfer_mode,
+            1 if page_first else 0))
+
+    def unregister_instance(self, instance_id: str) -> None:
+        check(self._lib.pf_engine_unregister_instance(self.handle, instance_id.encode()))
+
+    def batch_save_kv_blocks(self, instance_id: str, tp_rank: int, pp_rank: int, device_id: int,
+                             saves: Sequence[LayerSave]) -> None:
+        n = len(saves)
+        arr = (_lib.PfLayerSave * max(n, 1))()
+        keep = []
+        for i, s in enumerate(saves):
+            ids = (C.c_uint64 * max(len(s.block_ids), 1))(*[int(b) for b in s.block_ids])
+            name = s.layer_name.encode()
+            arr[i].layer_name = name
+            arr[i].block_ids = ids
+            arr[i].n_blocks = len(s.block_ids)
+            if len(s.block_hashes) != len(s.block_ids):
+                # offload.rs:328-335
+                raise _lib.InvalidArgument(
+                    _lib.PF_ERR_INVALID_ARGUMENT,
+                    f"block_ids length {len(s.block_ids)} does not match block_hashes "
+                    f"{len(s.block_hashes)} for layer {s.layer_name}")
+            ptrs, lens, bufs = _pack_hashes(s.block_hashes)
+            arr[i].block_hashes = ptrs
+            arr[i].block_hash_lens = lens
+            keep.append((ptrs, lens, bufs))
+            keep.append((ids, name))
+        check(self._lib.pf_engine_batch_save(self.handle, instance_id.encode(), tp_rank, pp_rank,
+                                             device_id, arr, n))
+
+    def query_prefix(self, instance_id: str, hashes: Sequence[bytes]) -> tuple[int, int]:
+        """-> (hit blocks, lease id); lease 0 when nothing hit."""
+        ptrs, lens, _bufs = _pack_hashes(hashes)
+        hits, lease = C.c_uint64(), C.c_uint64()
+        check(self._lib.pf_engine_query_prefix(self.handle, instance_id.encode(), ptrs, lens,
+                                               len(hashes), C.byref(hits), C.byref(lease)))
+        return hits.value, lease.value
+
+    def release_query_lease(self, lease: int) -> None:
+        check(self._lib.pf_engine_release_lease(self.handle, lease))
+
+    def batch_load_kv_blocks_multi_layer(self, instance_id: str, tp_rank: int, device_id: int,
+                                         layer_groups: Sequence[Sequence[str]], lease: int,
+                                         dest_block_ids_by_group: Sequence[Sequence[int | None]],
+                                         load_state: LoadState | None = None) -> Task:
+        g = len(layer_groups)
+        keep = []
+        group_ptrs = (C.POINTER(C.c_char_p) * max(g, 1))()
+        sizes = (C.c_uint64 * max(g, 1))()
+        dests = (C.POINTER(C.c_int64) * max(g, 1))()
+        n_blocks = len(dest_block_ids_by_group[0]) if g else 0
+        for i, names in enumerate(layer_groups):
+            arr = (C.c_char_p * max(len(names), 1))(*[s.encode() for s in names])
+            keep.append(arr)
+            group_ptrs[i] = arr
+            sizes[i] = len(names)
+            ids = dest_block_ids_by_group[i]
+            if len(ids) != n_blocks:
+                raise _lib.InvalidArgument(_lib.PF_ERR_INVALID_ARGUMENT,
+                                           "every load group needs one destination per leased block")
+            d = (C.c_int64 * max(n_blocks, 1))(*[-1 if v is None else int(v) for v in ids])
+            keep.append(d)
+            dests[i] = d
+        t = C.c_void_p()
+        shm = load_state.shm_name.encode() if load_state is not None else None
+        check(self._lib.pf_engine_batch_load(self.handle, instance_id.encode(), tp_rank, device_id,
+                                             g, group_ptrs, sizes, lease, dests, n_blocks, shm,
+                                             C.byref(t)))
+        return Task(t, keep)
+
+    def pool_usage(self) -> tuple[int, int]:
+        used, total = C.c_uint64(), C.c_uint64()
+        check(self._lib.pf_engine_pool_usage(self.handle, C.byref(used), C.byref(total)))
+        return used.value, total.value
+
+    @property
+    def cached_blocks(self) -> int:
+        return self._lib.pf_engine_cached_blocks(self.handle)
+
+    def evict_all(self) -> int:
+        return self._lib.pf_engine_evict_all(self.handle)
+
+    def close(self) -> None:
+        if self.handle is not None:
+            self._lib.pf_engine_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

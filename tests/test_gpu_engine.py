@@ -1,0 +1,310 @@
+"""Worker pool and save/query/load cycle on a real device, mirroring the
+reference's engine integration tests (pegaflow-core/tests/engine_basic.rs,
+hybrid_groups.rs, save_validation.rs) with the same closed-form patterns:
+block i filled with byte (i % 251) + 1, `overwrite(m)` = wrapping add."""
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from pegaflow_amd import _lib
+from pegaflow_amd.engine import (LOAD_STATE_ERROR, LOAD_STATE_SUCCESS, GpuWorkerPool, LayerSave,
+                                 LoadState, PegaEngine)
+from pegaflow_amd.layout import KVCacheLayout
+from pegaflow_amd.runtime import DeviceBuffer, PinnedMemory
+from pegaflow_amd.transfer import HostBlock, LayerTransferData, TransferMode
+from tests.helpers import block_fill_pattern, random_bytes, split_fill_pattern
+
+pytestmark = pytest.mark.gpu
+
+
+def make_block_hashes(n, salt):
+    """salt || u32le(idx)  (tests/common/helpers.rs:91-100)."""
+    return [bytes([salt]) + int(i).to_bytes(4, "little") for i in range(n)]
+
+
+class Layer:
+    def __init__(self, name, num_blocks, block_bytes, overwrite=0, split_kv_stride=None):
+        self.name, self.num_blocks, self.block_bytes = name, num_blocks, block_bytes
+        if split_kv_stride:
+            self.expected = split_fill_pattern(num_blocks, block_bytes, split_kv_stride)
+            self.reg = (block_bytes, split_kv_stride, 2)
+        else:
+            self.expected = block_fill_pattern(num_blocks, block_bytes)
+            self.reg = (block_bytes, 0, 1)
+        self.expected = (self.expected.astype(np.uint16) + overwrite).astype(np.uint8)
+        self.gpu = DeviceBuffer(self.expected.nbytes)
+        self.gpu.copy_from_host(self.expected)
+
+    def zero_gpu(self):
+        self.gpu.fill(0)
+
+    def assert_gpu_matches(self, expected):
+        assert np.array_equal(self.gpu.copy_to_host(), expected), f"GPU data mismatch in {self.name}"
+
+
+def register(engine, instance, layers, page_first=False, mode=TransferMode.DIRECT, ns="test-ns",
+             groups=None):
+    engine.register_context_layer_batch(
+        instance, ns, 0, 0, 0, 1, 1, [l.name for l in layers], [l.gpu.ptr for l in layers],
+        [l.expected.nbytes for l in layers], [l.num_blocks for l in layers],
+        [l.reg[0] for l in layers], [l.reg[1] for l in layers], [l.reg[2] for l in layers],
+        transfer_mode=mode, page_first=page_first, layer_group_ids=groups)
+
+
+@pytest.fixture(params=[False, True], ids=["block_ids", "descriptors"])
+def engine(request, gpu):
+    e = PegaEngine(pool_size=64 << 20, use_descriptor_backends=request.param)
+    yield e
+    e.close()
+
+
+def test_save_query_load_roundtrip(engine):
+    """engine_basic.rs:12-25."""
+    layer = Layer("layer_0", 4, 1024)
+    register(engine, "test-roundtrip", [layer])
+    hashes = make_block_hashes(4, 0)
+    engine.batch_save_kv_blocks("test-roundtrip", 0, 0, 0, [LayerSave("layer_0", [0, 1, 2, 3], hashes)])
+    layer.zero_gpu()
+    hits, lease = engine.query_prefix("test-roundtrip", hashes)
+    assert hits == 4 and lease != 0
+    engine.batch_load_kv_blocks_multi_layer("test-roundtrip", 0, 0, [["layer_0"]], lease,
+                                            [[0, 1, 2, 3]]).wait()
+    layer.assert_gpu_matches(layer.expected)
+    # saving the same hashes again stores nothing new (dedupe against the cache)
+    used = engine.pool_usage()[0]
+    engine.batch_save_kv_blocks("test-roundtrip", 0, 0, 0, [LayerSave("layer_0", [0, 1, 2, 3], hashes)])
+    assert engine.pool_usage()[0] == used and engine.cached_blocks == 4
+
+
+@pytest.mark.parametrize("mode", [TransferMode.DIRECT, TransferMode.KERNEL], ids=["direct", "kernel"])
+def test_split_layout_roundtrip_both_backends(engine, mode):
+    """K/V split registration (tests/common/harness.rs:53-80), both transfer modes."""
+    layer = Layer("kv", 16, 4096, split_kv_stride=16 * 4096)
+    register(engine, f"split-{mode}", [layer], mode=mode)
+    hashes = make_block_hashes(8, 3)
+    ids = [1, 3, 5, 7, 9, 11, 13, 15]
+    engine.batch_save_kv_blocks(f"split-{mode}", 0, 0, 0, [LayerSave("kv", ids, hashes)])
+    layer.zero_gpu()
+    hits, lease = engine.query_prefix(f"split-{mode}", hashes)
+    assert hits == 8
+    dest = [0, 2, 4, 6, 8, 10, 12, 14]
+    engine.batch_load_kv_blocks_multi_layer(f"split-{mode}", 0, 0, [["kv"]], lease, [dest]).wait()
+    want = np.zeros_like(layer.expected)
+    for src, dst in zip(ids, dest):
+        for region in (0, 16 * 4096):
+            want[region + dst * 4096: region + (dst + 1) * 4096] = \
+                layer.expected[region + src * 4096: region + (src + 1) * 4096]
+    layer.assert_gpu_matches(want)
+
+
+def test_page_first_multi_layer_roundtrip(engine, kats):
+    """engine_basic.rs:32-58: three layers of distinct sizes and contents in one page."""
+    case = next(c for c in kats["engine"] if c["name"] == "page_first_multi_layer_roundtrip")
+    layers = [Layer(l["name"], l["num_blocks"], l["block_bytes"], l["overwrite"]) for l in case["layers"]]
+    register(engine, "test-page-first", layers, page_first=True, mode=TransferMode.KERNEL)
+    hashes = make_block_hashes(4, 0xAB)
+    engine.batch_save_kv_blocks("test-page-first", 0, 0, 0,
+                                [LayerSave(l.name, [0, 1, 2, 3], hashes) for l in layers])
+    used, _total = engine.pool_usage()
+    assert used == 4 * case["expect"]["page_size"]  # one 3072-byte page per block
+    for l in layers:
+        l.zero_gpu()
+    hits, lease = engine.query_prefix("test-page-first", hashes)
+    assert hits == 4
+    engine.batch_load_kv_blocks_multi_layer("test-page-first", 0, 0, [[l.name for l in layers]],
+                                            lease, [[0, 1, 2, 3]]).wait()
+    for l in layers:
+        l.assert_gpu_matches(l.expected)
+
+
+def test_partial_layer_page_first_save_is_rejected(engine):
+    """engine_basic.rs:126-160: a page-first save must carry every layer of the shard."""
+    layers = [Layer("layer_a", 4, 512), Layer("layer_b", 4, 1024)]
+    register(engine, "test-partial", layers, page_first=True)
+    hashes = make_block_hashes(2, 1)
+    with pytest.raises(_lib.InvalidArgument, match="must cover all 2 layers of shard 0"):
+        engine.batch_save_kv_blocks("test-partial", 0, 0, 0, [LayerSave("layer_a", [0, 1], hashes)])
+    assert engine.pool_usage()[0] == 0
+
+
+def test_hybrid_groups_load_to_distinct_block_ids(engine, kats):
+    """engine_basic.rs:62-124: same hashes saved from different block ids per
+    layer, loaded into per-group destinations with skips; expected bytes are
+    given explicitly by the reference."""
+    case = next(c for c in kats["engine"] if c["name"] == "hybrid_groups_load_to_distinct_block_ids")
+    layers = [Layer(l["name"], l["num_blocks"], l["block_bytes"], l["overwrite"]) for l in case["layers"]]
+    register(engine, "test-hybrid-groups", layers)
+    hashes = make_block_hashes(2, 0xAC)
+    engine.batch_save_kv_blocks("test-hybrid-groups", 0, 0, 0, [
+        LayerSave(l["name"], l["save_ids"], hashes) for l in case["layers"]])
+    for l in layers:
+        l.zero_gpu()
+    hits, lease = engine.query_prefix("test-hybrid-groups", hashes)
+    assert hits == 2
+    engine.batch_load_kv_blocks_multi_layer(
+        "test-hybrid-groups", 0, 0, [["full_attention"], [], ["gdn"]], lease,
+        [[2, 3], [None, None], [None, 0]]).wait()
+    for l in layers:
+        want = np.zeros(4 * 1024, dtype=np.uint8)
+        for blk, fill in case["expect"][l.name].items():
+            want[int(blk) * 1024:(int(blk) + 1) * 1024] = fill
+        l.assert_gpu_matches(want)
+
+
+def test_save_validation_and_load_errors(engine):
+    """save_validation.rs:12-42 and the load-side checks of lib.rs:715-883."""
+    layer = Layer("layer_0", 4, 1024)
+    register(engine, "test-validate", [layer])
+    with pytest.raises(_lib.InvalidArgument, match="block_ids length 2 does not match block_hashes 1"):
+        engine.batch_save_kv_blocks("test-validate", 0, 0, 0,
+                                    [LayerSave("layer_0", [0, 1], make_block_hashes(1, 9))])
+    with pytest.raises(_lib.InvalidArgument, match=r"block_id 4 out of range \(num_blocks=4\) for layer layer_0"):
+        engine.batch_save_kv_blocks("test-validate", 0, 0, 0,
+                                    [LayerSave("layer_0", [4], make_block_hashes(1, 9))])
+    with pytest.raises(_lib.InvalidArgument, match="layer nope is not registered"):
+        engine.batch_save_kv_blocks("test-validate", 0, 0, 0,
+                                    [LayerSave("nope", [0], make_block_hashes(1, 9))])
+    with pytest.raises(_lib.InstanceMissing):
+        engine.batch_save_kv_blocks("ghost", 0, 0, 0, [])
+    with pytest.raises(_lib.InvalidArgument, match="registered for tp_rank 0, pp_rank 0"):
+        engine.batch_save_kv_blocks("test-validate", 0, 1, 0,
+                                    [LayerSave("layer_0", [0], make_block_hashes(1, 9))])
+    assert engine.pool_usage()[0] == 0
+    hashes = make_block_hashes(2, 5)
+    engine.batch_save_kv_blocks("test-validate", 0, 0, 0, [LayerSave("layer_0", [0, 1], hashes)])
+    # prefix semantics: a miss in the middle ends the prefix
+    hits, lease = engine.query_prefix("test-validate", [hashes[0], b"missing", hashes[1]])
+    assert hits == 1
+    ls = LoadState()
+    with pytest.raises(_lib.InvalidArgument, match="does not match destination block count"):
+        engine.batch_load_kv_blocks_multi_layer("test-validate", 0, 0, [["layer_0"]], lease,
+                                                [[0, 1]], load_state=ls)
+    assert ls.get() == LOAD_STATE_ERROR  # pre-submit failure marks the LoadState
+    ls.close()
+    with pytest.raises(_lib.StorageError, match="query lease"):
+        engine.batch_load_kv_blocks_multi_layer("test-validate", 0, 0, [["layer_0"]], lease, [[0]])
+    # zero resolved blocks: completes at once with success
+    hits, lease = engine.query_prefix("test-validate", hashes)
+    ls = LoadState()
+    engine.batch_load_kv_blocks_multi_layer("test-validate", 0, 0, [["layer_0"]], lease,
+                                            [[None, None]], load_state=ls).wait()
+    assert ls.get() == LOAD_STATE_SUCCESS
+    ls.close()
+    # registration errors
+    with pytest.raises(_lib.InvalidArgument, match="already exists"):
+        register(engine, "test-validate", [layer])
+    with pytest.raises(_lib.InvalidArgument, match="exists with tp=1, world=1, page_first=false"):
+        engine.register_context_layer_batch("test-validate", "test-ns", 0, 0, 0, 2, 2, ["x"],
+                                            [layer.gpu.ptr], [4096], [4], [1024], [0], [1])
+    with pytest.raises(_lib.InvalidArgument, match="layer bad: .*too small"):
+        engine.register_context_layer_batch("fresh", "test-ns", 0, 0, 0, 1, 1, ["bad"],
+                                            [layer.gpu.ptr], [1024], [4], [1024], [0], [1])
+    engine.unregister_instance("test-validate")
+    with pytest.raises(_lib.InstanceMissing):
+        engine.unregister_instance("test-validate")
+
+
+def test_pool_pressure_evicts_oldest_unleased_blocks(gpu):
+    """storage/mod.rs:294-330: allocate, evict, retry; exhausted when nothing
+    can be evicted."""
+    e = PegaEngine(pool_size=64 * 1024)
+    layer = Layer("layer_0", 64, 4096)
+    register(e, "pressure", [layer])
+    first = make_block_hashes(8, 1)
+    e.batch_save_kv_blocks("pressure", 0, 0, 0, [LayerSave("layer_0", list(range(8)), first)])
+    second = make_block_hashes(8, 2)
+    e.batch_save_kv_blocks("pressure", 0, 0, 0, [LayerSave("layer_0", list(range(8, 16)), second)])
+    assert e.cached_blocks == 16 and e.pool_usage()[0] == 64 * 1024
+    # a third batch only fits after evicting an older batch's allocation
+    third = make_block_hashes(8, 3)
+    e.batch_save_kv_blocks("pressure", 0, 0, 0, [LayerSave("layer_0", list(range(16, 24)), third)])
+    assert e.query_prefix("pressure", first)[0] == 0
+    assert e.query_prefix("pressure", third)[0] == 8
+    # leased blocks are not evictable: with everything leased the pool is exhausted
+    _h, l2 = e.query_prefix("pressure", second)
+    _h, l3 = e.query_prefix("pressure", third)
+    with pytest.raises(_lib.StorageError, match="pinned pool exhausted"):
+        e.batch_save_kv_blocks("pressure", 0, 0, 0,
+                               [LayerSave("layer_0", list(range(24, 32)), make_block_hashes(8, 4))])
+    e.release_query_lease(l2)
+    e.release_query_lease(l3)
+    e.close()
+
+
+def test_blockwise_alloc_and_odd_segment_size(gpu):
+    """--blockwise-alloc gives every block its own K and V allocation (the
+    worker then falls back to per-fragment descriptors); 1000-byte segments in
+    512-byte pool units leave unit padding that must never be written."""
+    for kw in (dict(blockwise_alloc=True), dict(unit_size_hint=512)):
+        e = PegaEngine(pool_size=8 << 20, **kw)
+        layer = Layer("kv", 16, 1000, split_kv_stride=16 * 1000)  # 1000-byte segments
+        register(e, "bw", [layer], mode=TransferMode.KERNEL)
+        hashes = make_block_hashes(5, 7)
+        ids = [2, 4, 6, 8, 10]
+        e.batch_save_kv_blocks("bw", 0, 0, 0, [LayerSave("kv", ids, hashes)])
+        layer.zero_gpu()
+        _h, lease = e.query_prefix("bw", hashes)
+        e.batch_load_kv_blocks_multi_layer("bw", 0, 0, [["kv"]], lease, [ids]).wait()
+        want = np.zeros_like(layer.expected)
+        for b in ids:
+            for region in (0, 16 * 1000):
+                want[region + b * 1000: region + (b + 1) * 1000] = \
+                    layer.expected[region + b * 1000: region + (b + 1) * 1000]
+        layer.assert_gpu_matches(want)
+        e.close()
+
+
+@pytest.mark.parametrize("use_desc", [False, True], ids=["block_ids", "descriptors"])
+@pytest.mark.parametrize("mode", [TransferMode.DIRECT, TransferMode.KERNEL], ids=["direct", "kernel"])
+def test_worker_pool_matches_oracle(gpu, mode, use_desc):
+    """Raw worker ABI: a save task then a load task with a LoadState, checked
+    against the oracle's descriptor executor on the same inputs."""
+    rng = np.random.default_rng(40)
+    nb, seg, n = 64, 8192, 24
+    cache0 = random_bytes(rng, 2 * nb * seg)
+    dev = DeviceBuffer(cache0.nbytes)
+    dev.copy_from_host(cache0)
+    host = PinnedMemory(2 * n * seg)
+    host.as_numpy()[:] = 0xC3
+    layout = KVCacheLayout(dev.ptr, cache0.nbytes, nb, seg, nb * seg, 2)
+    ids = rng.choice(nb, n, replace=False)
+    blocks = [HostBlock((host.host_ptr + i * seg, host.host_ptr + (n + i) * seg),
+                        (host.device_ptr + i * seg, host.device_ptr + (n + i) * seg), (1, 2),
+                        (seg, seg)) for i in range(n)]
+    pool = GpuWorkerPool(0, -1, mode, use_descriptor_backends=use_desc)
+    res = pool.batch_save([LayerTransferData("kv", layout, ids, blocks)]).wait()
+    assert res.done and res.bytes == 2 * n * seg
+    ocache = cache0.copy()
+    ok = np.full(n * seg, 0xC3, dtype=np.uint8)
+    ov = np.full(n * seg, 0xC3, dtype=np.uint8)
+    O.transfer_layer(O.layout_over(ocache, nb, seg, nb * seg, 2), ids.astype(np.uint32), ok, ov,
+                     host_is_src=False)
+    img = host.as_numpy()
+    assert np.array_equal(img[: n * seg], ok) and np.array_equal(img[n * seg:], ov)
+    dest = rng.choice(nb, n, replace=False)
+    dev.fill(0x11)
+    ls = LoadState()
+    pool.submit_load([LayerTransferData("kv", layout, dest, blocks)], ls).wait()
+    assert ls.get() == LOAD_STATE_SUCCESS
+    ocache2 = np.full_like(cache0, 0x11)
+    O.transfer_layer(O.layout_over(ocache2, nb, seg, nb * seg, 2), dest.astype(np.uint32), ok, ov,
+                     host_is_src=True)
+    assert np.array_equal(dev.copy_to_host(), ocache2)
+    # failure: a bad block id fails the task and flips the LoadState to error
+    bad_ls = LoadState()
+    bad = pool.submit_load([LayerTransferData("model.layers.3", layout, [nb], blocks[:1])], bad_ls)
+    with pytest.raises(_lib.StorageError, match=r"layer model.layers.3: block 64 out of range \(64 blocks\)"):
+        bad.wait()
+    assert bad_ls.get() == LOAD_STATE_ERROR
+    assert np.array_equal(dev.copy_to_host(), ocache2)
+    for x in (ls, bad_ls):
+        x.close()
+    pool.close()
+    host.close()
+    dev.close()
+
+
+def test_worker_pool_init_failure_is_synchronous(gpu):
+    with pytest.raises(_lib.PegaHipError, match="Failed to initialise GPU worker on device 99"):
+        GpuWorkerPool(99)
