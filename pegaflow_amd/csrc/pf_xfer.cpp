@@ -43,6 +43,7 @@ struct LayerPlan {
   uint64_t host_dev[2] = {0, 0};
   uint64_t host_stride = 0;
   const uint64_t* page_dev = nullptr;  // device-visible page bases, host array
+  const uint64_t* page_host = nullptr; // host addresses of the same pages
   uint64_t page_offset = 0;
   bool staged = false;
   bool vec_ok = false;
@@ -180,6 +181,7 @@ int Xfer::plan_layer(const pf_layer_blocks& in, size_t index, int path, LayerPla
     }
     far_aligned = far_aligned && aligned16(in.page_offset);
     p.page_dev = in.page_host_device;
+    p.page_host = in.page_host;
     p.page_offset = in.page_offset;
   } else {
     if (in.host_stride < p.frag_bytes) {
@@ -221,6 +223,10 @@ int Xfer::plan_layer(const pf_layer_blocks& in, size_t index, int path, LayerPla
       p.staged = false;
       break;
     case PF_PATH_STAGED:
+      if (paged) {
+        p.staged = false;  // run() decides: whole-page packing or an error
+        break;
+      }
       if (!dense) {
         return fail(PF_ERR_INVALID_ARGUMENT,
                     "layer %s: the staged path needs a dense host image (host_stride == fragment "
@@ -236,6 +242,169 @@ int Xfer::plan_layer(const pf_layer_blocks& in, size_t index, int path, LayerPla
       return fail(PF_ERR_INVALID_ARGUMENT, "unknown transfer path %d", path);
   }
   return PF_OK;
+}
+
+// Can this call be served by packing whole pages?  Needs: every layer paged over
+// the same pages and the same block list, one fragment per block, slices that
+// do not overlap and (for saves) cover their common range without gaps, and
+// pages laid back to back in runs.
+bool Xfer::plan_page_pack(const std::vector<LayerPlan>& plans, bool save, PagePack* out) {
+  const LayerPlan& first = plans.front();
+  const uint64_t n = first.n_blocks;
+  uint64_t lo = UINT64_MAX, hi = 0, covered = 0;
+  for (const LayerPlan& p : plans) {
+    if (p.page_dev == nullptr || p.n_seg != 1 || p.n_blocks != n) return false;
+    if (p.page_dev != first.page_dev &&
+        std::memcmp(p.page_dev, first.page_dev, n * sizeof(uint64_t)) != 0) {
+      return false;
+    }
+    if (p.ids != first.ids && std::memcmp(p.ids, first.ids, n * sizeof(uint32_t)) != 0) {
+      return false;
+    }
+    lo = std::min(lo, p.page_offset);
+    hi = std::max(hi, p.page_offset + p.frag_bytes);
+    covered += p.frag_bytes;
+  }
+  // Overlap check: sort the slices.
+  std::vector<std::pair<uint64_t, uint64_t>> slices;
+  for (const LayerPlan& p : plans) slices.emplace_back(p.page_offset, p.frag_bytes);
+  std::sort(slices.begin(), slices.end());
+  for (size_t i = 1; i < slices.size(); ++i) {
+    if (slices[i - 1].first + slices[i - 1].second > slices[i].first) return false;
+  }
+  const uint64_t page_bytes = hi - lo;
+  if (save) {
+    // A whole-page drain writes every byte of [lo, hi): all of it must be payload.
+    if (covered != page_bytes) return false;
+  } else if (covered * 10 < page_bytes * 9) {
+    return false;  // loading a small part of each page: do not drag the rest over the link
+  }
+  // Runs of pages that sit back to back, host and device side alike.
+  out->runs.clear();
+  uint64_t start = 0;
+  for (uint64_t i = 1; i <= n; ++i) {
+    const bool adjacent = i < n && first.page_dev[i] == first.page_dev[i - 1] + page_bytes &&
+                          first.page_host[i] == first.page_host[i - 1] + page_bytes;
+    if (!adjacent) {
+      out->runs.emplace_back(start, i - start);
+      start = i;
+    }
+  }
+  // Many short runs mean many small copies: not worth staging.
+  if (out->runs.size() * 8 > n && n > 8) return false;
+  out->lo = lo;
+  out->page_bytes = page_bytes;
+  return true;
+}
+
+int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uint64_t n_layers,
+                        bool save, hipStream_t s) {
+  const LayerPlan& first = plans.front();
+  const uint64_t n = first.n_blocks;
+  const size_t n_plans = plans.size();
+  uint64_t per_unit = std::max<uint64_t>(slot_bytes_ / pack.page_bytes, 1);
+  per_unit = std::min<uint64_t>(per_unit, kMaxTileBlocks);
+  if (n_plans > kMaxTileUnits) {
+    return fail(PF_ERR_INVALID_ARGUMENT, "too many layers in one page-packed call: %zu", n_plans);
+  }
+  struct Chunk {
+    uint64_t first, count;
+  };
+  std::vector<Chunk> chunks;
+  for (const auto& run : pack.runs) {
+    for (uint64_t off = 0; off < run.second; off += per_unit) {
+      chunks.push_back({run.first + off, std::min(per_unit, run.second - off)});
+    }
+  }
+  uint64_t max_chunk_bytes = 0, max_frag = 0;
+  for (const Chunk& c : chunks) max_chunk_bytes = std::max(max_chunk_bytes, c.count * pack.page_bytes);
+  for (const LayerPlan& p : plans) max_frag = std::max(max_frag, p.frag_bytes);
+  for (auto& sl : slots_) {
+    int st = ensure_slot(sl, max_chunk_bytes);
+    if (st != PF_OK) return st;
+  }
+  // Slab: one BlockUnit per (chunk, layer), then the shared id list.
+  const uint64_t units_bytes = (chunks.size() * n_plans * sizeof(BlockUnit) + 255) & ~255ull;
+  const uint64_t slab_bytes = units_bytes + ((n * sizeof(uint32_t) + 255) & ~255ull);
+  SlabPool::Slab* slab = nullptr;
+  int st = slabs_.acquire(slab_bytes, &slab);
+  if (st != PF_OK) return st;
+  uint8_t* slab_host = static_cast<uint8_t*>(slab->host);
+  const uint64_t slab_dev = reinterpret_cast<uint64_t>(slab->dev);
+  std::memcpy(slab_host + units_bytes, first.ids, n * sizeof(uint32_t));
+  BlockUnit* units_host = reinterpret_cast<BlockUnit*>(slab_host);
+  const BlockUnit* units_dev = reinterpret_cast<const BlockUnit*>(slab_dev);
+  std::vector<uint32_t> chunk_slot(chunks.size());
+  for (size_t ci = 0; ci < chunks.size(); ++ci) {
+    chunk_slot[ci] = next_slot_;
+    next_slot_ = (next_slot_ + 1) % n_slots_;
+    const uint64_t base = reinterpret_cast<uint64_t>(slots_[chunk_slot[ci]].buf);
+    for (size_t pi = 0; pi < n_plans; ++pi) {
+      const LayerPlan& p = plans[pi];
+      BlockUnit& u = units_host[ci * n_plans + pi];
+      std::memset(&u, 0, sizeof(u));
+      u.near_base = p.layout.data_ptr();
+      u.block_stride = p.layout.block_stride_bytes();
+      u.kv_stride = 0;
+      u.frag_bytes = p.frag_bytes;
+      u.far_base[0] = base + (p.page_offset - pack.lo);
+      u.far_stride = pack.page_bytes;
+      u.ids = reinterpret_cast<const uint32_t*>(slab_dev + units_bytes) + chunks[ci].first;
+      u.n_blocks = static_cast<uint32_t>(chunks[ci].count);
+      u.n_seg = 1;
+      u.tiles_per_frag = 1;
+      u.vec_ok = aligned16(p.layout.data_ptr()) && aligned16(p.layout.block_stride_bytes()) &&
+                 aligned16(p.page_offset - pack.lo) && aligned16(pack.page_bytes);
+    }
+  }
+
+  PF_HIP(hipMemcpyAsync(slab->dev, slab->host, slab_bytes, hipMemcpyHostToDevice, s));
+  hipStream_t side = timing_ ? s : side_;
+  if (side != s) {
+    PF_HIP(hipEventRecord(fork_, s));
+    PF_HIP(hipStreamWaitEvent(side, fork_, 0));
+  }
+  for (size_t ci = 0; ci < chunks.size(); ++ci) {
+    const Chunk& c = chunks[ci];
+    Slot& sl = slots_[chunk_slot[ci]];
+    uint8_t* host_ptr = reinterpret_cast<uint8_t*>(first.page_host[c.first] + pack.lo);
+    const uint64_t bytes = c.count * pack.page_bytes;
+    auto launch = [&](bool to_far) -> int {
+      int rc = timing_begin(s);
+      if (rc != PF_OK) return rc;
+      rc = launch_block_tiles(units_dev + ci * n_plans, static_cast<uint32_t>(n_plans),
+                              static_cast<uint32_t>(c.count), max_frag, to_far, s);
+      if (rc != PF_OK) return rc;
+      return timing_end(s);
+    };
+    if (save) {
+      if (sl.used) PF_HIP(hipStreamWaitEvent(s, sl.freed, 0));
+      st = launch(true);
+      if (st != PF_OK) return st;
+      PF_HIP(hipEventRecord(sl.ready, s));
+      PF_HIP(hipStreamWaitEvent(side, sl.ready, 0));
+      PF_HIP(hipMemcpyAsync(host_ptr, sl.buf, bytes, hipMemcpyDeviceToHost, side));
+      PF_HIP(hipEventRecord(sl.freed, side));
+    } else {
+      if (sl.used) PF_HIP(hipStreamWaitEvent(side, sl.freed, 0));
+      PF_HIP(hipMemcpyAsync(sl.buf, host_ptr, bytes, hipMemcpyHostToDevice, side));
+      PF_HIP(hipEventRecord(sl.ready, side));
+      PF_HIP(hipStreamWaitEvent(s, sl.ready, 0));
+      st = launch(false);
+      if (st != PF_OK) return st;
+      PF_HIP(hipEventRecord(sl.freed, s));
+    }
+    sl.used = true;
+  }
+  if (save && side != s) {
+    PF_HIP(hipEventRecord(join_, side));
+    PF_HIP(hipStreamWaitEvent(s, join_, 0));
+  }
+  // Every layer of a page lands together: all per-layer events fire at the end.
+  if (!layer_events_.empty()) {
+    for (uint64_t li = 0; li < n_layers; ++li) PF_HIP(hipEventRecord(layer_events_[li], s));
+  }
+  return slabs_.release_after(slab, s);
 }
 
 int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save,
@@ -265,6 +434,31 @@ int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool s
       for (uint64_t li = 0; li < n_layers; ++li) PF_HIP(hipEventRecord(layer_events_[li], s));
     }
     return PF_OK;
+  }
+  // Page-first images whose layer slices tile contiguous pages are packed page
+  // by page in staging and cross the link as whole pages.
+  if (path != PF_PATH_ZEROCOPY && plans.front().page_dev != nullptr) {
+    PagePack pack;
+    if (plan_page_pack(plans, save, &pack)) {
+      uint64_t total = 0;
+      for (const LayerPlan& p : plans) total += p.layer_bytes;
+      if (path == PF_PATH_STAGED || total >= auto_min_) {
+        last_path_ = PF_PATH_STAGED;
+        return run_page_pack(plans, pack, n_layers, save, s);
+      }
+    } else if (path == PF_PATH_STAGED) {
+      return fail(PF_ERR_INVALID_ARGUMENT,
+                  "the staged path needs a dense host image (host_stride == fragment size) or "
+                  "page-first layers that tile contiguous pages");
+    }
+  } else if (path == PF_PATH_STAGED) {
+    for (const LayerPlan& p : plans) {
+      if (p.page_dev != nullptr) {
+        return fail(PF_ERR_INVALID_ARGUMENT,
+                    "layer %s: the staged path needs a dense host image (host_stride == fragment "
+                    "size, no page table)", p.name.c_str());
+      }
+    }
   }
   last_path_ = plans.front().staged ? PF_PATH_STAGED : PF_PATH_ZEROCOPY;
 

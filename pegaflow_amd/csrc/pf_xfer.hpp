@@ -121,6 +121,15 @@ class Xfer {
     bool used = false;
   };
 
+  // Whole-page packing of page-first layers (see plan_page_pack).
+  struct PagePack {
+    uint64_t lo = 0;          // first covered byte of a page
+    uint64_t page_bytes = 0;  // covered bytes per page
+    std::vector<std::pair<uint64_t, uint64_t>> runs;  // (first position, count) of adjacent pages
+  };
+  bool plan_page_pack(const std::vector<LayerPlan>& plans, bool save, PagePack* out);
+  int run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uint64_t n_layers,
+                    bool save, hipStream_t s);
   int plan_layer(const pf_layer_blocks& in, size_t index, int path, LayerPlan* out, bool* skip);
   int ensure_slot(Slot& sl, uint64_t bytes);
   // Zero-copy form: grid-stride kernel over `n_units` units, capped grid.

@@ -334,3 +334,118 @@ def test_duplicate_source_ids_get_their_own_host_image(xfer, stream):
         assert np.array_equal(img[0], ek) and np.array_equal(img[1], ev)
     host.close()
     case.close()
+
+
+def _paged_setup(rng, sizes, num_blocks, n, page_gap_after=None, stride_extra=0):
+    """Layers of `sizes` bytes per block over pages laid back to back (with an
+    optional hole after position `page_gap_after`)."""
+    offsets = np.concatenate([[0], np.cumsum(sizes)[:-1]]).astype(int)
+    page = int(sum(sizes)) + stride_extra
+    hole = 3 if page_gap_after is not None else 0
+    pool = PinnedMemory((n + hole) * page)
+    pool.as_numpy()[:] = SENT
+    idx = np.arange(n)
+    if page_gap_after is not None:
+        idx = np.where(idx > page_gap_after, idx + hole, idx)
+    page_host = (pool.host_ptr + idx * page).astype(np.uint64)
+    page_dev = (pool.device_ptr + idx * page).astype(np.uint64)
+    ids = rng.choice(num_blocks, n, replace=False).astype(np.uint32)
+    cases = [Case(rng, num_blocks=num_blocks, seg=int(sz), segments=1) for sz in sizes]
+    return offsets, page, pool, idx, page_host, page_dev, ids, cases
+
+
+@pytest.mark.parametrize("variant", ["aligned", "two_runs", "unaligned_slices"])
+def test_page_first_whole_page_packing(variant, xfer, stream):
+    """Page-first layers that tile contiguous pages go through staging as whole
+    pages (several staging units, slot reuse), byte-exact against the oracle;
+    AUTO picks that path, ZEROCOPY must give the same bytes."""
+    rng = np.random.default_rng(61)
+    sizes = {"aligned": [512, 1024, 1536, 4096], "two_runs": [4096, 2048, 1024],
+             "unaligned_slices": [1000, 520, 24, 3000]}[variant]
+    n = 1000  # x page bytes >= 4 MiB, the AUTO threshold for staging
+    gap = 400 if variant == "two_runs" else None
+    offsets, page, pool, idx, page_host, page_dev, ids, cases = _paged_setup(
+        rng, sizes, num_blocks=1024, n=n, page_gap_after=gap)
+    layers = []
+    for li, c in enumerate(cases):
+        c.dev.copy_from_host(c.cache0)
+        layers.append(LayerBlocks(layout=c.product_layout(), block_ids=ids, page_host=page_host,
+                                  page_host_device=page_dev, page_offset=int(offsets[li]),
+                                  page_len=page, layer_name=f"layer_{li}"))
+    opool = np.full(pool.size, SENT, dtype=np.uint8)
+    opages = (opool.ctypes.data + idx * page).astype(np.uint64)
+    for li, c in enumerate(cases):
+        oc = c.cache0.copy()  # keep the oracle's "device" image alive across the call
+        O.transfer_layer_paged(c.oracle_layout(oc), ids, opages, int(offsets[li]),
+                               host_is_src=False)
+    for path, expect_path in ((TransferPath.AUTO, ST), (ST, ST), (ZC, ZC)):
+        pool.as_numpy()[:] = SENT
+        xfer.save(layers, stream, path)
+        stream.synchronize()
+        assert xfer.last_path == expect_path
+        assert np.array_equal(pool.as_numpy(), opool), (variant, path)
+    dest = rng.choice(1024, n, replace=False).astype(np.uint32)
+    for path in (TransferPath.AUTO, ZC):
+        for li, c in enumerate(cases):
+            c.dev.fill(SENT)
+            layers[li].block_ids = dest
+        xfer.load(layers, stream, path)
+        stream.synchronize()
+        for li, c in enumerate(cases):
+            oc = np.full_like(c.cache0, SENT)
+            O.transfer_layer_paged(c.oracle_layout(oc), dest, opages, int(offsets[li]),
+                                   host_is_src=True)
+            assert np.array_equal(c.dev.copy_to_host(), oc), (variant, path, li)
+    for c in cases:
+        c.close()
+    pool.close()
+
+
+def test_page_packing_is_refused_when_it_would_touch_foreign_bytes(xfer, stream):
+    """A save that covers only part of each page must not drain whole pages
+    (the rest of the page belongs to someone else); a load of most of a page may
+    read the whole page."""
+    rng = np.random.default_rng(62)
+    sizes = [4096] * 10
+    n = 600
+    offsets, page, pool, idx, page_host, page_dev, ids, cases = _paged_setup(
+        rng, sizes, num_blocks=700, n=n)
+
+    def layers_for(which, block_ids):
+        out = []
+        for li in which:
+            out.append(LayerBlocks(layout=cases[li].product_layout(), block_ids=block_ids,
+                                   page_host=page_host, page_host_device=page_dev,
+                                   page_offset=int(offsets[li]), page_len=page,
+                                   layer_name=f"layer_{li}"))
+        return out
+
+    for c in cases:
+        c.dev.copy_from_host(c.cache0)
+    subset = [0, 1, 2, 3, 4, 6, 7, 8, 9]  # layer 5 is missing: a hole in every page
+    with pytest.raises(_lib.InvalidArgument, match="tile contiguous pages"):
+        xfer.save(layers_for(subset, ids), stream, ST)
+    xfer.save(layers_for(subset, ids), stream, TransferPath.AUTO)
+    stream.synchronize()
+    assert xfer.last_path == ZC
+    img = pool.as_numpy().reshape(n, page)
+    assert (img[:, 5 * 4096: 6 * 4096] == SENT).all(), "bytes of the missing layer were written"
+    # fill in layer 5 too, then load the 9-of-10 subset: packing allowed (reads only)
+    xfer.save(layers_for([5], ids), stream, TransferPath.AUTO)
+    stream.synchronize()
+    dest = rng.choice(700, n, replace=False).astype(np.uint32)
+    for c in cases:
+        c.dev.fill(SENT)
+    xfer.load(layers_for(subset, dest), stream, TransferPath.AUTO)
+    stream.synchronize()
+    assert xfer.last_path == ST
+    opages = (pool.host_ptr + idx * page).astype(np.uint64)
+    for li, c in enumerate(cases):
+        oc = np.full_like(c.cache0, SENT)
+        if li in subset:
+            O.transfer_layer_paged(c.oracle_layout(oc), dest, opages, int(offsets[li]),
+                                   host_is_src=True)
+        assert np.array_equal(c.dev.copy_to_host(), oc), li
+    for c in cases:
+        c.close()
+    pool.close()
