@@ -1,19 +1,22 @@
 #!/usr/bin/env python3
 """Benchmark of the layer-wise KV block transfer path on one MI355X.
 
-Workload (BASELINE.json configs[1] + configs[2], Llama-3.1-8B shape):
+Default workload (BASELINE.json configs[1] + configs[2], Llama-3.1-8B shape):
   32 layers, each a K/V-split paged cache [2, 8192 blocks, 16, 8, 128] bf16
   (N(0,1), seeded); 5,000 blocks (8 requests x 625, a seeded permutation of
   the pool) are SAVED layer by layer into the pinned host pool (gather,
   GPU -> host) and then LOADED into freshly permuted destination block ids of
   a second, zeroed cache (scatter, host -> GPU).
 
-One step = one save pass + one load pass = 2 x 10,485,760,000 payload bytes.
-`value` = payload bytes of K steps / wall time of K steps, device inputs and
-the host pool resident before the timed region.  Save and load rates, the
-measured contiguous-copy link peak, the gather kernel's HBM roofline, the
-GEMM-overlap run and the CPU baseline (oracle memcpy executor on host cores)
-are reported in the same JSON line.
+One step = one save pass + one load pass.  `value` = payload bytes of K steps /
+wall time of K steps, device inputs and the host pool resident before the
+timed region.  Save and load rates, the measured contiguous-copy link peak,
+the gather kernel's HBM roofline, the GEMM-overlap run and the CPU baseline
+(oracle memcpy executor on host cores) are reported in the same JSON line.
+
+`--workload llama70b_fp8` and `--workload dsv3_mla` run BASELINE configs[3]
+and configs[4] through the same harness (extra measurements; the driver's
+line is the default workload).
 """
 
 from __future__ import annotations
@@ -36,17 +39,30 @@ HBM_PEAK_GBPS = 8000.0      # MI355X published HBM3E bandwidth
 # copy of exactly 1 GiB reads on the same counters (x2.000 and x1.000).
 MEASURED_TRAFFIC_DEFAULT_STAGED = int((160191.7 * 2.000 + 320043.6 * 1.000) * 1024)
 
-LLAMA = dict(layers=32, num_blocks=8192, block_tokens=16, kv_heads=8, head_dim=128, elem=2,
-             n_save=5000)
+WORKLOADS = {
+    # BASELINE configs[1] (save) + configs[2] (load)
+    "llama8b": dict(label="configs[1]+configs[2]: Llama-3.1-8B KV [2,8192,16,8,128] bf16",
+                    layers=32, num_blocks=8192, seg=16 * 8 * 128 * 2, split=True, n=5000,
+                    dtype="bf16", ids="permutation", page_first=False),
+    # BASELINE configs[3]
+    "llama70b_fp8": dict(label="configs[3]: Llama-3-70B KV [2,16384,16,8,128] fp8 e4m3",
+                         layers=80, num_blocks=16384, seg=16 * 8 * 128, split=True, n=8192,
+                         dtype="fp8", ids="runs", page_first=False),
+    # BASELINE configs[4]
+    "dsv3_mla": dict(label="configs[4]: DeepSeek-V3 MLA latent [4096,64,576] bf16, page-first",
+                     layers=61, num_blocks=4096, seg=64 * 576 * 2, split=False, n=2048,
+                     dtype="bf16", ids="permutation", page_first=True),
+}
 
 
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="llama8b")
     ap.add_argument("--path", choices=["auto", "staged", "zerocopy"], default="auto")
-    ap.add_argument("--layers", type=int, default=LLAMA["layers"])
+    ap.add_argument("--layers", type=int, default=0, help="override the layer count")
     ap.add_argument("--slot-mb", type=int, default=0)
     ap.add_argument("--slots", type=int, default=0)
     ap.add_argument("--unroll", type=int, default=0)
@@ -56,6 +72,31 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--seed", type=int, default=0)
     return ap.parse_args()
+
+
+def make_ids(np, kind, num_blocks, n, seed):
+    """Block ids of a workload: a seeded permutation prefix, or (configs[3])
+    half in contiguous runs of length 8..64 and half isolated, runs and
+    singles interleaved in random order."""
+    rng = np.random.default_rng(seed)
+    if kind == "permutation":
+        return rng.permutation(num_blocks)[:n].astype(np.uint32)
+    taken = np.zeros(num_blocks, dtype=bool)
+    pieces = []
+    in_runs = 0
+    while in_runs < n // 2:
+        length = int(min(rng.integers(8, 65), n // 2 - in_runs))
+        start = int(rng.integers(0, num_blocks - length))
+        if taken[start:start + length].any():
+            continue
+        taken[start:start + length] = True
+        pieces.append(np.arange(start, start + length))
+        in_runs += length
+    free = np.flatnonzero(~taken)
+    singles = rng.choice(free, n - in_runs, replace=False)
+    pieces += [np.array([s]) for s in singles]
+    order = rng.permutation(len(pieces))
+    return np.concatenate([pieces[i] for i in order]).astype(np.uint32)
 
 
 def main():
@@ -70,6 +111,7 @@ def main():
 
     from pegaflow_amd import _lib, runtime
     from pegaflow_amd.layout import KVCacheLayout
+    from pegaflow_amd.pool import LayerTopology, WorkerLayers
     from pegaflow_amd.runtime import Event, PinnedMemory, Stream
     from pegaflow_amd.transfer import BlockTransfer, LayerBlocks, TransferPath
 
@@ -80,41 +122,76 @@ def main():
     path = {"auto": TransferPath.AUTO, "staged": TransferPath.STAGED,
             "zerocopy": TransferPath.ZEROCOPY}[args.path]
 
-    n_layers = args.layers
-    nb = LLAMA["num_blocks"]
-    seg = LLAMA["block_tokens"] * LLAMA["kv_heads"] * LLAMA["head_dim"] * LLAMA["elem"]  # 32768
-    n = LLAMA["n_save"]
-    layer_bytes = 2 * nb * seg
-    buf = n * seg                      # one host segment buffer (K or V) of one layer
-    payload_per_layer = 2 * buf
+    w = WORKLOADS[args.workload]
+    n_layers = args.layers or w["layers"]
+    nb, seg, n = w["num_blocks"], w["seg"], w["n"]
+    nseg = 2 if w["split"] else 1
+    layer_bytes = nseg * nb * seg
+    payload_per_layer = nseg * n * seg
     payload = payload_per_layer * n_layers
+    names = [f"model.layers.{li}.self_attn.attn" for li in range(n_layers)]
 
     # ---- inputs, resident before timing ----------------------------------
     gen = torch.Generator(device=dev)
     gen.manual_seed(args.seed)
-    shape = (2, nb, LLAMA["block_tokens"], LLAMA["kv_heads"], LLAMA["head_dim"])
-    src_cache = [torch.empty(shape, device=dev, dtype=torch.bfloat16).normal_(generator=gen)
-                 for _ in range(n_layers)]
-    dst_cache = [torch.zeros(shape, device=dev, dtype=torch.bfloat16) for _ in range(n_layers)]
-    rng = np.random.default_rng(args.seed)
-    save_ids = rng.permutation(nb)[:n].astype(np.uint32)      # 8 requests x 625 blocks
-    load_ids = np.random.default_rng(args.seed + 1).permutation(nb)[:n].astype(np.uint32)
+
+    def new_cache(fill):
+        if w["dtype"] == "bf16":
+            t = torch.empty(layer_bytes // 2, device=dev, dtype=torch.bfloat16)
+            if fill:
+                t.normal_(generator=gen)
+            else:
+                t.zero_()
+            return t
+        t = torch.zeros(layer_bytes, device=dev, dtype=torch.uint8)
+        if fill:  # random fp8 e4m3 bytes without the NaN encodings 0x7F / 0xFF
+            t.random_(0, 256, generator=gen)
+            t[(t & 0x7F) == 0x7F] -= 1
+        return t
+
+    src_cache = [new_cache(True) for _ in range(n_layers)]
+    dst_cache = [new_cache(False) for _ in range(n_layers)]
+    save_ids = make_ids(np, w["ids"], nb, n, args.seed)
+    load_ids = make_ids(np, "permutation", nb, n, args.seed + 1)
     t0 = time.time()
     pool = PinnedMemory(payload)
     pool_alloc_s = time.time() - t0
     torch.cuda.synchronize()
 
-    def layers_for(caches, ids):
-        out = []
-        for li, t in enumerate(caches):
-            layout = KVCacheLayout(t.data_ptr(), layer_bytes, nb, seg, nb * seg, 2)
-            off = li * payload_per_layer
-            out.append(LayerBlocks(
-                layout=layout, block_ids=ids,
-                host=(pool.host_ptr + off, pool.host_ptr + off + buf),
-                host_device=(pool.device_ptr + off, pool.device_ptr + off + buf),
-                host_len=(buf, buf), host_stride=seg, layer_name=f"model.layers.{li}.self_attn.attn"))
-        return out
+    def layouts_for(caches):
+        kv = nb * seg if w["split"] else 0
+        return [KVCacheLayout(t.data_ptr(), layer_bytes, nb, seg, kv, nseg) for t in caches]
+
+    if w["page_first"]:
+        # One page per saved block, layers at the offsets the sealed topology
+        # assigns (ids follow the byte-wise sorted layer names).
+        topo = LayerTopology([WorkerLayers(0, 0, dict(zip(names, layouts_for(src_cache))))],
+                             tp_size=1, page_first=True)
+        page = topo.shard_page_size(0)
+        assert page * n == payload
+        offsets = [topo.page_placement(topo.layer_id(nm))[0] for nm in names]
+        page_host = (pool.host_ptr + np.arange(n, dtype=np.uint64) * page).astype(np.uint64)
+        page_dev = (pool.device_ptr + np.arange(n, dtype=np.uint64) * page).astype(np.uint64)
+
+        def layers_for(caches, ids):
+            return [LayerBlocks(layout=L, block_ids=ids, page_host=page_host,
+                                page_host_device=page_dev, page_offset=offsets[li], page_len=page,
+                                layer_name=names[li])
+                    for li, L in enumerate(layouts_for(caches))]
+    else:
+        buf = n * seg  # one host segment buffer (K or V) of one layer
+
+        def layers_for(caches, ids):
+            out = []
+            for li, L in enumerate(layouts_for(caches)):
+                off = li * payload_per_layer
+                out.append(LayerBlocks(
+                    layout=L, block_ids=ids,
+                    host=tuple(pool.host_ptr + off + s * buf for s in range(nseg)),
+                    host_device=tuple(pool.device_ptr + off + s * buf for s in range(nseg)),
+                    host_len=tuple(buf for _ in range(nseg)), host_stride=seg,
+                    layer_name=names[li]))
+            return out
 
     save_layers = layers_for(src_cache, save_ids)
     load_layers = layers_for(dst_cache, load_ids)
@@ -138,11 +215,13 @@ def main():
     torch.cuda.synchronize()
     stream.synchronize()
     save_ms = load_ms = 0.0
+    step_times = []
     t_start = time.perf_counter()
     for _ in range(args.steps):
         s_ms, l_ms = one_step()
         save_ms += s_ms
         load_ms += l_ms
+        step_times.append((round(s_ms, 2), round(l_ms, 2)))
     stream.synchronize()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t_start
@@ -154,16 +233,20 @@ def main():
     load_gbps = payload * args.steps / (load_ms / 1e3) / 1e9
 
     # ---- byte-exactness of what was just timed (untimed) -------------------
-    pool_np = pool.as_numpy()
+    pool_t = torch.from_numpy(pool.as_numpy())
+    sid = torch.from_numpy(save_ids.astype(np.int64))
+    lid = torch.from_numpy(load_ids.astype(np.int64))
     for li in sorted({0, n_layers - 1}):
-        src = src_cache[li].view(torch.uint8).reshape(2, nb, seg)
-        img = torch.from_numpy(pool_np[li * payload_per_layer:(li + 1) * payload_per_layer]
-                               .reshape(2, n, seg))
-        want = src[:, torch.from_numpy(save_ids.astype(np.int64)).to(dev)].cpu()
+        src = src_cache[li].view(torch.uint8).reshape(nseg, nb, seg)
+        want = src[:, sid.to(dev)].cpu()                       # [nseg, n, seg]
+        if w["page_first"]:
+            img = pool_t.reshape(n, page)[:, offsets[li]:offsets[li] + seg].reshape(1, n, seg)
+        else:
+            img = pool_t[li * payload_per_layer:(li + 1) * payload_per_layer].reshape(nseg, n, seg)
         assert torch.equal(img, want), f"layer {li}: saved image differs from the device cache"
-        dst = dst_cache[li].view(torch.uint8).reshape(2, nb, seg).cpu()
+        dst = dst_cache[li].view(torch.uint8).reshape(nseg, nb, seg).cpu()
         expect = torch.zeros_like(dst)
-        expect[:, torch.from_numpy(load_ids.astype(np.int64))] = want
+        expect[:, lid] = want
         assert torch.equal(dst, expect), f"layer {li}: loaded cache differs"
 
     # ---- link peak: one large contiguous pinned <-> device copy -----------
@@ -185,14 +268,12 @@ def main():
     h2d_peak = time_copy(lambda: runtime.memcpy_h2d_async(scratch.data_ptr(), pool.host_ptr,
                                                           link_bytes, stream))
     # Restore what the link test overwrote in the pool.
-    xfer.save(save_layers[:max(1, (link_bytes + payload_per_layer - 1) // payload_per_layer)],
-              stream, path)
+    xfer.save(save_layers, stream, path)
     stream.synchronize()
 
     # ---- HBM copy ceiling with the same tile shape -------------------------
     scratch2 = torch.empty(link_bytes, device=dev, dtype=torch.uint8)
     lib = _lib.load()
-    unroll = args.unroll or 4
 
     def plain():
         # tile_unroll 0: the same one-tile-per-workgroup form as the staged kernels
@@ -200,7 +281,8 @@ def main():
                                      stream.handle))
     hbm_copy_gbps = 2 * time_copy(plain, reps=20)
 
-    # ---- roofline of the dominant kernel (separate, untimed pass) ---------
+    # ---- roofline of the dominant kernel (separate, untimed pass; in this pass
+    # the copies share the kernels' stream, so every timed launch runs alone) ---
     xfer.set_kernel_timing(True)
     xfer.save(save_layers, stream, path)
     stream.synchronize()
@@ -212,12 +294,12 @@ def main():
     launches = k_save_n + k_load_n
     avg_launch_ms = (k_save_ms + k_load_ms) / max(launches, 1)
     bytes_per_launch = 2 * payload / max(launches, 1)          # payload bytes one launch moves
+    default_shape = (args.workload == "llama8b" and not args.layers and not args.slot_mb)
     if used_path == "staged":
         # device gather/scatter: every payload byte is read once and written
         # once in HBM -> 2 x payload algorithmic bytes per launch
         alg_bytes = 2 * bytes_per_launch
         achieved = alg_bytes / (avg_launch_ms / 1e3) / 1e9
-        default_shape = (n_layers == LLAMA["layers"] and not args.slot_mb)
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                     "traffic": MEASURED_TRAFFIC_DEFAULT_STAGED if default_shape else None,
@@ -247,15 +329,15 @@ def main():
             "save_frac_of_theoretical": round(save_gbps / PCIE_GEN5_X16_GBPS, 4),
             "load_frac_of_theoretical": round(load_gbps / PCIE_GEN5_X16_GBPS, 4)}
 
-    # ---- compute overlap (configs[2]): load next to a GEMM stream ---------
+    # ---- compute overlap (configs[2]): transfers next to a GEMM stream ----
     overlap = None
     if not args.no_overlap:
-        overlap = run_overlap(torch, xfer, load_layers, stream, path, payload, n_layers)
+        overlap = run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_layers)
 
     # ---- CPU baseline: the oracle's memcpy executor on the host cores -----
     cpu = None
     if not args.no_cpu:
-        cpu = run_cpu_baseline(np, nb, seg, n, save_ids, load_ids, args.cpu_seconds, args.seed)
+        cpu = run_cpu_baseline(np, w, save_ids, load_ids, args.cpu_seconds, args.seed)
 
     result = {
         "metric": "KV save/load GB/s (GPU<->pinned host) & % of link peak, Llama-3.1-8B shape",
@@ -270,13 +352,14 @@ def main():
         "vs_baseline": None,
         "dtype": "u8",
         "data": "synthetic",
-        "config": {"workload": "configs[1]+configs[2]: Llama-3.1-8B KV [2,8192,16,8,128] bf16, "
-                               f"{n_layers} layers, 5000 blocks saved then loaded per step",
+        "config": {"workload": f"{w['label']}, {n_layers} layers, {n} blocks saved then loaded "
+                               "per step",
                    "layers": n_layers, "blocks": n, "fragment_bytes": seg,
                    "payload_bytes_per_direction": payload, "path": used_path,
-                   "staging_slot_mb": args.slot_mb or 512, "staging_slots": args.slots or 2,
-                   "tile_unroll": unroll},
+                   "host_layout": "page-first" if w["page_first"] else "layer-first",
+                   "staging_slot_mb": args.slot_mb or 512, "staging_slots": args.slots or 2},
         "save_gbps": round(save_gbps, 3),
+        "step_save_load_ms": step_times[:16],
         "load_gbps": round(load_gbps, 3),
         "roofline": roofline,
         "link": link,
@@ -288,8 +371,8 @@ def main():
     print(json.dumps(result))
 
 
-def run_overlap(torch, xfer, load_layers, stream, path, payload, n_layers):
-    """Load pass alone, GEMM stream alone, then both at once."""
+def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_layers):
+    """Transfer alone, GEMM stream alone, then both at once (load and save)."""
     from pegaflow_amd.runtime import Event
     dev = torch.device("cuda:0")
     m = 4096
@@ -314,39 +397,38 @@ def run_overlap(torch, xfer, load_layers, stream, path, payload, n_layers):
     gemms(200)
     torch.cuda.synchronize()
     gemm_alone_ms = g0.elapsed_time(g1) / 200
+    out = {"gemm": "4096x4096x4096 bf16, back to back on its own stream",
+           "gemm_alone_tflops": round(flop / (gemm_alone_ms / 1e3) / 1e12, 1)}
+    for name, fn, layers in (("load", xfer.load, load_layers), ("save", xfer.save, save_layers)):
+        e0.record(stream)
+        fn(layers, stream, path)
+        e1.record(stream)
+        e1.synchronize()
+        alone_ms = e0.elapsed_ms(e1)
+        count = max(50, int(alone_ms / gemm_alone_ms * 1.2))
+        if name == "load":
+            xfer.set_layer_events(layer_ev)
+        gemms(count)
+        e0.record(stream)
+        fn(layers, stream, path)
+        e1.record(stream)
+        e1.synchronize()
+        torch.cuda.synchronize()
+        xfer.set_layer_events(None)
+        both_ms = e0.elapsed_ms(e1)
+        out[f"gemm_with_{name}_tflops"] = round(flop / (g0.elapsed_time(g1) / count / 1e3) / 1e12, 1)
+        out[f"{name}_alone_gbps"] = round(payload / (alone_ms / 1e3) / 1e9, 2)
+        out[f"{name}_with_gemm_gbps"] = round(payload / (both_ms / 1e3) / 1e9, 2)
+        if name == "load":
+            done = [e0.elapsed_ms(le) for le in layer_ev]
+            per_layer = [done[0]] + [done[i] - done[i - 1] for i in range(1, len(done))]
+            out["per_layer_ms_mean"] = round(sum(per_layer) / len(per_layer), 3)
+            out["per_layer_ms_max"] = round(max(per_layer), 3)
+            out["first_layer_ready_ms"] = round(done[0], 3)
+    return out
 
-    e0.record(stream)
-    xfer.load(load_layers, stream, path)
-    e1.record(stream)
-    e1.synchronize()
-    load_alone_ms = e0.elapsed_ms(e1)
 
-    count = max(50, int(load_alone_ms / gemm_alone_ms * 1.2))
-    xfer.set_layer_events(layer_ev)
-    gemms(count)
-    e0.record(stream)
-    xfer.load(load_layers, stream, path)
-    e1.record(stream)
-    e1.synchronize()
-    torch.cuda.synchronize()
-    xfer.set_layer_events(None)
-    load_overlap_ms = e0.elapsed_ms(e1)
-    gemm_overlap_ms = g0.elapsed_time(g1) / count
-    done = [e0.elapsed_ms(le) for le in layer_ev]
-    per_layer = [done[0]] + [done[i] - done[i - 1] for i in range(1, len(done))]
-    return {
-        "gemm": "4096x4096x4096 bf16, back to back on its own stream",
-        "gemm_alone_tflops": round(flop / (gemm_alone_ms / 1e3) / 1e12, 1),
-        "gemm_with_load_tflops": round(flop / (gemm_overlap_ms / 1e3) / 1e12, 1),
-        "load_alone_gbps": round(payload / (load_alone_ms / 1e3) / 1e9, 2),
-        "load_with_gemm_gbps": round(payload / (load_overlap_ms / 1e3) / 1e9, 2),
-        "per_layer_ms_mean": round(sum(per_layer) / len(per_layer), 3),
-        "per_layer_ms_max": round(max(per_layer), 3),
-        "first_layer_ready_ms": round(done[0], 3),
-    }
-
-
-def run_cpu_baseline(np, nb, seg, n, save_ids, load_ids, seconds, seed):
+def run_cpu_baseline(np, w, save_ids, load_ids, seconds, seed):
     """Same workload shape, host cores only: one layer's cache resident in
     host memory, gathered into a host pool and scattered back with the
     oracle's memcpy-per-descriptor executor (a restatement of the reference's
@@ -354,13 +436,16 @@ def run_cpu_baseline(np, nb, seg, n, save_ids, load_ids, seconds, seed):
     Sample: repeated save+load of one layer until `seconds` elapse."""
     from oracle import oracle as O
     threads = min(16, os.cpu_count() or 1)
+    nb, seg, n = w["num_blocks"], w["seg"], w["n"]
+    nseg = 2 if w["split"] else 1
     rng = np.random.default_rng(seed)
-    cache = rng.integers(0, 256, size=2 * nb * seg, dtype=np.uint8)
+    cache = rng.integers(0, 256, size=nseg * nb * seg, dtype=np.uint8)
     dst = np.zeros_like(cache)
     host_k = np.zeros(n * seg, dtype=np.uint8)
-    host_v = np.zeros(n * seg, dtype=np.uint8)
-    src_layout = O.layout_over(cache, nb, seg, nb * seg, 2)
-    dst_layout = O.layout_over(dst, nb, seg, nb * seg, 2)
+    host_v = np.zeros(n * seg, dtype=np.uint8) if nseg == 2 else None
+    kv = nb * seg if nseg == 2 else 0
+    src_layout = O.layout_over(cache, nb, seg, kv, nseg)
+    dst_layout = O.layout_over(dst, nb, seg, kv, nseg)
 
     def once(t):
         O.transfer_layer(src_layout, save_ids, host_k, host_v, host_is_src=False, threads=t)
@@ -376,10 +461,10 @@ def run_cpu_baseline(np, nb, seg, n, save_ids, load_ids, seconds, seed):
             el = time.perf_counter() - t0
             if el >= budget:
                 break
-        out[label] = 2 * 2 * n * seg * reps / el / 1e9
+        out[label] = 2 * nseg * n * seg * reps / el / 1e9
     return {"value": round(out["all"], 2), "unit": "GB/s", "cores": threads, "kind": "port",
             "single_thread_gbps": round(out["one"], 2),
-            "sample": f"one layer [2,{nb},{seg}B] host-resident, {n} blocks saved+loaded "
+            "sample": f"one layer [{nseg},{nb},{seg}B] host-resident, {n} blocks saved+loaded "
                       f"repeatedly for ~{seconds:.0f}s (oracle memcpy executor)"}
 
 

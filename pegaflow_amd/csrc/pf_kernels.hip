@@ -161,7 +161,8 @@ __global__ __launch_bounds__(kLanes) void block_units_kernel(const BlockUnit* __
 // Block-ID gather / scatter, one small tile per workgroup (the HBM-bound form
 // used between the KV cache and a device staging buffer).
 //
-// grid = (tiles per fragment, list positions, 2 * units); a workgroup of LT
+// grid = (tiles per fragment, list positions, SEGS * units), SEGS being the
+// largest segment count among the units of the launch; a workgroup of LT
 // lanes moves LT*16 bytes with one 16-byte load per lane.  Measured on MI355X
 // against the alternatives at the Llama shape (5000 x 2 x 32 KiB per launch):
 // this form reaches ~6.3 TB/s (read+write), a 16 KiB-per-workgroup grid-stride
@@ -169,11 +170,11 @@ __global__ __launch_bounds__(kLanes) void block_units_kernel(const BlockUnit* __
 // keeps every SIMD full of waves, and the 3-D grid needs no division.
 // Remapping workgroups so that each XCD owns whole fragments changed nothing
 // (no data is reused, so there is no L2 locality to win).
-template <int LT, bool TO_FAR>
+template <int LT, bool TO_FAR, int SEGS>
 __global__ __launch_bounds__(LT) void block_tiles_kernel(const BlockUnit* __restrict__ units) {
   constexpr uint32_t kTile = LT * 16;
-  const BlockUnit* __restrict__ up = units + (blockIdx.z >> 1);
-  const uint32_t seg = blockIdx.z & 1u;
+  const BlockUnit* __restrict__ up = units + (SEGS == 2 ? blockIdx.z >> 1 : blockIdx.z);
+  const uint32_t seg = SEGS == 2 ? (blockIdx.z & 1u) : 0u;
   const uint32_t pos = blockIdx.y;
   const uint64_t frag_bytes = up->frag_bytes;
   const uint64_t off = static_cast<uint64_t>(blockIdx.x) * kTile;
@@ -297,8 +298,11 @@ int launch_block_units(const BlockUnit* units, uint32_t n_units, uint64_t max_ti
 }
 
 int launch_block_tiles(const BlockUnit* units, uint32_t n_units, uint32_t max_blocks,
-                       uint64_t max_frag_bytes, bool to_far, hipStream_t s) {
+                       uint64_t max_frag_bytes, uint32_t max_seg, bool to_far, hipStream_t s) {
   if (n_units == 0 || max_blocks == 0 || max_frag_bytes == 0) return PF_OK;
+  if (max_seg != 1 && max_seg != 2) {
+    return fail(PF_ERR_INVALID_ARGUMENT, "tile launch: %u segments per block", max_seg);
+  }
   constexpr uint64_t kTile = kTileLanes * 16;
   const uint64_t gx = (max_frag_bytes + kTile - 1) / kTile;
   if (n_units > kMaxTileUnits || max_blocks > kMaxTileBlocks || gx > 0x7FFFFFFFull) {
@@ -306,11 +310,19 @@ int launch_block_tiles(const BlockUnit* units, uint32_t n_units, uint32_t max_bl
                 "tile launch out of range: %u units, %u blocks, %llu-byte fragments", n_units,
                 max_blocks, static_cast<unsigned long long>(max_frag_bytes));
   }
-  dim3 grid(static_cast<uint32_t>(gx), max_blocks, 2 * n_units), block(kTileLanes, 1, 1);
-  if (to_far) {
-    hipLaunchKernelGGL((block_tiles_kernel<kTileLanes, true>), grid, block, 0, s, units);
+  dim3 grid(static_cast<uint32_t>(gx), max_blocks, max_seg * n_units), block(kTileLanes, 1, 1);
+  if (max_seg == 2) {
+    if (to_far) {
+      hipLaunchKernelGGL((block_tiles_kernel<kTileLanes, true, 2>), grid, block, 0, s, units);
+    } else {
+      hipLaunchKernelGGL((block_tiles_kernel<kTileLanes, false, 2>), grid, block, 0, s, units);
+    }
   } else {
-    hipLaunchKernelGGL((block_tiles_kernel<kTileLanes, false>), grid, block, 0, s, units);
+    if (to_far) {
+      hipLaunchKernelGGL((block_tiles_kernel<kTileLanes, true, 1>), grid, block, 0, s, units);
+    } else {
+      hipLaunchKernelGGL((block_tiles_kernel<kTileLanes, false, 1>), grid, block, 0, s, units);
+    }
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail_hip(e, "block_tiles_kernel launch");

@@ -50,9 +50,10 @@ constexpr uint32_t kMaxTileBlocks = 65535;
 constexpr uint32_t kMaxTileUnits = 32767;
 
 // Launch the one-tile-per-workgroup form over `n_units` units: the HBM-bound
-// kernel of the staged path.  Every unit needs n_blocks <= kMaxTileBlocks.
+// kernel of the staged path.  Every unit needs n_blocks <= kMaxTileBlocks;
+// max_seg (1 or 2) is the largest n_seg among the units.
 int launch_block_tiles(const BlockUnit* units, uint32_t n_units, uint32_t max_blocks,
-                       uint64_t max_frag_bytes, bool to_far, hipStream_t s);
+                       uint64_t max_frag_bytes, uint32_t max_seg, bool to_far, hipStream_t s);
 
 // Plain device copy kernel of the same tile shape, for calibrating counters
 // and measuring the HBM copy ceiling: copies `bytes` (multiple of 16).

@@ -102,7 +102,8 @@ int Xfer::launch_tiles(const BlockUnit* dev_unit, const BlockUnit& host_unit, bo
                        hipStream_t s) {
   int st = timing_begin(s);
   if (st != PF_OK) return st;
-  st = launch_block_tiles(dev_unit, 1, host_unit.n_blocks, host_unit.frag_bytes, to_far, s);
+  st = launch_block_tiles(dev_unit, 1, host_unit.n_blocks, host_unit.frag_bytes, host_unit.n_seg,
+                          to_far, s);
   if (st != PF_OK) return st;
   return timing_end(s);
 }
@@ -373,7 +374,7 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
       int rc = timing_begin(s);
       if (rc != PF_OK) return rc;
       rc = launch_block_tiles(units_dev + ci * n_plans, static_cast<uint32_t>(n_plans),
-                              static_cast<uint32_t>(c.count), max_frag, to_far, s);
+                              static_cast<uint32_t>(c.count), max_frag, 1, to_far, s);
       if (rc != PF_OK) return rc;
       return timing_end(s);
     };
