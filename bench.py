@@ -71,6 +71,8 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--settle-max", type=int, default=8,
+                    help="upper bound on the untimed passes run after the warmup until two agree")
     return ap.parse_args()
 
 
@@ -212,6 +214,17 @@ def main():
 
     for _ in range(args.warmup):
         one_step()
+    # A process that starts right after another one released tens of GiB of
+    # device and pinned memory sees the driver's clean-up of that memory as
+    # slower passes for a second or two.  Untimed passes until two in a row
+    # agree (bounded) keep that out of the timed steps; the count is reported.
+    settle_steps, prev = 0, None
+    while settle_steps < args.settle_max:
+        cur = sum(one_step())
+        settle_steps += 1
+        if prev is not None and abs(cur - prev) <= 0.015 * min(cur, prev):
+            break
+        prev = cur
     torch.cuda.synchronize()
     stream.synchronize()
     save_ms = load_ms = 0.0
@@ -334,6 +347,12 @@ def main():
     if not args.no_overlap:
         overlap = run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_layers)
 
+    # ---- both directions at once (the worker pool runs a load thread and a
+    # save thread per GPU: gpu_worker.rs:116-345 of the reference) ----------
+    duplex = None
+    if not args.no_overlap:
+        duplex = run_duplex(xfer, save_layers, load_layers, stream, path, payload, args)
+
     # ---- CPU baseline: the oracle's memcpy executor on the host cores -----
     cpu = None
     if not args.no_cpu:
@@ -360,11 +379,13 @@ def main():
                    "staging_slot_mb": args.slot_mb or 512, "staging_slots": args.slots or 2},
         "save_gbps": round(save_gbps, 3),
         "step_save_load_ms": step_times[:16],
+        "settle_steps": settle_steps,
         "load_gbps": round(load_gbps, 3),
         "roofline": roofline,
         "link": link,
         "cpu_baseline": cpu,
         "overlap": overlap,
+        "duplex": duplex,
         "pool_alloc_s": round(pool_alloc_s, 2),
         "device": runtime.device_name(0),
     }
@@ -428,6 +449,40 @@ def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_
     return out
 
 
+def run_duplex(xfer, save_layers, load_layers, stream, path, payload, args):
+    """A save and a load in flight together, each with its own stream and
+    staging slots, as the two worker threads of one GPU issue them.  (The
+    load reads the host image while the save rewrites it with the same bytes;
+    only the rates are used.)"""
+    from pegaflow_amd.runtime import Event, Stream
+    from pegaflow_amd.transfer import BlockTransfer
+    xfer2 = BlockTransfer(staging_slot_bytes=args.slot_mb << 20, staging_slots=args.slots,
+                          tile_unroll=args.unroll, zerocopy_max_workgroups=args.zc_max_wg)
+    stream2 = Stream()
+    ev = [Event(timing=True) for _ in range(4)]
+    xfer2.load(load_layers, stream2, path)   # allocate its staging
+    stream2.synchronize()
+    stream.synchronize()
+    best = None
+    for _ in range(2):
+        ev[0].record(stream)
+        ev[2].record(stream2)
+        xfer.save(save_layers, stream, path)
+        xfer2.load(load_layers, stream2, path)
+        ev[1].record(stream)
+        ev[3].record(stream2)
+        ev[1].synchronize()
+        ev[3].synchronize()
+        save_ms, load_ms = ev[0].elapsed_ms(ev[1]), ev[2].elapsed_ms(ev[3])
+        span_ms = max(ev[0].elapsed_ms(ev[1]), ev[0].elapsed_ms(ev[3]))
+        best = {"save_gbps": round(payload / save_ms / 1e6, 2),
+                "load_gbps": round(payload / load_ms / 1e6, 2),
+                "aggregate_gbps": round(2 * payload / span_ms / 1e6, 2)}
+    xfer2.close()
+    stream2.close()
+    return best
+
+
 def run_cpu_baseline(np, w, save_ids, load_ids, seconds, seed):
     """Same workload shape, host cores only: one layer's cache resident in
     host memory, gathered into a host pool and scattered back with the
@@ -462,8 +517,29 @@ def run_cpu_baseline(np, w, save_ids, load_ids, seconds, seed):
             if el >= budget:
                 break
         out[label] = 2 * nseg * n * seg * reps / el / 1e9
+    # configs[0] verbatim (Qwen3-0.6B: 28 layers [2,2048,32768 B], 64 blocks
+    # drawn per layer), gather into the pool then scatter back, all threads.
+    q_layers, q_nb, q_n = 28, 2048, 64
+    q_caches = [np.full(2 * q_nb * 32768, li + 1, dtype=np.uint8) for li in range(q_layers)]
+    q_ids = [rng.choice(q_nb, q_n, replace=False).astype(np.uint32) for _ in range(q_layers)]
+    q_layouts = [O.layout_over(c, q_nb, 32768, q_nb * 32768, 2) for c in q_caches]
+    q_k = np.zeros(q_n * 32768, dtype=np.uint8)
+    q_v = np.zeros(q_n * 32768, dtype=np.uint8)
+
+    def qwen_pass():
+        for lay, lid in zip(q_layouts, q_ids):
+            O.transfer_layer(lay, lid, q_k, q_v, host_is_src=False, threads=threads)
+            O.transfer_layer(lay, lid, q_k, q_v, host_is_src=True, threads=threads)
+
+    qwen_pass()
+    reps, t0 = 0, time.perf_counter()
+    while reps < 3 or time.perf_counter() - t0 < 1.0:
+        qwen_pass()
+        reps += 1
+    q_gbps = 2 * q_layers * 2 * q_n * 32768 * reps / (time.perf_counter() - t0) / 1e9
     return {"value": round(out["all"], 2), "unit": "GB/s", "cores": threads, "kind": "port",
             "single_thread_gbps": round(out["one"], 2),
+            "configs0_qwen3_0p6b_gbps": round(q_gbps, 2),
             "sample": f"one layer [{nseg},{nb},{seg}B] host-resident, {n} blocks saved+loaded "
                       f"repeatedly for ~{seconds:.0f}s (oracle memcpy executor)"}
 

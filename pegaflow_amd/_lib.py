@@ -7,7 +7,9 @@ Python or CPU fallback for anything that moves bytes.
 from __future__ import annotations
 
 import ctypes as C
+import importlib.util
 import os
+import sys
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpegahip.so")
@@ -280,6 +282,29 @@ class WorkerMissing(PegaHipError):
 _lib = None
 
 
+def _bind_to_pytorch_hip_runtime() -> None:
+    """PyTorch's ROCm wheels carry their own libamdhip64 (same SONAME as the
+    system one).  Two HIP runtimes in one process do not both get the GPU, and
+    which one a process ends up with would depend on import order.  When such
+    a wheel is installed and PyTorch is not loaded yet, load its runtime first
+    so that libpegahip binds to the copy PyTorch will use.  Set
+    PEGAHIP_SYSTEM_HIP_RUNTIME=1 to keep the system runtime instead."""
+    if "torch" in sys.modules or os.environ.get("PEGAHIP_SYSTEM_HIP_RUNTIME") == "1":
+        return
+    try:
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        return
+    if spec is None or not spec.submodule_search_locations:
+        return
+    bundled = os.path.join(list(spec.submodule_search_locations)[0], "lib", "libamdhip64.so")
+    if os.path.exists(bundled):
+        try:
+            C.CDLL(bundled, mode=C.RTLD_GLOBAL)
+        except OSError:
+            pass
+
+
 def load():
     """Load libpegahip.so and set every prototype.  Raises if it is absent."""
     global _lib
@@ -290,6 +315,7 @@ def load():
             f"{LIB_PATH} is missing: build it with `make -C pegaflow_amd/csrc` "
             "(or `python -c 'import __graft_entry__ as g; g.build()'`). "
             "pegaflow_amd has no fallback path.")
+    _bind_to_pytorch_hip_runtime()
     lib = C.CDLL(LIB_PATH)
     for name, (restype, argtypes) in PROTOTYPES.items():
         fn = getattr(lib, name)
