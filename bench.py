@@ -33,11 +33,15 @@ if ROOT not in sys.path:
 
 PCIE_GEN5_X16_GBPS = 63.0   # 32 GT/s x 16 lanes x 128/130 / 8
 HBM_PEAK_GBPS = 8000.0      # MI355X published HBM3E bandwidth
-# HBM bytes one staged gather/scatter launch moves at the default workload
-# (5000 blocks x 2 x 32 KiB), from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
-# of this script: 160191.7 and 320043.6 KiB per dispatch, scaled by what a plain
-# copy of exactly 1 GiB reads on the same counters (x2.000 and x1.000).
-MEASURED_TRAFFIC_DEFAULT_STAGED = int((160191.7 * 2.000 + 320043.6 * 1.000) * 1024)
+# HBM bytes one staged gather/scatter launch moves (mean over the launches of a
+# step) at each workload's default shape, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this script: KiB per dispatch, scaled by what a plain copy
+# of exactly 1 GiB reads on the same counters (x2.000 and x1.000).
+MEASURED_TRAFFIC_STAGED = {
+    "llama8b": int((160184.2 * 2.000 + 320034.9 * 1.000) * 1024),
+    "llama70b_fp8": int((131358.9 * 2.000 + 262171.2 * 1.000) * 1024),
+    "dsv3_mla": int((249956.5 * 2.000 + 499880.8 * 1.000) * 1024),
+}
 
 WORKLOADS = {
     # BASELINE configs[1] (save) + configs[2] (load)
@@ -307,7 +311,7 @@ def main():
     launches = k_save_n + k_load_n
     avg_launch_ms = (k_save_ms + k_load_ms) / max(launches, 1)
     bytes_per_launch = 2 * payload / max(launches, 1)          # payload bytes one launch moves
-    default_shape = (args.workload == "llama8b" and not args.layers and not args.slot_mb)
+    default_shape = not args.layers and not args.slot_mb
     if used_path == "staged":
         # device gather/scatter: every payload byte is read once and written
         # once in HBM -> 2 x payload algorithmic bytes per launch
@@ -315,7 +319,7 @@ def main():
         achieved = alg_bytes / (avg_launch_ms / 1e3) / 1e9
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                    "traffic": MEASURED_TRAFFIC_DEFAULT_STAGED if default_shape else None,
+                    "traffic": MEASURED_TRAFFIC_STAGED[args.workload] if default_shape else None,
                     "kernel": "block_tiles_kernel (staged gather/scatter)",
                     "launches": launches, "avg_launch_us": round(avg_launch_ms * 1e3, 2),
                     "alg_bytes_per_launch": int(alg_bytes),
