@@ -30,6 +30,18 @@ typedef __attribute__((address_space(4))) const uint64_t c_u64;
 
 constexpr int kLanes = 256;
 
+// 16-byte global stores with an explicit cache policy.  Measured on MI355X at
+// the Llama shape (5000 x 2 x 32 KiB gathered or scattered per launch), all 49
+// load x store policy pairs: a dense destination is written fastest with
+// "sc1 nt" (6.35 TB/s against 6.30 for plain nt), a destination scattered over
+// the cache with "sc1" and no nt (6.13 TB/s against 5.72 for nt).
+__device__ __forceinline__ void store16_sc1_nt(uint64_t dst, u32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(dst), "v"(v) : "memory");
+}
+__device__ __forceinline__ void store16_sc1(uint64_t dst, u32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst), "v"(v) : "memory");
+}
+
 // Copy `bytes` <= U*4096 from src to dst; both 16-byte aligned.
 template <int U>
 __device__ __forceinline__ void copy_tile_vec(uint64_t dst, uint64_t src, uint32_t bytes) {
@@ -198,11 +210,18 @@ __global__ __launch_bounds__(LT) void block_tiles_kernel(const BlockUnit* __rest
   const uint32_t lane = threadIdx.x;
   if (up->vec_ok) {
     const g_u32x4* __restrict__ s = reinterpret_cast<const g_u32x4*>(src);
-    g_u32x4* __restrict__ d = reinterpret_cast<g_u32x4*>(dst);
     const uint32_t nvec = bytes >> 4;
     if (lane < nvec) {
-      const u32x4 v = __builtin_nontemporal_load(s + lane);
-      __builtin_nontemporal_store(v, d + lane);
+      // Gather: ordinary load of the scattered source, streaming store to the
+      // dense staging side.  Scatter: streaming load of the dense side,
+      // cached-scope store to the scattered destination.
+      if (TO_FAR) {
+        const u32x4 v = s[lane];
+        store16_sc1_nt(dst + lane * 16ull, v);
+      } else {
+        const u32x4 v = __builtin_nontemporal_load(s + lane);
+        store16_sc1(dst + lane * 16ull, v);
+      }
     }
     const uint32_t j = (nvec << 4) + lane;
     if (j < bytes) reinterpret_cast<g_u8*>(dst)[j] = reinterpret_cast<const g_u8*>(src)[j];
