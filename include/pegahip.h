@@ -532,6 +532,15 @@ int pf_engine_unregister_instance(pf_engine_t e, const char* instance_id);
 int pf_engine_batch_save(pf_engine_t e, const char* instance_id, uint64_t tp_rank,
                          uint64_t pp_rank, int device_id, const pf_layer_save* saves,
                          uint64_t n_saves);
+/* Where the time of the last successful save went; the reference records the
+ * same phases as metrics (offload.rs:560-574).  assemble_ms (building the
+ * blocks that enter the store) runs while the copy is in flight, inside
+ * transfer_ms. */
+typedef struct pf_save_profile {
+  double validate_ms, filter_ms, alloc_ms, assemble_ms, transfer_ms, publish_ms, total_ms;
+  uint64_t bytes;
+} pf_save_profile;
+int pf_engine_last_save_profile(pf_engine_t e, pf_save_profile* out);
 /* Longest cached prefix of the hashes and a lease over those blocks (0 = none). */
 int pf_engine_query_prefix(pf_engine_t e, const char* instance_id,
                            const uint8_t* const* hashes, const uint32_t* hash_lens, uint64_t n,

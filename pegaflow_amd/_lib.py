@@ -128,6 +128,12 @@ class PfLayerSave(C.Structure):
                 ("block_hash_lens", C.POINTER(u32)), ("n_blocks", u64)]
 
 
+class PfSaveProfile(C.Structure):
+    _fields_ = [("validate_ms", C.c_double), ("filter_ms", C.c_double), ("alloc_ms", C.c_double),
+                ("assemble_ms", C.c_double), ("transfer_ms", C.c_double),
+                ("publish_ms", C.c_double), ("total_ms", C.c_double), ("bytes", u64)]
+
+
 # name -> (restype, argtypes).  Every symbol include/pegahip.h declares.
 PROTOTYPES = {
     "pf_last_error": (C.c_char_p, []),
@@ -248,6 +254,7 @@ PROTOTYPES = {
                                        C.POINTER(C.POINTER(C.c_char_p)), C.POINTER(u64), u64,
                                        C.POINTER(C.POINTER(C.c_int64)), u64, C.c_char_p,
                                        C.POINTER(vp)]),
+    "pf_engine_last_save_profile": (C.c_int, [vp, C.POINTER(PfSaveProfile)]),
     "pf_engine_pool_usage": (C.c_int, [vp, C.POINTER(u64), C.POINTER(u64)]),
     "pf_engine_cached_blocks": (u64, [vp]),
     "pf_engine_evict_all": (u64, [vp]),

@@ -54,31 +54,52 @@ class Segment {
   std::shared_ptr<PinnedAllocation> allocation_;
 };
 
-// block.rs:90-199: an ordered list of segments, layout-agnostic.
+// block.rs:90-199: an ordered list of segments, layout-agnostic.  One or two
+// segments (every layout on the path) live inline; more spill to the heap.
 class RawBlock {
  public:
   RawBlock() = default;
-  explicit RawBlock(std::vector<Segment> segments) : segments_(std::move(segments)) {
-    for (const auto& s : segments_) total_size_ += s.size();
+  explicit RawBlock(std::vector<Segment> segments) {
+    n_ = segments.size();
+    for (size_t i = 0; i < segments.size(); ++i) {
+      total_size_ += segments[i].size();
+      if (i < 2) {
+        inline_[i] = std::move(segments[i]);
+      } else {
+        extra_.push_back(std::move(segments[i]));
+      }
+    }
   }
-  static RawBlock single_segment(Segment s) { return RawBlock(std::vector<Segment>{std::move(s)}); }
+  static RawBlock single_segment(Segment s) {
+    RawBlock b;
+    b.n_ = 1;
+    b.total_size_ = s.size();
+    b.inline_[0] = std::move(s);
+    return b;
+  }
   static RawBlock two_segments(Segment k, Segment v) {
-    return RawBlock(std::vector<Segment>{std::move(k), std::move(v)});
+    RawBlock b;
+    b.n_ = 2;
+    b.total_size_ = k.size() + v.size();
+    b.inline_[0] = std::move(k);
+    b.inline_[1] = std::move(v);
+    return b;
   }
-  size_t num_segments() const { return segments_.size(); }
+  size_t num_segments() const { return n_; }
   bool segment_mapped_ptr(size_t i, MappedPinnedPtr* out) const {
-    if (i >= segments_.size()) return false;
-    *out = segments_[i].ptr();
+    if (i >= n_) return false;
+    *out = at(i).ptr();
     return true;
   }
-  uint64_t segment_allocation_id(size_t i) const {
-    return i < segments_.size() ? segments_[i].allocation_id() : 0;
-  }
-  uint64_t segment_size(size_t i) const { return i < segments_.size() ? segments_[i].size() : 0; }
+  uint64_t segment_allocation_id(size_t i) const { return i < n_ ? at(i).allocation_id() : 0; }
+  uint64_t segment_size(size_t i) const { return i < n_ ? at(i).size() : 0; }
   uint64_t memory_footprint() const { return total_size_; }
 
  private:
-  std::vector<Segment> segments_;
+  const Segment& at(size_t i) const { return i < 2 ? inline_[i] : extra_[i - 2]; }
+  Segment inline_[2];
+  std::vector<Segment> extra_;
+  size_t n_ = 0;
   uint64_t total_size_ = 0;
 };
 
@@ -114,7 +135,21 @@ class InflightBlock {
   }
   size_t total_slots() const { return slots_.size(); }
   size_t filled_count() const { return slots_.size() - remaining_; }
+  bool complete() const { return remaining_ == 0; }
   std::shared_ptr<SealedBlock> seal() { return std::make_shared<SealedBlock>(std::move(slots_)); }
+  // Move every filled slot of `other` into this block (slots already filled
+  // here are kept: a repeated slot is a duplicate, as in insert_slot).
+  Insert absorb(InflightBlock&& other) {
+    Insert last = Insert::Duplicate;
+    const size_t n = other.slots_.size() < slots_.size() ? other.slots_.size() : slots_.size();
+    for (size_t i = 0; i < n; ++i) {
+      if (!other.filled_[i]) continue;
+      Insert r = insert_slot(i, std::move(other.slots_[i]));
+      if (r == Insert::Completed) return r;
+      if (r == Insert::Inserted) last = r;
+    }
+    return last;
+  }
 
  private:
   std::vector<RawBlock> slots_;

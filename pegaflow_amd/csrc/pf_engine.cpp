@@ -1,6 +1,8 @@
 #include "pf_engine.hpp"
 
 #include <algorithm>
+#include <chrono>
+#include <cstring>
 #include <set>
 
 #include "pf_common.hpp"
@@ -20,13 +22,56 @@ int bad(std::string* err, int code, std::string msg) {
 }  // namespace
 
 // Per-layer state of one save (offload.rs:52-66).
+// One distinct (group, hash sequence) of a save call; layers that carry the
+// same one share it.
+struct SaveList {
+  uint32_t group = 0;
+  const uint8_t* const* hashes = nullptr;
+  const uint32_t* lens = nullptr;
+  size_t n = 0;
+  std::vector<BlockKey> keys;  // group-encoded key of each position
+  std::vector<uint32_t> kept;  // positions not in the store yet, ascending
+  bool same_as(uint32_t g, const LayerSaveView& s) const {
+    if (g != group || s.n_hashes != n) return false;
+    if (s.hashes == hashes && s.hash_lens == lens) return true;
+    for (size_t i = 0; i < n; ++i) {
+      if (s.hash_lens[i] != lens[i]) return false;
+      if (s.hashes[i] != hashes[i] && std::memcmp(s.hashes[i], hashes[i], lens[i]) != 0) {
+        return false;
+      }
+    }
+    return true;
+  }
+};
+
 struct SaveLayerCtx {
   std::string layer_name;
   KVCacheLayout layout;
   size_t slot_id = 0;
   uint32_t group = 0;
-  std::vector<std::pair<uint64_t, std::string>> blocks_to_save;  // (block_idx, raw hash)
-  std::vector<std::shared_ptr<RawBlock>> raw_blocks;             // parallel to blocks_to_save
+  const uint64_t* block_ids = nullptr;         // the caller's list, all positions
+  size_t list = 0;                             // index of its SaveList
+  std::shared_ptr<std::vector<uint32_t>> ids;  // device block of each kept position
+  uint64_t stride = 0;                         // host stride of one position
+  // Batch image: one K (and V) allocation; blockwise: one per kept position.
+  std::vector<std::shared_ptr<PinnedAllocation>> k_allocs, v_allocs;
+  std::vector<RawBlock> raw_blocks;            // blockwise only: handles the task points at
+
+  // The host image of kept position q as a block of its own (offload.rs:454-509).
+  bool make_raw(size_t q, bool blockwise, RawBlock* out) const {
+    const size_t a = blockwise ? q : 0;
+    const uint64_t off = blockwise ? 0 : q * stride;
+    Segment k;
+    if (!Segment::create(k_allocs[a]->as_ptr() + off, stride, k_allocs[a], &k)) return false;
+    if (v_allocs.empty()) {
+      *out = RawBlock::single_segment(std::move(k));
+      return true;
+    }
+    Segment v;
+    if (!Segment::create(v_allocs[a]->as_ptr() + off, stride, v_allocs[a], &v)) return false;
+    *out = RawBlock::two_segments(std::move(k), std::move(v));
+    return true;
+  }
 };
 
 // ---------------------------------------------------------------------------
@@ -313,7 +358,7 @@ int Engine::alloc_page_first_targets(const LayerTopology& topo, SaveLayerCtx* ct
   const size_t shard = ctxs[0].slot_id;
   size_t page_size = 0;
   topo.shard_page_size(shard, &page_size);
-  const auto& reference = ctxs[0].blocks_to_save;
+  const SaveLayerCtx& first = ctxs[0];
   std::set<size_t> layer_ids;
   for (size_t i = 0; i < n; ++i) {
     if (ctxs[i].layout.is_split()) {
@@ -324,7 +369,8 @@ int Engine::alloc_page_first_targets(const LayerTopology& topo, SaveLayerCtx* ct
       return bad(err, PF_ERR_INVALID_ARGUMENT,
                  "page-first save spans multiple shards (one writer must save one shard)");
     }
-    if (ctxs[i].blocks_to_save != reference) {
+    // Same hashes (same list) and same block ids, position by position.
+    if (ctxs[i].list != first.list || *ctxs[i].ids != *first.ids) {
       return bad(err, PF_ERR_INVALID_ARGUMENT,
                  "page-first save requires the same block set across all layers");
     }
@@ -345,39 +391,52 @@ int Engine::alloc_page_first_targets(const LayerTopology& topo, SaveLayerCtx* ct
                    " distinct (one worker must write a shard's entire page)");
   }
   if (page_size == 0) return bad(err, PF_ERR_STORAGE, "page size is zero");
-  for (size_t b = 0; b < reference.size(); ++b) {
+  const size_t num = first.ids->size();
+  auto page_ptrs = std::make_shared<std::vector<MappedPinnedPtr>>();
+  auto page_ids = std::make_shared<std::vector<uint64_t>>();
+  page_ptrs->reserve(num);
+  page_ids->reserve(num);
+  for (size_t b = 0; b < num; ++b) {
     auto page = allocate(page_size, numa);
     if (!page) return bad(err, PF_ERR_STORAGE, "pinned pool exhausted while allocating page");
+    MappedPinnedPtr p;
+    if (!page->mapped_ptr_for_host_range(page->as_ptr(), page_size, &p)) {
+      return bad(err, PF_ERR_STORAGE, "page exceeds its pinned allocation");
+    }
+    page_ptrs->push_back(p);
+    page_ids->push_back(page->allocation_id());
     pages->push_back(std::move(page));
   }
   for (size_t i = 0; i < n; ++i) {
     size_t id = 0, offset = 0, layer_bytes = 0;
     topo.layer_id(ctxs[i].layer_name, &id, nullptr);
     topo.page_placement(id, &offset, &layer_bytes);
+    if (offset + layer_bytes > page_size) {
+      return bad(err, PF_ERR_STORAGE, "page slice exceeds its pinned allocation");
+    }
     LayerTransferData ltd;
     ltd.layer_name = ctxs[i].layer_name;
     ltd.layout = ctxs[i].layout;
-    for (size_t b = 0; b < reference.size(); ++b) {
-      Segment seg;
-      const auto& page = (*pages)[b];
-      if (!Segment::create(page->as_ptr() + offset, layer_bytes, page, &seg)) {
-        return bad(err, PF_ERR_STORAGE, "page slice exceeds its pinned allocation");
-      }
-      auto raw = std::make_shared<RawBlock>(RawBlock::single_segment(std::move(seg)));
-      TransferBlock tb;
-      tb.block_idx = reference[b].first;
-      tb.block.raw = raw.get();
-      tb.block.keep = raw;
-      ltd.blocks.push_back(std::move(tb));
-    }
+    ltd.image.kind = HostImage::Kind::Paged;
+    ltd.image.block_ids = ctxs[i].ids;
+    ltd.image.pages = page_ptrs;
+    ltd.image.page_allocation_ids = page_ids;
+    ltd.image.offset = offset;
+    ltd.image.page_len = page_size;
     out->push_back(std::move(ltd));
   }
   return PF_OK;
 }
 
 int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank, size_t pp_rank,
-                                 int device_id, const std::vector<LayerSave>& saves,
+                                 int device_id, const std::vector<LayerSaveView>& saves,
                                  std::string* err) {
+  using Clock = std::chrono::steady_clock;
+  const auto t_begin = Clock::now();
+  auto ms_since = [](Clock::time_point t) {
+    return std::chrono::duration<double, std::milli>(Clock::now() - t).count();
+  };
+  SaveProfile prof;
   auto instance = get_instance(instance_id, err);
   if (!instance) return PF_ERR_INSTANCE_MISSING;
   auto topo = instance->sealed_topology(err);
@@ -397,70 +456,101 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
                    std::to_string(gpu->reg.pp_rank) + ", but save requested tp_rank " +
                    std::to_string(tp_rank) + ", pp_rank " + std::to_string(pp_rank));
   }
+  // Layers that carry the same hash sequence for the same group (the usual
+  // case: one request's blocks saved for every layer) share one SaveList, so
+  // the store is consulted once per block, not once per (layer, block).
+  std::vector<SaveList> lists;
   std::vector<SaveLayerCtx> ctxs;
-  std::set<std::pair<uint32_t, std::string>> hashes_to_save;
-  for (const LayerSave& s : saves) {
-    if (s.block_ids.size() != s.block_hashes.size()) {
+  for (const LayerSaveView& s : saves) {
+    const std::string layer_name = s.layer_name ? s.layer_name : "";
+    if (s.n_ids != s.n_hashes) {
       return bad(err, PF_ERR_INVALID_ARGUMENT,
-                 "block_ids length " + std::to_string(s.block_ids.size()) +
-                     " does not match block_hashes " + std::to_string(s.block_hashes.size()) +
-                     " for layer " + s.layer_name);
+                 "block_ids length " + std::to_string(s.n_ids) + " does not match block_hashes " +
+                     std::to_string(s.n_hashes) + " for layer " + layer_name);
     }
     size_t layer_id = 0;
     std::string cause;
-    if (!topo->layer_id(s.layer_name, &layer_id, &cause)) {
+    if (!topo->layer_id(layer_name, &layer_id, &cause)) {
       return bad(err, PF_ERR_INVALID_ARGUMENT, cause);
     }
-    auto lit = gpu->reg.kv_caches.find(s.layer_name);
+    auto lit = gpu->reg.kv_caches.find(layer_name);
     if (lit == gpu->reg.kv_caches.end()) {
-      return bad(err, PF_ERR_INVALID_ARGUMENT,
-                 "layer " + s.layer_name + " not registered on device");
+      return bad(err, PF_ERR_INVALID_ARGUMENT, "layer " + layer_name + " not registered on device");
     }
     SaveLayerCtx ctx;
-    ctx.layer_name = s.layer_name;
+    ctx.layer_name = layer_name;
     ctx.layout = lit->second;
     if (!topo->slot_index(layer_id, tp_rank, &ctx.slot_id, &cause)) {
       return bad(err, PF_ERR_INVALID_ARGUMENT, cause);
     }
     ctx.group = topo->group_of_layer(layer_id);
     const uint64_t nb = ctx.layout.num_blocks();
-    for (size_t i = 0; i < s.block_ids.size(); ++i) {
+    for (size_t i = 0; i < s.n_ids; ++i) {
       if (s.block_ids[i] >= nb) {
         return bad(err, PF_ERR_INVALID_ARGUMENT,
                    "block_id " + std::to_string(s.block_ids[i]) + " out of range (num_blocks=" +
-                       std::to_string(nb) + ") for layer " + s.layer_name);
+                       std::to_string(nb) + ") for layer " + layer_name);
       }
-      ctx.blocks_to_save.emplace_back(s.block_ids[i], s.block_hashes[i]);
     }
-    if (ctx.blocks_to_save.empty()) continue;
-    for (auto& b : ctx.blocks_to_save) hashes_to_save.emplace(ctx.group, b.second);
+    if (s.n_ids == 0) continue;
+    ctx.block_ids = s.block_ids;
+    size_t li = lists.size();
+    for (size_t k = lists.size(); k-- > 0;) {
+      if (lists[k].same_as(ctx.group, s)) {
+        li = k;
+        break;
+      }
+    }
+    if (li == lists.size()) {
+      SaveList l;
+      l.group = ctx.group;
+      l.hashes = s.hashes;
+      l.lens = s.hash_lens;
+      l.n = s.n_hashes;
+      lists.push_back(std::move(l));
+    }
+    ctx.list = li;
     ctxs.push_back(std::move(ctx));
   }
   if (ctxs.empty()) return PF_OK;
+  prof.validate_ms = ms_since(t_begin);
 
   // ---- Phase 1: drop hashes whose group-encoded key is already cached -----
+  auto t_phase = Clock::now();
+  size_t to_save = 0;
   {
+    for (SaveList& l : lists) {
+      l.keys.reserve(l.n);
+      for (size_t i = 0; i < l.n; ++i) {
+        l.keys.push_back(BlockKey{
+            ns, group_hash(std::string(reinterpret_cast<const char*>(l.hashes[i]), l.lens[i]),
+                           l.group)});
+      }
+    }
     std::lock_guard<std::mutex> lock(mu_);
-    for (auto it = hashes_to_save.begin(); it != hashes_to_save.end();) {
-      BlockKey key{ns, group_hash(it->second, it->first)};
-      it = sealed_.count(key) ? hashes_to_save.erase(it) : std::next(it);
+    for (SaveList& l : lists) {
+      for (size_t i = 0; i < l.n; ++i) {
+        if (!sealed_.count(l.keys[i])) l.kept.push_back(static_cast<uint32_t>(i));
+      }
+      to_save += l.kept.size();
     }
   }
-  if (hashes_to_save.empty()) return PF_OK;
-  for (auto& ctx : ctxs) {
-    auto& v = ctx.blocks_to_save;
-    v.erase(std::remove_if(v.begin(), v.end(),
-                           [&](const std::pair<uint64_t, std::string>& b) {
-                             return !hashes_to_save.count({ctx.group, b.second});
-                           }),
-            v.end());
-  }
+  if (to_save == 0) return PF_OK;
   ctxs.erase(std::remove_if(ctxs.begin(), ctxs.end(),
-                            [](const SaveLayerCtx& c) { return c.blocks_to_save.empty(); }),
+                            [&](const SaveLayerCtx& c) { return lists[c.list].kept.empty(); }),
              ctxs.end());
   if (ctxs.empty()) return PF_OK;
+  for (SaveLayerCtx& ctx : ctxs) {
+    const SaveList& l = lists[ctx.list];
+    auto ids = std::make_shared<std::vector<uint32_t>>();
+    ids->reserve(l.kept.size());
+    for (uint32_t pos : l.kept) ids->push_back(static_cast<uint32_t>(ctx.block_ids[pos]));
+    ctx.ids = std::move(ids);
+  }
+  prof.filter_ms = ms_since(t_phase);
 
   // ---- Phase 2: pinned allocation + host images ----------------------------
+  t_phase = Clock::now();
   const NumaNode numa = gpu->preferred_numa;
   const bool page_first = topo->is_page_first();
   std::vector<LayerTransferData> gpu_layers;
@@ -472,7 +562,7 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
   } else {
     for (auto& ctx : ctxs) {
       const KVCacheLayout& layout = ctx.layout;
-      const size_t num = ctx.blocks_to_save.size();
+      const size_t num = ctx.ids->size();
       const size_t alloc_count = cfg_.blockwise_alloc ? num : 1;
       const size_t per_alloc = cfg_.blockwise_alloc ? 1 : num;
       auto alloc_pinned = [&](uint64_t stride, const char* what,
@@ -488,91 +578,169 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
         }
         return PF_OK;
       };
+      const bool split = layout.is_split();
+      ctx.stride = split ? layout.padded_segment_bytes() : layout.padded_block_bytes();
       for (size_t a = 0; a < alloc_count; ++a) {
-        if (layout.is_split()) {
-          const uint64_t stride = layout.padded_segment_bytes();
-          std::shared_ptr<PinnedAllocation> k_alloc, v_alloc;
-          int st = alloc_pinned(stride, "K segment buffer", &k_alloc);
-          if (st == PF_OK) st = alloc_pinned(stride, "V segment buffer", &v_alloc);
-          if (st != PF_OK) return st;
-          for (size_t i = 0; i < per_alloc; ++i) {
-            Segment k, v;
-            if (!Segment::create(k_alloc->as_ptr() + i * stride, stride, k_alloc, &k) ||
-                !Segment::create(v_alloc->as_ptr() + i * stride, stride, v_alloc, &v)) {
-              return bad(err, PF_ERR_STORAGE, "segment exceeds its pinned allocation");
-            }
-            ctx.raw_blocks.push_back(
-                std::make_shared<RawBlock>(RawBlock::two_segments(std::move(k), std::move(v))));
-          }
-        } else {
-          const uint64_t stride = layout.padded_block_bytes();
-          std::shared_ptr<PinnedAllocation> alloc;
-          int st = alloc_pinned(stride, "block buffer", &alloc);
-          if (st != PF_OK) return st;
-          for (size_t i = 0; i < per_alloc; ++i) {
-            Segment s;
-            if (!Segment::create(alloc->as_ptr() + i * stride, stride, alloc, &s)) {
-              return bad(err, PF_ERR_STORAGE, "segment exceeds its pinned allocation");
-            }
-            ctx.raw_blocks.push_back(
-                std::make_shared<RawBlock>(RawBlock::single_segment(std::move(s))));
-          }
-        }
+        std::shared_ptr<PinnedAllocation> k_alloc, v_alloc;
+        int st = alloc_pinned(ctx.stride, split ? "K segment buffer" : "block buffer", &k_alloc);
+        if (st == PF_OK && split) st = alloc_pinned(ctx.stride, "V segment buffer", &v_alloc);
+        if (st != PF_OK) return st;
+        ctx.k_allocs.push_back(std::move(k_alloc));
+        if (split) ctx.v_allocs.push_back(std::move(v_alloc));
       }
       LayerTransferData ltd;
       ltd.layer_name = ctx.layer_name;
       ltd.layout = layout;
-      for (size_t i = 0; i < num; ++i) {
-        TransferBlock tb;
-        tb.block_idx = ctx.blocks_to_save[i].first;
-        tb.block.raw = ctx.raw_blocks[i].get();
-        tb.block.keep = ctx.raw_blocks[i];
-        ltd.blocks.push_back(std::move(tb));
+      if (!cfg_.blockwise_alloc) {
+        // One K buffer and one V buffer (or one block buffer): a uniform image.
+        ltd.image.kind = HostImage::Kind::Uniform;
+        ltd.image.block_ids = ctx.ids;
+        ltd.image.stride = ctx.stride;
+        const uint64_t bytes = ctx.stride * num;
+        if (!ctx.k_allocs[0]->mapped_ptr_for_host_range(ctx.k_allocs[0]->as_ptr(), bytes,
+                                                        &ltd.image.seg[0]) ||
+            (split && !ctx.v_allocs[0]->mapped_ptr_for_host_range(ctx.v_allocs[0]->as_ptr(), bytes,
+                                                                  &ltd.image.seg[1]))) {
+          return bad(err, PF_ERR_STORAGE, "segment exceeds its pinned allocation");
+        }
+        ltd.image.seg_allocation_id[0] = ctx.k_allocs[0]->allocation_id();
+        if (split) ltd.image.seg_allocation_id[1] = ctx.v_allocs[0]->allocation_id();
+      } else {
+        // One allocation per block and segment: per-block handles.
+        ctx.raw_blocks.reserve(num);
+        for (size_t q = 0; q < num; ++q) {
+          RawBlock raw;
+          if (!ctx.make_raw(q, cfg_.blockwise_alloc, &raw)) {
+            return bad(err, PF_ERR_STORAGE, "segment exceeds its pinned allocation");
+          }
+          ctx.raw_blocks.push_back(std::move(raw));
+        }
+        ltd.blocks.reserve(num);
+        for (size_t q = 0; q < num; ++q) {
+          TransferBlock tb;
+          tb.block_idx = (*ctx.ids)[q];
+          tb.block.raw = &ctx.raw_blocks[q];
+          ltd.blocks.push_back(std::move(tb));
+        }
       }
       gpu_layers.push_back(std::move(ltd));
     }
   }
+  prof.alloc_ms = ms_since(t_phase);
 
-  // ---- Phase 3: one GPU copy task, one synchronisation ---------------------
-  TaskResult res = gpu->worker_pool->batch_save(std::move(gpu_layers)).get();
-  if (res.status != PF_OK) return bad(err, res.status, res.message);
+  // ---- Phase 3: one GPU copy task, one synchronisation.  While the bytes
+  // move, the blocks that will enter the store are assembled on this thread;
+  // nothing becomes visible before the copy has succeeded. ------------------
+  t_phase = Clock::now();
+  std::future<TaskResult> pending = gpu->worker_pool->batch_save(std::move(gpu_layers));
 
-  // ---- Phase 4: insert into the store --------------------------------------
-  std::lock_guard<std::mutex> lock(mu_);
-  auto insert = [&](const BlockKey& key, size_t total_slots, size_t slot_id, RawBlock block) {
-    if (sealed_.count(key)) return;
-    auto it = inflight_.find(key);
-    if (it == inflight_.end()) it = inflight_.emplace(key, InflightBlock(total_slots)).first;
-    if (it->second.insert_slot(slot_id, std::move(block)) == InflightBlock::Insert::Completed) {
-      sealed_[key] = it->second.seal();
-      sealed_order_.push_back(key);
-      inflight_.erase(it);
-    }
+  struct Assembled {
+    const BlockKey* key;
+    InflightBlock block;
   };
-  if (page_first) {
-    const size_t slot_id = ctxs[0].slot_id;
-    size_t page_size = 0;
-    topo->shard_page_size(slot_id, &page_size);
-    for (size_t b = 0; b < pages.size(); ++b) {
-      Segment seg;
-      Segment::create(pages[b]->as_ptr(), page_size, pages[b], &seg);
-      insert(BlockKey{ns, ctxs[0].blocks_to_save[b].second}, topo->total_slots(), slot_id,
-             RawBlock::single_segment(std::move(seg)));
-    }
-  } else {
-    for (auto& ctx : ctxs) {
+  std::vector<Assembled> assembled;
+  int prep_status = PF_OK;
+  std::string prep_err;
+  if (!page_first) {
+    assembled.reserve(to_save);
+    for (size_t li = 0; li < lists.size() && prep_status == PF_OK; ++li) {
+      const SaveList& l = lists[li];
+      if (l.kept.empty()) continue;
       size_t total_slots = 0;
       std::string cause;
-      if (!topo->group_total_slots(ctx.group, &total_slots, &cause)) {
-        return bad(err, PF_ERR_INVALID_ARGUMENT, cause);
+      if (!topo->group_total_slots(l.group, &total_slots, &cause)) {
+        prep_status = PF_ERR_INVALID_ARGUMENT;
+        prep_err = cause;
+        break;
       }
-      for (size_t i = 0; i < ctx.blocks_to_save.size(); ++i) {
-        insert(BlockKey{ns, group_hash(ctx.blocks_to_save[i].second, ctx.group)}, total_slots,
-               ctx.slot_id, std::move(*ctx.raw_blocks[i]));
+      std::vector<SaveLayerCtx*> members;
+      for (auto& ctx : ctxs) {
+        if (ctx.list == li) members.push_back(&ctx);
+      }
+      for (size_t q = 0; q < l.kept.size() && prep_status == PF_OK; ++q) {
+        Assembled a{&l.keys[l.kept[q]], InflightBlock(total_slots)};
+        for (SaveLayerCtx* ctx : members) {
+          RawBlock raw;
+          if (!ctx->make_raw(q, cfg_.blockwise_alloc, &raw)) {
+            prep_status = PF_ERR_STORAGE;
+            prep_err = "segment exceeds its pinned allocation";
+            break;
+          }
+          a.block.insert_slot(ctx->slot_id, std::move(raw));
+        }
+        assembled.push_back(std::move(a));
       }
     }
   }
+  prof.assemble_ms = ms_since(t_phase);
+
+  TaskResult res = pending.get();
+  prof.transfer_ms = ms_since(t_phase);
+  if (res.status != PF_OK) return bad(err, res.status, res.message);
+  if (prep_status != PF_OK) return bad(err, prep_status, prep_err);
+
+  // ---- Phase 4: publish -----------------------------------------------------
+  t_phase = Clock::now();
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    auto seal = [&](const BlockKey& key, InflightBlock* b) {
+      sealed_[key] = b->seal();
+      sealed_order_.push_back(key);
+    };
+    if (page_first) {
+      const SaveList& l = lists[ctxs[0].list];
+      const size_t slot_id = ctxs[0].slot_id;
+      size_t page_size = 0;
+      topo->shard_page_size(slot_id, &page_size);
+      for (size_t b = 0; b < pages.size(); ++b) {
+        Segment seg;
+        Segment::create(pages[b]->as_ptr(), page_size, pages[b], &seg);
+        // Page-first keys carry the raw hash (one group per shard page).
+        const std::string raw_hash(reinterpret_cast<const char*>(l.hashes[l.kept[b]]),
+                                   l.lens[l.kept[b]]);
+        BlockKey key{ns, raw_hash};
+        if (sealed_.count(key)) continue;
+        auto it = inflight_.find(key);
+        if (it == inflight_.end()) {
+          it = inflight_.emplace(key, InflightBlock(topo->total_slots())).first;
+        }
+        if (it->second.insert_slot(slot_id, RawBlock::single_segment(std::move(seg))) ==
+            InflightBlock::Insert::Completed) {
+          seal(key, &it->second);
+          inflight_.erase(it);
+        }
+      }
+    } else {
+      for (Assembled& a : assembled) {
+        const BlockKey& key = *a.key;
+        if (sealed_.count(key)) continue;
+        auto it = inflight_.find(key);
+        if (it == inflight_.end()) {
+          if (a.block.complete()) {
+            seal(key, &a.block);
+          } else {
+            inflight_.emplace(key, std::move(a.block));
+          }
+        } else if (it->second.absorb(std::move(a.block)) == InflightBlock::Insert::Completed) {
+          seal(key, &it->second);
+          inflight_.erase(it);
+        }
+      }
+    }
+  }
+  prof.publish_ms = ms_since(t_phase);
+  prof.total_ms = ms_since(t_begin);
+  prof.bytes = res.bytes;
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    last_save_profile_ = prof;
+  }
   return PF_OK;
+}
+
+SaveProfile Engine::last_save_profile() {
+  std::lock_guard<std::mutex> lock(mu_);
+  return last_save_profile_;
 }
 
 int Engine::query_prefix(const std::string& instance_id, const std::vector<std::string>& hashes,
@@ -696,6 +864,14 @@ int Engine::batch_load_kv_blocks_multi_layer(
     block_cache.insert(block_cache.end(), blocks.begin(), blocks.end());
   }
   // One LayerTransferData per layer.
+  struct PageList {
+    std::shared_ptr<std::vector<MappedPinnedPtr>> pages;
+    std::shared_ptr<std::vector<uint64_t>> alloc_ids;
+    std::shared_ptr<std::vector<uint32_t>> ids;
+    uint64_t page_len = 0;
+  };
+  std::map<std::pair<size_t, size_t>, PageList> page_lists;
+  const bool page_first = topo->is_page_first();
   std::vector<LayerTransferData> layers;
   for (size_t gi = 0; gi < layer_groups.size(); ++gi) {
     for (const std::string& name : layer_groups[gi]) {
@@ -716,6 +892,43 @@ int Engine::batch_load_kv_blocks_multi_layer(
       LayerTransferData ltd;
       ltd.layer_name = name;
       ltd.layout = lit->second;
+      if (page_first && !targets[gi].empty()) {
+        // Every layer of a shard reads the same pages at its own offset: one
+        // shared page list per (group, slot) instead of per-block handles.
+        PageList& pl = page_lists[{gi, slot_id}];
+        if (!pl.pages) {
+          auto pages = std::make_shared<std::vector<MappedPinnedPtr>>();
+          auto alloc_ids = std::make_shared<std::vector<uint64_t>>();
+          auto ids = std::make_shared<std::vector<uint32_t>>();
+          uint64_t page_len = UINT64_MAX;
+          for (auto& t : targets[gi]) {
+            const RawBlock* raw = block_cache[t.second]->get_slot(slot_id);
+            MappedPinnedPtr p;
+            if (!raw || !raw->segment_mapped_ptr(0, &p)) {
+              return bad(err, PF_ERR_INVALID_ARGUMENT,
+                         "stored block is missing slot " + std::to_string(slot_id) +
+                             " for layer " + name);
+            }
+            pages->push_back(p);
+            alloc_ids->push_back(raw->segment_allocation_id(0));
+            ids->push_back(static_cast<uint32_t>(t.first));
+            page_len = std::min(page_len, raw->segment_size(0));
+          }
+          pl.pages = std::move(pages);
+          pl.alloc_ids = std::move(alloc_ids);
+          pl.ids = std::move(ids);
+          pl.page_len = page_len;
+        }
+        ltd.image.kind = HostImage::Kind::Paged;
+        ltd.image.block_ids = pl.ids;
+        ltd.image.pages = pl.pages;
+        ltd.image.page_allocation_ids = pl.alloc_ids;
+        ltd.image.offset = host_offset;
+        ltd.image.page_len = pl.page_len;
+        layers.push_back(std::move(ltd));
+        continue;
+      }
+      ltd.blocks.reserve(targets[gi].size());
       for (auto& t : targets[gi]) {
         const auto& sealed = block_cache[t.second];
         const RawBlock* raw = sealed->get_slot(slot_id);
@@ -727,12 +940,16 @@ int Engine::batch_load_kv_blocks_multi_layer(
         TransferBlock tb;
         tb.block_idx = t.first;
         tb.block.raw = raw;
-        tb.block.keep = sealed;
         tb.block.offset = host_offset;
         ltd.blocks.push_back(std::move(tb));
       }
       if (!ltd.blocks.empty()) layers.push_back(std::move(ltd));
     }
+  }
+  // The leased blocks stay alive through the first layer of the task.
+  if (!layers.empty()) {
+    layers.front().keep.reserve(block_cache.size());
+    for (auto& b : block_cache) layers.front().keep.push_back(b);
   }
   if (layers.empty()) {
     // Nothing to load: complete at once (lib.rs:885-890).

@@ -33,11 +33,22 @@ struct EngineConfig {
   uint64_t unit_size_hint = 0;
 };
 
-// block.rs:20-25.
-struct LayerSave {
-  std::string layer_name;
-  std::vector<uint64_t> block_ids;
-  std::vector<std::string> block_hashes;
+// block.rs:20-25, as a view of the caller's arrays (valid for the call).
+struct LayerSaveView {
+  const char* layer_name = nullptr;
+  const uint64_t* block_ids = nullptr;
+  size_t n_ids = 0;
+  const uint8_t* const* hashes = nullptr;
+  const uint32_t* hash_lens = nullptr;
+  size_t n_hashes = 0;
+};
+
+// Where the time of the last successful save went (offload.rs:560-574 records
+// the same phases as metrics).  assemble_ms runs inside transfer_ms.
+struct SaveProfile {
+  double validate_ms = 0, filter_ms = 0, alloc_ms = 0, assemble_ms = 0, transfer_ms = 0,
+         publish_ms = 0, total_ms = 0;
+  uint64_t bytes = 0;
 };
 
 // One lease's destinations: per load group, one entry per leased block; -1 = skip.
@@ -99,7 +110,8 @@ class Engine {
   // offload.rs:293-659.  Returns once the bytes are in host memory and the
   // blocks are queryable.
   int batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank, size_t pp_rank,
-                           int device_id, const std::vector<LayerSave>& saves, std::string* err);
+                           int device_id, const std::vector<LayerSaveView>& saves, std::string* err);
+  SaveProfile last_save_profile();
   // Longest cached prefix of `hashes` (group 0 keys) + a lease over those
   // blocks (lib.rs:506-546,614-629).
   int query_prefix(const std::string& instance_id, const std::vector<std::string>& hashes,
@@ -142,6 +154,7 @@ class Engine {
   };
   std::map<uint64_t, Lease> leases_;
   uint64_t next_lease_ = 1;
+  SaveProfile last_save_profile_;
 };
 
 }  // namespace pf

@@ -316,25 +316,42 @@ int pf_engine_batch_save(pf_engine_t e, const char* instance_id, uint64_t tp_ran
                          uint64_t n_saves) {
   PF_REQUIRE_PTR(e);
   PF_REQUIRE_PTR(instance_id);
-  std::vector<pf::LayerSave> v;
+  std::vector<pf::LayerSaveView> v(n_saves);
   for (uint64_t i = 0; i < n_saves; ++i) {
-    pf::LayerSave s;
-    s.layer_name = saves[i].layer_name ? saves[i].layer_name : "";
-    s.block_ids.assign(saves[i].block_ids, saves[i].block_ids + saves[i].n_blocks);
+    v[i].layer_name = saves[i].layer_name;
+    v[i].block_ids = saves[i].block_ids;
+    v[i].n_ids = saves[i].n_blocks;
     // A NULL hash list with blocks present is a length mismatch, as in the
     // reference's engine-level contract (offload.rs:328-335).
-    if (saves[i].block_hashes) {
-      for (uint64_t b = 0; b < saves[i].n_blocks; ++b) {
-        s.block_hashes.push_back(hash_of(saves[i].block_hashes[b], saves[i].block_hash_lens[b]));
-      }
+    const bool has_hashes = saves[i].block_hashes != nullptr && saves[i].block_hash_lens != nullptr;
+    v[i].hashes = has_hashes ? saves[i].block_hashes : nullptr;
+    v[i].hash_lens = has_hashes ? saves[i].block_hash_lens : nullptr;
+    v[i].n_hashes = has_hashes ? saves[i].n_blocks : 0;
+    if (saves[i].n_blocks != 0 && saves[i].block_ids == nullptr) {
+      return pf::fail(PF_ERR_INVALID_ARGUMENT, "layer save %llu has blocks but no block_ids",
+                      static_cast<unsigned long long>(i));
     }
-    v.push_back(std::move(s));
   }
   std::string err;
   int st = reinterpret_cast<pf::Engine*>(e)->batch_save_kv_blocks(instance_id, tp_rank, pp_rank,
                                                                   device_id, v, &err);
   if (st != PF_OK) pf::last_error() = err;
   return st;
+}
+
+int pf_engine_last_save_profile(pf_engine_t e, pf_save_profile* out) {
+  PF_REQUIRE_PTR(e);
+  PF_REQUIRE_PTR(out);
+  const pf::SaveProfile p = reinterpret_cast<pf::Engine*>(e)->last_save_profile();
+  out->validate_ms = p.validate_ms;
+  out->filter_ms = p.filter_ms;
+  out->alloc_ms = p.alloc_ms;
+  out->assemble_ms = p.assemble_ms;
+  out->transfer_ms = p.transfer_ms;
+  out->publish_ms = p.publish_ms;
+  out->total_ms = p.total_ms;
+  out->bytes = p.bytes;
+  return PF_OK;
 }
 
 int pf_engine_query_prefix(pf_engine_t e, const char* instance_id, const uint8_t* const* hashes,

@@ -10,11 +10,60 @@
 namespace pf {
 
 bool build_copy_descs(const std::vector<LayerTransferData>& layers, std::vector<CopyDesc>* out,
-                      uint64_t* total_bytes, std::string* err) {
+                      uint64_t* total_bytes, std::string* err, size_t begin, size_t end) {
   out->clear();
   uint64_t total = 0;
-  for (size_t li = 0; li < layers.size(); ++li) {
+  if (end <= begin) {
+    begin = 0;
+    end = layers.size();
+  }
+  for (size_t li = begin; li < end && li < layers.size(); ++li) {
     const LayerTransferData& layer = layers[li];
+    if (layer.image.kind != HostImage::Kind::None) {
+      // The same descriptors per-block handles over this image would give.
+      const HostImage& im = layer.image;
+      const size_t n = im.size();
+      const bool paged = im.kind == HostImage::Kind::Paged;
+      if (paged && (!im.pages || im.pages->size() != n || !im.page_allocation_ids ||
+                    im.page_allocation_ids->size() != n)) {
+        *err = "layer " + layer.layer_name + ": host image has a page list of the wrong length";
+        return false;
+      }
+      for (size_t i = 0; i < n; ++i) {
+        BlockCopies bc;
+        std::string cause;
+        if (!layer.layout.block_copies((*im.block_ids)[i], &bc, &cause)) {
+          *err = "layer " + layer.layer_name + ": " + cause;
+          return false;
+        }
+        MappedPinnedPtr k, v;
+        uint64_t k_alloc, v_alloc;
+        if (paged) {
+          k = (*im.pages)[i].add(im.offset);
+          v = k.add(bc.k.bytes);
+          k_alloc = v_alloc = (*im.page_allocation_ids)[i];
+        } else {
+          k = im.seg[0].add(i * im.stride);
+          k_alloc = im.seg_allocation_id[0];
+          if (bc.n == 2 && im.seg[1].host != nullptr) {
+            v = im.seg[1].add(i * im.stride);
+            v_alloc = im.seg_allocation_id[1];
+          } else {
+            v = k.add(bc.k.bytes);
+            v_alloc = k_alloc;
+          }
+        }
+        out->push_back({bc.k.addr, k.host, reinterpret_cast<uint64_t>(k.device), bc.k.bytes, li,
+                        k_alloc});
+        total += bc.k.bytes;
+        if (bc.n == 2) {
+          out->push_back({bc.v.addr, v.host, reinterpret_cast<uint64_t>(v.device), bc.v.bytes, li,
+                          v_alloc});
+          total += bc.v.bytes;
+        }
+      }
+      continue;
+    }
     for (const TransferBlock& tb : layer.blocks) {
       BlockCopies bc;
       std::string cause;
@@ -63,6 +112,12 @@ struct BlockForm {
   std::vector<std::vector<uint32_t>> ids;
   std::vector<std::vector<uint64_t>> page_host;
   std::vector<std::vector<uint64_t>> page_dev;
+  // Page tables of host images, one per distinct page list, so that the
+  // layers of a page-first task pass the very same table.
+  std::vector<const void*> image_pages;
+  std::vector<std::vector<uint64_t>> image_page_host;
+  std::vector<std::vector<uint64_t>> image_page_dev;
+  std::vector<int> layer_table;  // per layer: index into image_pages, or -1
   uint64_t total_bytes = 0;
 };
 
@@ -71,25 +126,69 @@ struct BlockForm {
 // neither form (e.g. K and V of each block in unrelated allocations); the
 // caller then falls back to per-fragment descriptors.  Errors are reported
 // through *err with *failed = true.
-bool to_block_form(const std::vector<LayerTransferData>& layers, BlockForm* out, bool* failed,
-                   std::string* err) {
+bool to_block_form(const std::vector<LayerTransferData>& all_layers, size_t begin, size_t end,
+                   BlockForm* out, bool* failed, std::string* err) {
   *failed = false;
-  const size_t n_layers = layers.size();
+  const size_t n_layers = end - begin;
   out->layers.resize(n_layers);
   out->ids.resize(n_layers);
   out->page_host.resize(n_layers);
   out->page_dev.resize(n_layers);
+  out->layer_table.assign(n_layers, -1);
   for (size_t li = 0; li < n_layers; ++li) {
-    const LayerTransferData& layer = layers[li];
+    const LayerTransferData& layer = all_layers[begin + li];
     pf_layer_blocks& lb = out->layers[li];
     std::memset(&lb, 0, sizeof(lb));
     lb.layer_name = layer.layer_name.c_str();
     lb.layout = layer.layout.c();
+    const bool split = layer.layout.is_split();
+    const uint64_t frag = layer.layout.fragment_bytes();
+    if (layer.image.kind != HostImage::Kind::None) {
+      const HostImage& im = layer.image;
+      const size_t n_im = im.size();
+      lb.n_blocks = n_im;
+      if (n_im == 0) continue;
+      // Block ids are range-checked by the transfer engine's own planning.
+      lb.block_ids = im.block_ids->data();
+      out->total_bytes += frag * (split ? 2 : 1) * n_im;
+      if (im.kind == HostImage::Kind::Uniform) {
+        const int n_seg = split ? 2 : 1;
+        for (int sgi = 0; sgi < n_seg; ++sgi) {
+          const MappedPinnedPtr base = (sgi == 1 && im.seg[1].host == nullptr)
+                                           ? im.seg[0].add(frag) : im.seg[sgi];
+          lb.host[sgi] = base.host;
+          lb.host_device[sgi] = reinterpret_cast<uint64_t>(base.device);
+          lb.host_len[sgi] = (n_im - 1) * im.stride + frag;
+        }
+        lb.host_stride = im.stride;
+        continue;
+      }
+      if (!im.pages || im.pages->size() != n_im) {
+        *err = "layer " + layer.layer_name + ": host image has a page list of the wrong length";
+        *failed = true;
+        return false;
+      }
+      size_t ti = 0;
+      while (ti < out->image_pages.size() && out->image_pages[ti] != im.pages.get()) ++ti;
+      if (ti == out->image_pages.size()) {
+        out->image_pages.push_back(im.pages.get());
+        out->image_page_host.emplace_back(n_im);
+        out->image_page_dev.emplace_back(n_im);
+        for (size_t i = 0; i < n_im; ++i) {
+          out->image_page_host[ti][i] = reinterpret_cast<uint64_t>((*im.pages)[i].host);
+          out->image_page_dev[ti][i] = reinterpret_cast<uint64_t>((*im.pages)[i].device);
+        }
+      }
+      // (the vectors are filled once and never resized afterwards; the outer
+      // vectors may grow, so the pointers are taken after the loop below)
+      lb.page_offset = im.offset;
+      lb.page_len = im.page_len;
+      out->layer_table[li] = static_cast<int>(ti);
+      continue;
+    }
     const size_t n = layer.blocks.size();
     lb.n_blocks = n;
     if (n == 0) continue;
-    const bool split = layer.layout.is_split();
-    const uint64_t frag = layer.layout.fragment_bytes();
     std::vector<uint32_t>& ids = out->ids[li];
     ids.resize(n);
     std::vector<MappedPinnedPtr> k(n), v(n);
@@ -167,6 +266,12 @@ bool to_block_form(const std::vector<LayerTransferData>& layers, BlockForm* out,
     lb.page_host_device = pd.data();
     lb.page_offset = 0;
     lb.page_len = frag * (split ? 2 : 1);
+  }
+  for (size_t li = 0; li < n_layers; ++li) {
+    const int ti = out->layer_table[li];
+    if (ti < 0) continue;
+    out->layers[li].page_host = out->image_page_host[ti].data();
+    out->layers[li].page_host_device = out->image_page_dev[ti].data();
   }
   return true;
 }
@@ -293,32 +398,47 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
     TaskResult res;
     std::string err;
     int st = PF_OK;
-    bool done_fast = false;
-    if (xfer) {
-      BlockForm form;
-      bool failed = false;
-      if (to_block_form(task->layers, &form, &failed, &err)) {
-        st = is_load ? xfer->load(form.layers.data(), form.layers.size(), path, stream)
-                     : xfer->save(form.layers.data(), form.layers.size(), path, stream);
-        if (st != PF_OK) err = last_error();
-        res.bytes = form.total_bytes;
-        done_fast = true;
-      } else if (failed) {
-        st = PF_ERR_STORAGE;
-        done_fast = true;
+    // A task whose layers come as per-block handles is converted in two
+    // parts: a few layers first, so that the device starts on them while the
+    // (much larger) rest is still being converted.  Everything is only
+    // enqueued; there is still one synchronisation.  Tasks described by host
+    // images need no conversion work and go in one call, which also keeps the
+    // layers of page-first pages together for whole-page staging.
+    const size_t n_layers = task->layers.size();
+    bool per_block = false;
+    for (const auto& l : task->layers) per_block |= !l.blocks.empty();
+    size_t first_part = n_layers ? n_layers : 1;
+    if (xfer && per_block && n_layers >= 16) first_part = n_layers / 16 < 2 ? 2 : n_layers / 16;
+    for (size_t begin = 0; begin < n_layers && st == PF_OK;) {
+      const size_t end = begin == 0 ? (first_part < n_layers ? first_part : n_layers) : n_layers;
+      bool done_fast = false;
+      if (xfer) {
+        BlockForm form;
+        bool failed = false;
+        if (to_block_form(task->layers, begin, end, &form, &failed, &err)) {
+          st = is_load ? xfer->load(form.layers.data(), form.layers.size(), path, stream)
+                       : xfer->save(form.layers.data(), form.layers.size(), path, stream);
+          if (st != PF_OK) err = last_error();
+          res.bytes += form.total_bytes;
+          done_fast = true;
+        } else if (failed) {
+          st = PF_ERR_STORAGE;
+          done_fast = true;
+        }
       }
-    }
-    if (!done_fast) {
-      std::vector<CopyDesc> copies;
-      uint64_t total = 0;
-      if (!build_copy_descs(task->layers, &copies, &total, &err)) {
-        st = PF_ERR_STORAGE;
-      } else {
-        st = is_load ? backend->h2d(copies.data(), copies.size(), stream)
-                     : backend->d2h(copies.data(), copies.size(), stream);
-        if (st != PF_OK) err = last_error();
-        res.bytes = total;
+      if (!done_fast) {
+        std::vector<CopyDesc> copies;
+        uint64_t total = 0;
+        if (!build_copy_descs(task->layers, &copies, &total, &err, begin, end)) {
+          st = PF_ERR_STORAGE;
+        } else {
+          st = is_load ? backend->h2d(copies.data(), copies.size(), stream)
+                       : backend->d2h(copies.data(), copies.size(), stream);
+          if (st != PF_OK) err = last_error();
+          res.bytes += total;
+        }
       }
+      begin = end;
     }
     if (st == PF_OK) {
       // One synchronisation for all layers.

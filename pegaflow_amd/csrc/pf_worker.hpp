@@ -38,11 +38,37 @@ struct TransferBlock {
   HostBlock block;
 };
 
-// gpu_worker.rs:54-59.
+// The host side of a whole layer when it is regular, so that a task of
+// hundreds of thousands of fragments needs no per-block handle.  It describes
+// exactly the blocks a list of TransferBlocks over the same memory would:
+//   Uniform: list position i at seg[s] + i * stride (the batch image of a
+//            save: one K buffer and one V buffer, or one block buffer);
+//   Paged:   list position i at pages[i] + offset, V right behind K (one page
+//            or one allocation per block).
+struct HostImage {
+  enum class Kind { None, Uniform, Paged };
+  Kind kind = Kind::None;
+  std::shared_ptr<const std::vector<uint32_t>> block_ids;  // device block of each position
+  MappedPinnedPtr seg[2];
+  uint64_t seg_allocation_id[2] = {0, 0};
+  uint64_t stride = 0;
+  std::shared_ptr<const std::vector<MappedPinnedPtr>> pages;
+  std::shared_ptr<const std::vector<uint64_t>> page_allocation_ids;
+  uint64_t offset = 0;
+  uint64_t page_len = 0;
+  std::vector<std::shared_ptr<const void>> keep;  // what owns the memory
+  size_t size() const { return block_ids ? block_ids->size() : 0; }
+};
+
+// gpu_worker.rs:54-59.  Either `blocks` (one handle per block) or `image`.
 struct LayerTransferData {
   std::string layer_name;
   KVCacheLayout layout;
   std::vector<TransferBlock> blocks;
+  HostImage image;
+  // Owners of the host memory for the whole layer (or task), for callers that
+  // would otherwise repeat one owner in every block's `keep`.
+  std::vector<std::shared_ptr<const void>> keep;
 };
 
 // Result of a task: status code (PF_OK or an error class) and message.
@@ -104,7 +130,8 @@ class GpuWorkerPool {
 };
 
 // gpu_worker.rs:353-423 over the C++ types (the C-ABI form is pf_build_copy_descs).
+// Layers [begin, end) only when end > begin; the whole task otherwise.
 bool build_copy_descs(const std::vector<LayerTransferData>& layers, std::vector<CopyDesc>* out,
-                      uint64_t* total_bytes, std::string* err);
+                      uint64_t* total_bytes, std::string* err, size_t begin = 0, size_t end = 0);
 
 }  // namespace pf

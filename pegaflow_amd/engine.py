@@ -282,6 +282,12 @@ class PegaEngine:
                                              C.byref(t)))
         return Task(t, keep)
 
+    def last_save_profile(self) -> dict:
+        """Milliseconds per phase of the last successful save (and its bytes)."""
+        p = _lib.PfSaveProfile()
+        check(self._lib.pf_engine_last_save_profile(self.handle, C.byref(p)))
+        return {name: getattr(p, name) for name, _ in p._fields_}
+
     def pool_usage(self) -> tuple[int, int]:
         used, total = C.c_uint64(), C.c_uint64()
         check(self._lib.pf_engine_pool_usage(self.handle, C.byref(used), C.byref(total)))
