@@ -73,6 +73,7 @@ def parse_args():
     ap.add_argument("--zc-max-wg", type=int, default=0)
     ap.add_argument("--no-overlap", action="store_true", help="skip the GEMM-overlap section")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-engine", action="store_true", help="skip the save/query/load engine section")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--settle-max", type=int, default=8,
@@ -357,6 +358,11 @@ def main():
     if not args.no_overlap:
         duplex = run_duplex(xfer, save_layers, load_layers, stream, path, payload, args)
 
+    # ---- the same workload through the save / query / load engine -----------
+    engine = None
+    if not args.no_engine:
+        engine = run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, payload)
+
     # ---- CPU baseline: the oracle's memcpy executor on the host cores -----
     cpu = None
     if not args.no_cpu:
@@ -390,6 +396,7 @@ def main():
         "cpu_baseline": cpu,
         "overlap": overlap,
         "duplex": duplex,
+        "engine": engine,
         "pool_alloc_s": round(pool_alloc_s, 2),
         "device": runtime.device_name(0),
     }
@@ -450,6 +457,71 @@ def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_
             out["per_layer_ms_mean"] = round(sum(per_layer) / len(per_layer), 3)
             out["per_layer_ms_max"] = round(max(per_layer), 3)
             out["first_layer_ready_ms"] = round(done[0], 3)
+    return out
+
+
+def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, payload):
+    """End to end through pf_engine_*: registration, batch_save (host image
+    allocation in the pinned pool, one worker task, block bookkeeping), prefix
+    query, batch_load into a second instance of the same namespace.  Times are
+    wall clock around the C calls with the arguments packed beforehand."""
+    from pegaflow_amd.engine import LayerSave, LoadState, PackedSaves, PegaEngine
+    from pegaflow_amd.transfer import TransferMode
+    nb, seg, n = w["num_blocks"], w["seg"], w["n"]
+    nseg = 2 if w["split"] else 1
+    n_layers = len(names)
+    eng = PegaEngine(pool_size=int(payload * 1.2) + (256 << 20))
+    kv = nb * seg if nseg == 2 else 0
+    for inst, caches in (("bench-src", src_cache), ("bench-dst", dst_cache)):
+        eng.register_context_layer_batch(
+            inst, "bench", 0, 0, 0, 1, 1, names, [t.data_ptr() for t in caches],
+            [nseg * nb * seg] * n_layers, [nb] * n_layers, [seg] * n_layers, [kv] * n_layers,
+            [nseg] * n_layers, transfer_mode=TransferMode.DIRECT, page_first=w["page_first"])
+    for t in dst_cache:
+        t.zero_()
+    torch.cuda.synchronize()
+    out = {"transfer_mode": "direct"}
+    reps = 3
+    save_s, load_s, query_s = [], [], []
+    for rep in range(reps):
+        hashes = [bytes([rep]) + int(i).to_bytes(4, "little") + bytes(27) for i in range(n)]
+        packed = PackedSaves([LayerSave(nm, save_ids, hashes) for nm in names])
+        t0 = time.perf_counter()
+        eng.batch_save_kv_blocks("bench-src", 0, 0, 0, packed)
+        save_s.append(time.perf_counter() - t0)
+        t0 = time.perf_counter()
+        hits, lease = eng.query_prefix("bench-dst", hashes)
+        query_s.append(time.perf_counter() - t0)
+        assert hits == n, f"engine query found {hits} of {n} blocks"
+        state = LoadState()
+        t0 = time.perf_counter()
+        task = eng.batch_load_kv_blocks_multi_layer("bench-dst", 0, 0, [names], lease,
+                                                    [load_ids.tolist()], state)
+        res = task.wait()   # raises if the load failed
+        load_s.append(time.perf_counter() - t0)
+        assert res.done and state.get() == 1, "engine load did not complete"
+        task.close()
+        state.close()
+        if rep == reps - 1:
+            out["save_profile_ms"] = {k: round(v, 2) for k, v in eng.last_save_profile().items()
+                                      if k != "bytes"}
+        eng.evict_all()
+    dev = src_cache[0].device
+    sid = torch.from_numpy(save_ids.astype(np.int64)).to(dev)
+    lid = torch.from_numpy(load_ids.astype(np.int64)).to(dev)
+    for li in sorted({0, n_layers - 1}):
+        s_ = src_cache[li].view(torch.uint8).reshape(nseg, nb, seg)
+        d_ = dst_cache[li].view(torch.uint8).reshape(nseg, nb, seg)
+        if not torch.equal(d_[:, lid], s_[:, sid]):
+            print(f"bench.py: engine round trip differs on layer {li}", file=sys.stderr)
+            sys.exit(1)
+    out["save_gbps"] = round(payload / min(save_s) / 1e9, 2)
+    out["load_gbps"] = round(payload / min(load_s) / 1e9, 2)
+    out["save_gbps_all"] = [round(payload / t / 1e9, 2) for t in save_s]
+    out["load_gbps_all"] = [round(payload / t / 1e9, 2) for t in load_s]
+    out["query_ms"] = round(min(query_s) * 1e3, 2)
+    out["blocks"] = n
+    eng.close()
     return out
 
 

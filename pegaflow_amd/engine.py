@@ -10,6 +10,8 @@ import ctypes as C
 from dataclasses import dataclass
 from typing import Sequence
 
+import numpy as np
+
 from . import _lib
 from ._lib import check
 from .transfer import LayerTransferData, TransferMode
@@ -162,11 +164,53 @@ class LayerSave:
 
 
 def _pack_hashes(hashes: Sequence[bytes]):
+    """-> (pointer array, length array, backing buffer) for a list of byte strings."""
     n = len(hashes)
-    bufs = [(C.c_uint8 * max(len(h), 1)).from_buffer_copy(h if h else b"\0") for h in hashes]
-    ptrs = (C.POINTER(C.c_uint8) * max(n, 1))(*[C.cast(b, C.POINTER(C.c_uint8)) for b in bufs])
-    lens = (C.c_uint32 * max(n, 1))(*[len(h) for h in hashes])
-    return ptrs, lens, bufs
+    lens_np = np.fromiter((len(h) for h in hashes), dtype=np.uint32, count=n)
+    blob = np.frombuffer(b"".join(hashes) + b"\0", dtype=np.uint8)
+    starts = np.zeros(max(n, 1), dtype=np.uint64)
+    if n > 1:
+        np.cumsum(lens_np[:-1], out=starts[1:n])
+    addrs = (starts + np.uint64(blob.ctypes.data)).astype(np.uint64)
+    ptrs = C.cast(addrs.ctypes.data, C.POINTER(C.POINTER(C.c_uint8)))
+    lens_keep = np.ascontiguousarray(lens_np if n else np.zeros(1, dtype=np.uint32))
+    lens = C.cast(lens_keep.ctypes.data, C.POINTER(C.c_uint32))
+    return ptrs, lens, (blob, addrs, lens_keep)
+
+
+class PackedSaves:
+    """The C form of a list of LayerSave, reusable across calls.  Layers that
+    pass the very same hash list object share one packed copy."""
+
+    def __init__(self, saves: Sequence[LayerSave]):
+        n = len(saves)
+        self.n = n
+        self.array = (_lib.PfLayerSave * max(n, 1))()
+        self._keep = []
+        packed_hashes = {}
+        for i, s in enumerate(saves):
+            if len(s.block_hashes) != len(s.block_ids):
+                # offload.rs:328-335
+                raise _lib.InvalidArgument(
+                    _lib.PF_ERR_INVALID_ARGUMENT,
+                    f"block_ids length {len(s.block_ids)} does not match block_hashes "
+                    f"{len(s.block_hashes)} for layer {s.layer_name}")
+            ids = np.ascontiguousarray(s.block_ids, dtype=np.uint64)
+            if ids.size == 0:
+                ids = np.zeros(1, dtype=np.uint64)
+            name = s.layer_name.encode()
+            key = id(s.block_hashes)
+            if key not in packed_hashes:
+                packed_hashes[key] = _pack_hashes(s.block_hashes)
+            ptrs, lens, _ = packed_hashes[key]
+            a = self.array[i]
+            a.layer_name = name
+            a.block_ids = C.cast(ids.ctypes.data, C.POINTER(C.c_uint64))
+            a.n_blocks = len(s.block_ids)
+            a.block_hashes = ptrs
+            a.block_hash_lens = lens
+            self._keep.append((ids, name, s.block_hashes))
+        self._keep.append(packed_hashes)
 
 
 class PegaEngine:
@@ -218,29 +262,10 @@ class PegaEngine:
         check(self._lib.pf_engine_unregister_instance(self.handle, instance_id.encode()))
 
     def batch_save_kv_blocks(self, instance_id: str, tp_rank: int, pp_rank: int, device_id: int,
-                             saves: Sequence[LayerSave]) -> None:
-        n = len(saves)
-        arr = (_lib.PfLayerSave * max(n, 1))()
-        keep = []
-        for i, s in enumerate(saves):
-            ids = (C.c_uint64 * max(len(s.block_ids), 1))(*[int(b) for b in s.block_ids])
-            name = s.layer_name.encode()
-            arr[i].layer_name = name
-            arr[i].block_ids = ids
-            arr[i].n_blocks = len(s.block_ids)
-            if len(s.block_hashes) != len(s.block_ids):
-                # offload.rs:328-335
-                raise _lib.InvalidArgument(
-                    _lib.PF_ERR_INVALID_ARGUMENT,
-                    f"block_ids length {len(s.block_ids)} does not match block_hashes "
-                    f"{len(s.block_hashes)} for layer {s.layer_name}")
-            ptrs, lens, bufs = _pack_hashes(s.block_hashes)
-            arr[i].block_hashes = ptrs
-            arr[i].block_hash_lens = lens
-            keep.append((ptrs, lens, bufs))
-            keep.append((ids, name))
+                             saves: Sequence[LayerSave] | PackedSaves) -> None:
+        packed = saves if isinstance(saves, PackedSaves) else PackedSaves(saves)
         check(self._lib.pf_engine_batch_save(self.handle, instance_id.encode(), tp_rank, pp_rank,
-                                             device_id, arr, n))
+                                             device_id, packed.array, packed.n))
 
     def query_prefix(self, instance_id: str, hashes: Sequence[bytes]) -> tuple[int, int]:
         """-> (hit blocks, lease id); lease 0 when nothing hit."""
