@@ -308,3 +308,86 @@ def test_worker_pool_matches_oracle(gpu, mode, use_desc):
 def test_worker_pool_init_failure_is_synchronous(gpu):
     with pytest.raises(_lib.PegaHipError, match="Failed to initialise GPU worker on device 99"):
         GpuWorkerPool(99)
+
+
+def test_layers_saved_in_separate_calls_complete_the_same_blocks(engine):
+    """Slots of a block may arrive in several saves (block.rs:346-454): the block
+    is queryable only once every layer's slot is in, and layers that carry
+    different hash lists in one call are kept apart."""
+    a = Layer("layer_a", 8, 2048)
+    b = Layer("layer_b", 8, 1024, overwrite=7, split_kv_stride=8 * 1024)
+    register(engine, "two-calls", [a, b])
+    hashes = make_block_hashes(4, 9)
+    ids_a, ids_b = [0, 2, 4, 6], [7, 5, 3, 1]
+    engine.batch_save_kv_blocks("two-calls", 0, 0, 0, [LayerSave("layer_a", ids_a, hashes)])
+    assert engine.query_prefix("two-calls", hashes) == (0, 0)
+    assert engine.cached_blocks == 0
+    other = make_block_hashes(2, 10)
+    engine.batch_save_kv_blocks("two-calls", 0, 0, 0, [
+        LayerSave("layer_b", ids_b, hashes),           # completes the four blocks
+        LayerSave("layer_a", [1, 3], other),           # a different list in the same call
+    ])
+    hits, lease = engine.query_prefix("two-calls", hashes)
+    assert hits == 4 and engine.cached_blocks == 4
+    assert engine.query_prefix("two-calls", other) == (0, 0)    # layer_b's slots still missing
+    a.zero_gpu()
+    b.zero_gpu()
+    dest = [1, 3, 5, 7]
+    engine.batch_load_kv_blocks_multi_layer("two-calls", 0, 0, [["layer_a", "layer_b"]], lease,
+                                            [dest]).wait()
+    want_a = np.zeros_like(a.expected)
+    want_b = np.zeros_like(b.expected)
+    for pos, dst in enumerate(dest):
+        want_a[dst * 2048:(dst + 1) * 2048] = a.expected[ids_a[pos] * 2048:(ids_a[pos] + 1) * 2048]
+        for region in (0, 8 * 1024):
+            src = ids_b[pos]
+            want_b[region + dst * 1024: region + (dst + 1) * 1024] = \
+                b.expected[region + src * 1024: region + (src + 1) * 1024]
+    a.assert_gpu_matches(want_a)
+    b.assert_gpu_matches(want_b)
+
+
+def test_repeated_hash_in_one_list_keeps_the_first_image(engine):
+    """Duplicate hashes are not rejected (offload.rs:348-368): every occurrence is
+    copied, the first one enters the store."""
+    layer = Layer("layer_0", 8, 1024)
+    register(engine, "dup-hash", [layer])
+    h = make_block_hashes(2, 4)
+    engine.batch_save_kv_blocks("dup-hash", 0, 0, 0,
+                                [LayerSave("layer_0", [5, 6, 2], [h[0], h[1], h[0]])])
+    assert engine.cached_blocks == 2
+    layer.zero_gpu()
+    hits, lease = engine.query_prefix("dup-hash", h)
+    assert hits == 2
+    engine.batch_load_kv_blocks_multi_layer("dup-hash", 0, 0, [["layer_0"]], lease, [[0, 1]]).wait()
+    want = np.zeros_like(layer.expected)
+    want[0:1024] = layer.expected[5 * 1024:6 * 1024]
+    want[1024:2048] = layer.expected[6 * 1024:7 * 1024]
+    layer.assert_gpu_matches(want)
+    prof = engine.last_save_profile()
+    assert prof["bytes"] == 3 * 1024 and prof["total_ms"] >= prof["transfer_ms"] > 0
+
+
+def test_packed_saves_are_reusable_and_share_hash_lists(engine):
+    from pegaflow_amd.engine import PackedSaves
+    layers = [Layer(f"l{i}", 6, 512, overwrite=i) for i in range(3)]
+    register(engine, "packed", layers)
+    hashes = make_block_hashes(3, 6)
+    packed = PackedSaves([LayerSave(l.name, np.array([4, 0, 2], dtype=np.uint64), hashes)
+                          for l in layers])
+    engine.batch_save_kv_blocks("packed", 0, 0, 0, packed)
+    assert engine.cached_blocks == 3
+    engine.evict_all()
+    assert engine.cached_blocks == 0
+    engine.batch_save_kv_blocks("packed", 0, 0, 0, packed)
+    hits, lease = engine.query_prefix("packed", hashes)
+    assert hits == 3
+    for l in layers:
+        l.zero_gpu()
+    engine.batch_load_kv_blocks_multi_layer("packed", 0, 0, [[l.name for l in layers]], lease,
+                                            [[1, 3, 5]]).wait()
+    for l in layers:
+        want = np.zeros_like(l.expected)
+        for src, dst in zip([4, 0, 2], [1, 3, 5]):
+            want[dst * 512:(dst + 1) * 512] = l.expected[src * 512:(src + 1) * 512]
+        l.assert_gpu_matches(want)
