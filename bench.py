@@ -64,7 +64,10 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="llama8b")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["ref_transfer_bench"],
+                    default="llama8b",
+                    help="ref_transfer_bench = the shapes of the reference's own "
+                         "benches/transfer_h2d.rs through the descriptor backends")
     ap.add_argument("--path", choices=["auto", "staged", "zerocopy"], default="auto")
     ap.add_argument("--layers", type=int, default=0, help="override the layer count")
     ap.add_argument("--slot-mb", type=int, default=0)
@@ -129,6 +132,9 @@ def main():
     path = {"auto": TransferPath.AUTO, "staged": TransferPath.STAGED,
             "zerocopy": TransferPath.ZEROCOPY}[args.path]
 
+    if args.workload == "ref_transfer_bench":
+        run_ref_transfer_bench(torch, np, args)
+        return
     w = WORKLOADS[args.workload]
     n_layers = args.layers or w["layers"]
     nb, seg, n = w["num_blocks"], w["seg"], w["n"]
@@ -458,6 +464,98 @@ def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_
             out["per_layer_ms_max"] = round(max(per_layer), 3)
             out["first_layer_ready_ms"] = round(done[0], 3)
     return out
+
+
+def run_ref_transfer_bench(torch, np, args):
+    """The reference's transfer bench (pegaflow-core/benches/transfer_h2d.rs:23-33,
+    62-109,301-339): 4 KiB fragments, device slots of 8 KiB, 1024..65536
+    fragments, layouts contiguous / strided_device / shuffled (xorshift64
+    Fisher-Yates), both directions, 3 warm-up and 20 timed iterations of
+    submit + synchronise, GiB/s = bytes * iters / seconds / 2^30 -- through
+    the two descriptor backends and, for comparison, the block-ID path."""
+    from pegaflow_amd.layout import KVCacheLayout
+    from pegaflow_amd.runtime import PinnedMemory, Stream
+    from pegaflow_amd.transfer import (BlockTransfer, KernelBackend, LayerBlocks, MemcpyBackend,
+                                       TransferPath, desc_array)
+    seg, stride_factor, warmup, iters = 4096, 2, 3, 20
+    counts = [1024, 4096, 16384, 65536]
+    dev = torch.device("cuda:0")
+    max_n = max(counts)
+    device_buf = torch.full((max_n * seg * stride_factor,), 0xA5, device=dev, dtype=torch.uint8)
+    host = PinnedMemory(max_n * seg)
+    idx = np.arange(max_n * seg, dtype=np.uint64)
+    host.as_numpy()[:] = ((idx * 31 + 7) & 0xFF).astype(np.uint8)
+    torch.cuda.synchronize()
+    stream = Stream()
+    backends = {"direct": MemcpyBackend(), "kernel": KernelBackend()}
+    xfer = BlockTransfer()
+
+    def shuffle(n):
+        mask, state = (1 << 64) - 1, 0x9E3779B97F4A7C15
+        perm = list(range(n))
+        for i in range(n - 1, 0, -1):
+            state ^= (state << 13) & mask
+            state ^= state >> 7
+            state ^= (state << 17) & mask
+            j = state % (i + 1)
+            perm[i], perm[j] = perm[j], perm[i]
+        return np.array(perm, dtype=np.uint64)
+
+    def gib_s(fn, nbytes):
+        for _ in range(warmup):
+            fn()
+            stream.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+            stream.synchronize()
+        return nbytes * iters / (time.perf_counter() - t0) / 2 ** 30
+
+    rows = []
+    for n in counts:
+        pos = np.arange(n, dtype=np.uint64)
+        layouts = {
+            # device slot of list position i; the host side is always dense in list order
+            "contiguous": pos,
+            "strided_device": pos * stride_factor,
+            "shuffled": shuffle(n) * stride_factor,
+        }
+        for lname, slot in layouts.items():
+            descs = desc_array(device_buf.data_ptr() + slot * seg, host.host_ptr + pos * seg,
+                               host.device_ptr + pos * seg, seg, 0, 1)
+            # the same bytes by block id: a contiguous layout of 4 KiB blocks
+            layout = KVCacheLayout(device_buf.data_ptr(), device_buf.numel(), max_n * stride_factor,
+                                   seg, 0, 1)
+            lb = [LayerBlocks(layout=layout, block_ids=slot.astype(np.uint32),
+                              host=(host.host_ptr,), host_device=(host.device_ptr,),
+                              host_len=(n * seg,), host_stride=seg)]
+            row = {"fragments": n, "layout": lname}
+            for bname, b in backends.items():
+                row[f"{bname}_d2h"] = round(gib_s(lambda: b.d2h(descs, stream), n * seg), 2)
+                row[f"{bname}_h2d"] = round(gib_s(lambda: b.h2d(descs, stream), n * seg), 2)
+            row["block_ids_d2h"] = round(gib_s(lambda: xfer.save(lb, stream, TransferPath.AUTO),
+                                               n * seg), 2)
+            row["block_ids_h2d"] = round(gib_s(lambda: xfer.load(lb, stream, TransferPath.AUTO),
+                                               n * seg), 2)
+            rows.append(row)
+            print("bench.py: " + json.dumps(row), file=sys.stderr, flush=True)
+    # byte check of the last case (shuffled, 65536 fragments, after its final load)
+    got = device_buf.view(max_n * stride_factor, seg)[torch.from_numpy(
+        layouts["shuffled"].astype(np.int64)).to(dev)].cpu().numpy().reshape(-1)
+    if not np.array_equal(got, host.as_numpy()[:max_n * seg]):
+        print("bench.py: device bytes differ from the host image", file=sys.stderr)
+        sys.exit(1)
+    headline = next(r for r in rows if r["fragments"] == 65536 and r["layout"] == "shuffled")
+    print(json.dumps({
+        "metric": "descriptor backends at the shapes of the reference's transfer bench "
+                  "(4 KiB fragments), GiB/s",
+        "value": headline["kernel_h2d"], "unit": "GiB/s", "n_gpus": 1, "steps": iters,
+        "warmup": warmup, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "benches/transfer_h2d.rs shapes: 4 KiB fragments, "
+                               "1024..65536 per batch, contiguous/strided/shuffled, "
+                               "value = kernel backend, shuffled, 65536 fragments, H2D"},
+        "table": rows}))
 
 
 def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, payload):

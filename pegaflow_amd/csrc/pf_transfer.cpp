@@ -146,22 +146,205 @@ int SlabPool::release_after(Slab* slab, hipStream_t s) {
 // MemcpyBackend
 // ---------------------------------------------------------------------------
 
-int MemcpyBackend::h2d(const CopyDesc* copies, uint64_t n, hipStream_t s) {
-  for (const MergedRange& m : merge(copies, n)) {
-    hipError_t e =
-        hipMemcpyHtoDAsync(reinterpret_cast<hipDeviceptr_t>(m.device), m.host, m.size, s);
-    if (e != hipSuccess) return fail_hip(e, "hipMemcpyHtoDAsync");
-  }
-  return PF_OK;
+MemcpyBackend::~MemcpyBackend() {
+  if (staging_) (void)hipFree(staging_);
+  (void)hipGetLastError();
 }
 
-int MemcpyBackend::d2h(const CopyDesc* copies, uint64_t n, hipStream_t s) {
-  for (const MergedRange& m : merge(copies, n)) {
-    hipError_t e =
-        hipMemcpyDtoHAsync(m.host, reinterpret_cast<hipDeviceptr_t>(m.device), m.size, s);
-    if (e != hipSuccess) return fail_hip(e, "hipMemcpyDtoHAsync");
+namespace {
+
+// A merged range that keeps what the staged forms need.
+struct Range {
+  uint64_t device;
+  uint8_t* host;
+  uint64_t host_device;
+  uint64_t size;
+  uint64_t host_allocation;
+};
+
+// The reference's merge rule (memcpy.rs:25-55), keeping the device-visible
+// host address and the host allocation of the descriptor that opened a range.
+std::vector<Range> merge_ranges(const CopyDesc* copies, uint64_t n) {
+  std::vector<Range> out;
+  out.reserve(n);
+  uint64_t run_first = 0;
+  for (uint64_t i = 0; i < n; ++i) {
+    const CopyDesc& c = copies[i];
+    if (!out.empty()) {
+      Range& run = out.back();
+      const CopyDesc& first = copies[run_first];
+      if (first.device_allocation == c.device_allocation &&
+          first.host_allocation == c.host_allocation && run.device + run.size == c.device &&
+          run.host + run.size == static_cast<uint8_t*>(c.host)) {
+        run.size += c.size;
+        continue;
+      }
+    }
+    run_first = i;
+    out.push_back({c.device, static_cast<uint8_t*>(c.host), c.host_device, c.size,
+                   c.host_allocation});
   }
-  return PF_OK;
+  return out;
+}
+
+hipError_t copy_range(const Range& r, bool host_is_src, hipStream_t s) {
+  return host_is_src
+             ? hipMemcpyHtoDAsync(reinterpret_cast<hipDeviceptr_t>(r.device), r.host, r.size, s)
+             : hipMemcpyDtoHAsync(r.host, reinterpret_cast<hipDeviceptr_t>(r.device), r.size, s);
+}
+
+}  // namespace
+
+int MemcpyBackend::submit(const CopyDesc* copies, uint64_t n, bool host_is_src, hipStream_t s) {
+  const std::vector<Range> ranges = merge_ranges(copies, n);
+  const char* what = host_is_src ? "hipMemcpyHtoDAsync" : "hipMemcpyDtoHAsync";
+  if (ranges.size() <= kFewRanges) {
+    for (const Range& r : ranges) {
+      hipError_t e = copy_range(r, host_is_src, s);
+      if (e != hipSuccess) return fail_hip(e, what);
+    }
+    return PF_OK;
+  }
+
+  // Sort the ranges into: large (own copy), members of a host-dense run
+  // (staged), isolated small ones.  A run is a maximal sequence, in list
+  // order per host allocation, of small ranges whose host sides follow one
+  // another without a gap.
+  struct Run {
+    uint8_t* host_begin;
+    uint64_t bytes;
+    std::vector<uint32_t> members;  // indices into `ranges`
+  };
+  std::vector<Run> runs;
+  std::vector<std::pair<uint64_t, size_t>> open;  // host allocation -> index of its open run
+  for (size_t i = 0; i < ranges.size(); ++i) {
+    const Range& r = ranges[i];
+    if (r.size >= kLargeRange || r.size == 0) continue;
+    size_t oi = 0;
+    while (oi < open.size() && open[oi].first != r.host_allocation) ++oi;
+    if (oi < open.size()) {
+      Run& run = runs[open[oi].second];
+      if (run.host_begin + run.bytes == r.host && run.bytes + r.size <= kStagingBytes) {
+        run.bytes += r.size;
+        run.members.push_back(static_cast<uint32_t>(i));
+        continue;
+      }
+      open[oi].second = runs.size();
+    } else {
+      if (open.size() >= 64) open.erase(open.begin());  // bound the linear search
+      open.emplace_back(r.host_allocation, runs.size());
+    }
+    runs.push_back(Run{r.host, r.size, {static_cast<uint32_t>(i)}});
+  }
+  std::vector<uint32_t> isolated;
+  bool isolated_mapped = true;
+  uint64_t staged_pieces = 0, max_staged_piece = 0, max_run_bytes = 0;
+  for (const Run& run : runs) {
+    if (run.members.size() == 1) {
+      isolated.push_back(run.members[0]);
+      isolated_mapped = isolated_mapped && ranges[run.members[0]].host_device != 0;
+    } else {
+      staged_pieces += run.members.size();
+      max_run_bytes = std::max(max_run_bytes, run.bytes + 16);
+      for (uint32_t m : run.members) max_staged_piece = std::max(max_staged_piece, ranges[m].size);
+    }
+  }
+  const bool isolated_by_kernel = isolated_mapped && isolated.size() > kFewRanges;
+
+  // Large ranges, and isolated ones that cannot use the kernel: one copy each.
+  for (const Range& r : ranges) {
+    if (r.size >= kLargeRange) {
+      hipError_t e = copy_range(r, host_is_src, s);
+      if (e != hipSuccess) return fail_hip(e, what);
+    }
+  }
+  if (!isolated_by_kernel) {
+    for (uint32_t i : isolated) {
+      hipError_t e = copy_range(ranges[i], host_is_src, s);
+      if (e != hipSuccess) return fail_hip(e, what);
+    }
+  }
+  const uint64_t table_rows = staged_pieces + (isolated_by_kernel ? isolated.size() : 0);
+  if (table_rows == 0) return PF_OK;
+  if (table_rows > 0x7FFFFFFFull) {
+    return fail(PF_ERR_INVALID_ARGUMENT, "descriptor batch of %llu exceeds the kernel limit",
+                static_cast<unsigned long long>(table_rows));
+  }
+
+  if (staged_pieces != 0 && staging_cap_ < max_run_bytes) {
+    // Grow-only; the stream order of the previous batch protects the old buffer.
+    if (staging_) {
+      PF_HIP(hipStreamSynchronize(s));
+      PF_HIP(hipFree(staging_));
+      staging_ = nullptr;
+      staging_cap_ = 0;
+    }
+    uint64_t cap = 1ull << 20;
+    while (cap < max_run_bytes) cap <<= 1;
+    PF_HIP(hipMalloc(&staging_, cap));
+    staging_cap_ = cap;
+  }
+
+  SlabPool::Slab* slab = nullptr;
+  int st = slabs_.acquire(table_rows * 3 * sizeof(uint64_t), &slab);
+  if (st != PF_OK) return st;
+  uint64_t* table = static_cast<uint64_t*>(slab->host);
+  const uint64_t* table_dev = static_cast<const uint64_t*>(slab->dev);
+  uint64_t row = 0;
+  // Rows of the isolated ranges first, then run by run.
+  uint64_t max_isolated = 0;
+  if (isolated_by_kernel) {
+    for (uint32_t i : isolated) {
+      const Range& r = ranges[i];
+      table[3 * row + 0] = host_is_src ? r.device : r.host_device;
+      table[3 * row + 1] = host_is_src ? r.host_device : r.device;
+      table[3 * row + 2] = r.size;
+      max_isolated = std::max(max_isolated, r.size);
+      ++row;
+    }
+  }
+  const uint64_t staging_base = reinterpret_cast<uint64_t>(staging_);
+  for (const Run& run : runs) {
+    if (run.members.size() == 1) continue;
+    // Keep the host side's alignment modulo 16 so aligned pieces stay on the
+    // 16-byte path of the kernel.
+    const uint64_t pad = reinterpret_cast<uint64_t>(run.host_begin) & 15ull;
+    for (uint32_t m : run.members) {
+      const Range& r = ranges[m];
+      const uint64_t in_staging = staging_base + pad + static_cast<uint64_t>(r.host - run.host_begin);
+      table[3 * row + 0] = host_is_src ? r.device : in_staging;
+      table[3 * row + 1] = host_is_src ? in_staging : r.device;
+      table[3 * row + 2] = r.size;
+      ++row;
+    }
+  }
+  PF_HIP(hipMemcpyAsync(slab->dev, slab->host, table_rows * 3 * sizeof(uint64_t),
+                        hipMemcpyHostToDevice, s));
+  row = 0;
+  if (isolated_by_kernel) {
+    st = launch_desc_copy(table_dev, isolated.size(), max_isolated, s);
+    if (st != PF_OK) return st;
+    row = isolated.size();
+  }
+  // One staging buffer, everything in stream order: pack, then copy (save),
+  // or copy, then unpack (load); the next run waits for the previous one.
+  for (const Run& run : runs) {
+    if (run.members.size() == 1) continue;
+    const uint64_t pad = reinterpret_cast<uint64_t>(run.host_begin) & 15ull;
+    uint8_t* in_staging = static_cast<uint8_t*>(staging_) + pad;
+    if (host_is_src) {
+      PF_HIP(hipMemcpyHtoDAsync(reinterpret_cast<hipDeviceptr_t>(in_staging), run.host_begin,
+                                run.bytes, s));
+    }
+    st = launch_desc_copy(table_dev + 3 * row, run.members.size(), max_staged_piece, s);
+    if (st != PF_OK) return st;
+    if (!host_is_src) {
+      PF_HIP(hipMemcpyDtoHAsync(run.host_begin, reinterpret_cast<hipDeviceptr_t>(in_staging),
+                                run.bytes, s));
+    }
+    row += run.members.size();
+  }
+  return slabs_.release_after(slab, s);
 }
 
 // ---------------------------------------------------------------------------

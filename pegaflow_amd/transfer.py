@@ -34,7 +34,21 @@ class CopyDesc:
     host_allocation: int = 0
 
 
-def _pack(copies: Sequence[CopyDesc]):
+def desc_array(device, host, host_device, size, device_allocation=0, host_allocation=0) -> np.ndarray:
+    """Descriptor batch as a uint64 array of shape (n, 6) in ``CopyDesc`` field
+    order (the memory layout of ``pf_copy_desc``); arguments broadcast."""
+    cols = np.broadcast_arrays(*[np.asarray(c, dtype=np.uint64) for c in
+                                 (device, host, host_device, size, device_allocation,
+                                  host_allocation)])
+    return np.ascontiguousarray(np.stack(cols, axis=-1).reshape(-1, 6))
+
+
+def _pack(copies):
+    if isinstance(copies, np.ndarray):
+        if copies.dtype != np.uint64 or copies.ndim != 2 or copies.shape[1] != 6 \
+                or not copies.flags.c_contiguous:
+            raise ValueError("descriptor array must be C-contiguous uint64 of shape (n, 6)")
+        return C.cast(copies.ctypes.data, C.POINTER(_lib.PfCopyDesc)), copies.shape[0]
     n = len(copies)
     arr = (_lib.PfCopyDesc * max(n, 1))()
     for i, c in enumerate(copies):
