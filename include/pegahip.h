@@ -277,7 +277,11 @@ typedef struct pf_xfer_config {
   uint64_t auto_staged_min_bytes;   /* 0 = default threshold for PF_PATH_AUTO */
   uint32_t tile_unroll;             /* zero-copy kernel: 16-byte loads in flight per lane:
                                        1,2,4,8; 0 = default (4) */
-  uint32_t reserved;
+  uint32_t copy_stream;             /* staged path: where the link copies run.
+                                       0 = default (side stream when a call has more than
+                                       one staged unit), 1 = a side stream of the engine (the
+                                       copy of one unit overlaps the gather of the next),
+                                       2 = the caller's stream (in order, no second queue) */
 } pf_xfer_config;
 
 typedef struct pf_xfer_s* pf_xfer_t;

@@ -360,7 +360,7 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
   }
 
   PF_HIP(hipMemcpyAsync(slab->dev, slab->host, slab_bytes, hipMemcpyHostToDevice, s));
-  hipStream_t side = timing_ ? s : side_;
+  hipStream_t side = use_side_stream(chunks.size()) ? side_ : s;
   if (side != s) {
     PF_HIP(hipEventRecord(fork_, s));
     PF_HIP(hipStreamWaitEvent(side, fork_, 0));
@@ -586,7 +586,9 @@ int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool s
   PF_HIP(hipMemcpyAsync(slab->dev, slab->host, slab_bytes, hipMemcpyHostToDevice, s));
   // With kernel timing on, the DMA copies run on the caller's stream too, so
   // that every timed kernel executes alone (a measurement mode: no overlap).
-  hipStream_t side = timing_ ? s : side_;
+  size_t staged_units = 0;
+  for (const UnitRef& r : unit_refs) staged_units += plans[r.plan].staged ? 1 : 0;
+  hipStream_t side = use_side_stream(staged_units) ? side_ : s;
   bool side_used = false;
   auto fork_side = [&]() -> int {
     if (side_used || side == s) return PF_OK;

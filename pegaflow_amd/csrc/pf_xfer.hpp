@@ -25,7 +25,16 @@ struct LayerPlan;
 // 512 MiB 56.7 GB/s of a 57.3 GB/s link), so a slot holds a whole layer.
 constexpr uint64_t kDefaultSlotBytes = 512ull << 20;
 constexpr uint32_t kDefaultSlots = 2;
-constexpr uint64_t kDefaultAutoStagedMin = 4ull << 20;
+// PF_PATH_AUTO stages a dense layer (or a page-packed call) from this size on.
+// Measured on MI355X, one call then a synchronise, nothing else running: the
+// zero-copy kernel saves faster than the staged path up to 32 MiB (4 MiB:
+// 41.0 against 33.9 GB/s; 32 MiB: 52.3 against 52.1) and slower from 64 MiB
+// on (53.2 against 53.9; 128 MiB: 54.0 against 55.1); many small layers in
+// one call favour it even more (8 x 4 MiB: 50.3 against 37.3).  Loads are
+// faster zero-copy at every size (128 MiB: 56.9 against 55.1 GB/s), but a
+// long zero-copy transfer slows kernels that run beside it, which a staged
+// one does not, so large loads are staged as well.
+constexpr uint64_t kDefaultAutoStagedMin = 64ull << 20;
 constexpr int kDefaultUnroll = 4;
 // Zero-copy launches are capped to a few workgroups: the host link, not the
 // GPU, is the bound, and fewer in-flight requests use it better.  Measured on
@@ -42,6 +51,7 @@ class Xfer {
       if (cfg->zerocopy_max_workgroups) zc_max_wg_ = cfg->zerocopy_max_workgroups;
       if (cfg->auto_staged_min_bytes) auto_min_ = cfg->auto_staged_min_bytes;
       if (cfg->tile_unroll) unroll_ = static_cast<int>(cfg->tile_unroll);
+      if (cfg->copy_stream) copy_stream_ = cfg->copy_stream;
     }
   }
 
@@ -158,6 +168,18 @@ class Xfer {
   int last_path_ = 0;
 
   bool timing_ = false;
+  uint32_t copy_stream_ = 0;  // 0 = by unit count, 1 = side stream, 2 = caller's stream
+  // A second stream pays off only when the copy of one unit can overlap the
+  // gather of the next.  Measured on MI355X (Llama layer shape, one call then
+  // a synchronise): a single unit of 4 / 16 / 64 / 312 MiB moves at 33.6 /
+  // 48.7 / 54.3 / 56.0 GB/s in order on the caller's stream against 24.8 /
+  // 44.4 / 52.8 / 55.6 GB/s with the hand-off to a side stream; from two
+  // units on the side stream wins (56.6 against 55.8 GB/s at 32 units).
+  bool use_side_stream(size_t staged_units) const {
+    if (timing_ || copy_stream_ == 2) return false;
+    if (copy_stream_ == 1) return true;
+    return staged_units > 1;
+  }
   std::vector<std::pair<hipEvent_t, hipEvent_t>> timing_pool_;
   size_t timing_used_ = 0;
 };

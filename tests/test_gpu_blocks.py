@@ -30,7 +30,7 @@ def stream(gpu):
 def xfer(gpu):
     # Small staging slots so that modest test sizes already span several
     # units and reuse slots.
-    x = BlockTransfer(staging_slot_bytes=1 << 20, staging_slots=2)
+    x = BlockTransfer(staging_slot_bytes=1 << 20, staging_slots=2, auto_staged_min_bytes=4 << 20)
     yield x
     x.close()
 
