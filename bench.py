@@ -365,6 +365,12 @@ def main():
         duplex = run_duplex(xfer, save_layers, load_layers, stream, path, payload, args)
 
     # ---- the same workload through the save / query / load engine -----------
+    # The bench's own engine and stream are released first: a process gets few
+    # hardware queues (GPU_MAX_HW_QUEUES, 4 by default) and streams beyond that
+    # number share them, which would serialise the pool's two workers.
+    xfer.close()
+    stream.close()
+    pool.close()
     engine = None
     if not args.no_engine:
         engine = run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, payload)
@@ -568,7 +574,7 @@ def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, pa
     nb, seg, n = w["num_blocks"], w["seg"], w["n"]
     nseg = 2 if w["split"] else 1
     n_layers = len(names)
-    eng = PegaEngine(pool_size=int(payload * 1.2) + (256 << 20))
+    eng = PegaEngine(pool_size=int(payload * 2.3) + (256 << 20))
     kv = nb * seg if nseg == 2 else 0
     for inst, caches in (("bench-src", src_cache), ("bench-dst", dst_cache)):
         eng.register_context_layer_batch(
@@ -613,6 +619,43 @@ def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, pa
         if not torch.equal(d_[:, lid], s_[:, sid]):
             print(f"bench.py: engine round trip differs on layer {li}", file=sys.stderr)
             sys.exit(1)
+    # A save and a load at once (the pool's two workers), from two threads.
+    import threading
+    try:
+        hashes_a = [b"A" + int(i).to_bytes(4, "little") + bytes(27) for i in range(n)]
+        hashes_b = [b"B" + int(i).to_bytes(4, "little") + bytes(27) for i in range(n)]
+        packed_a = PackedSaves([LayerSave(nm, save_ids, hashes_a) for nm in names])
+        packed_b = PackedSaves([LayerSave(nm, save_ids, hashes_b) for nm in names])
+        eng.batch_save_kv_blocks("bench-src", 0, 0, 0, packed_a)
+        hits, lease = eng.query_prefix("bench-dst", hashes_a)
+        times = {}
+
+        def do_save():
+            t0 = time.perf_counter()
+            eng.batch_save_kv_blocks("bench-src", 0, 0, 0, packed_b)
+            times["save"] = time.perf_counter() - t0
+
+        def do_load():
+            t0 = time.perf_counter()
+            task = eng.batch_load_kv_blocks_multi_layer("bench-dst", 0, 0, [names], lease,
+                                                        [load_ids.tolist()])
+            task.wait()
+            times["load"] = time.perf_counter() - t0
+            task.close()
+
+        threads = [threading.Thread(target=do_save), threading.Thread(target=do_load)]
+        t0 = time.perf_counter()
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        span = time.perf_counter() - t0
+        out["concurrent_save_and_load"] = {
+            "save_gbps": round(payload / times["save"] / 1e9, 2),
+            "load_gbps": round(payload / times["load"] / 1e9, 2),
+            "aggregate_gbps": round(2 * payload / span / 1e9, 2)}
+    except Exception as exc:  # pool too small for two images, etc.: report, do not fail the bench
+        out["concurrent_save_and_load"] = {"error": str(exc)}
     out["save_gbps"] = round(payload / min(save_s) / 1e9, 2)
     out["load_gbps"] = round(payload / min(load_s) / 1e9, 2)
     out["save_gbps_all"] = [round(payload / t / 1e9, 2) for t in save_s]
@@ -625,36 +668,41 @@ def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, pa
 
 def run_duplex(xfer, save_layers, load_layers, stream, path, payload, args):
     """A save and a load in flight together, each with its own stream and
-    staging slots, as the two worker threads of one GPU issue them.  (The
-    load reads the host image while the save rewrites it with the same bytes;
-    only the rates are used.)"""
+    engine, as the two worker threads of one GPU issue them.  (The load reads
+    the host image while the save rewrites it with the same bytes; only the
+    rates are used.)  Two forms: link copies on each engine's side stream (the
+    stand-alone default) and on the callers' streams (what the worker pool
+    configures, so that the two directions never share a hardware queue)."""
     from pegaflow_amd.runtime import Event, Stream
     from pegaflow_amd.transfer import BlockTransfer
-    xfer2 = BlockTransfer(staging_slot_bytes=args.slot_mb << 20, staging_slots=args.slots,
-                          tile_unroll=args.unroll, zerocopy_max_workgroups=args.zc_max_wg)
-    stream2 = Stream()
+    out = {}
     ev = [Event(timing=True) for _ in range(4)]
-    xfer2.load(load_layers, stream2, path)   # allocate its staging
-    stream2.synchronize()
-    stream.synchronize()
-    best = None
-    for _ in range(2):
-        ev[0].record(stream)
-        ev[2].record(stream2)
-        xfer.save(save_layers, stream, path)
-        xfer2.load(load_layers, stream2, path)
-        ev[1].record(stream)
-        ev[3].record(stream2)
-        ev[1].synchronize()
-        ev[3].synchronize()
-        save_ms, load_ms = ev[0].elapsed_ms(ev[1]), ev[2].elapsed_ms(ev[3])
-        span_ms = max(ev[0].elapsed_ms(ev[1]), ev[0].elapsed_ms(ev[3]))
-        best = {"save_gbps": round(payload / save_ms / 1e6, 2),
-                "load_gbps": round(payload / load_ms / 1e6, 2),
-                "aggregate_gbps": round(2 * payload / span_ms / 1e6, 2)}
-    xfer2.close()
-    stream2.close()
-    return best
+    for label, mode in (("side_stream_copies", 1), ("in_order_copies", 2)):
+        xa, xb = (BlockTransfer(staging_slot_bytes=args.slot_mb << 20, staging_slots=args.slots,
+                                tile_unroll=args.unroll, zerocopy_max_workgroups=args.zc_max_wg,
+                                copy_stream=mode) for _ in range(2))
+        sa, sb = Stream(), Stream()
+        xa.save(save_layers, sa, path)   # allocate staging
+        xb.load(load_layers, sb, path)
+        sa.synchronize()
+        sb.synchronize()
+        for _ in range(2):
+            ev[0].record(sa)
+            ev[2].record(sb)
+            xa.save(save_layers, sa, path)
+            xb.load(load_layers, sb, path)
+            ev[1].record(sa)
+            ev[3].record(sb)
+            ev[1].synchronize()
+            ev[3].synchronize()
+            save_ms, load_ms = ev[0].elapsed_ms(ev[1]), ev[2].elapsed_ms(ev[3])
+            span_ms = max(ev[0].elapsed_ms(ev[1]), ev[0].elapsed_ms(ev[3]))
+            out[label] = {"save_gbps": round(payload / save_ms / 1e6, 2),
+                          "load_gbps": round(payload / load_ms / 1e6, 2),
+                          "aggregate_gbps": round(2 * payload / span_ms / 1e6, 2)}
+        for o in (xa, xb, sa, sb):
+            o.close()
+    return out
 
 
 def run_cpu_baseline(np, w, save_ids, load_ids, seconds, seed):
