@@ -186,6 +186,7 @@ Engine::~Engine() {
   leases_.clear();
   inflight_.clear();
   sealed_.clear();
+  lru_.clear();
 }
 
 std::shared_ptr<InstanceContext> Engine::get_instance(const std::string& id, std::string* err) {
@@ -310,21 +311,20 @@ int Engine::unregister_instance(const std::string& instance_id, std::string* err
   return PF_OK;
 }
 
+void Engine::seal_insert(const BlockKey& key, std::shared_ptr<SealedBlock> block) {
+  // mu_ held by the caller; the key is not present.
+  lru_.push_back(key);
+  sealed_[key] = SealedEntry{std::move(block), std::prev(lru_.end())};
+}
+
 bool Engine::evict_one() {
-  // mu_ held by the caller.  Oldest first; blocks that are leased or being
-  // loaded (someone else holds a reference) stay.
-  for (size_t i = 0; i < sealed_order_.size();) {
-    auto sit = sealed_.find(sealed_order_[i]);
-    if (sit == sealed_.end()) {
-      sealed_order_.erase(sealed_order_.begin() + static_cast<std::ptrdiff_t>(i));
-      continue;
-    }
-    if (sit->second.use_count() > 1) {
-      ++i;
-      continue;
-    }
-    sealed_.erase(sit);
-    sealed_order_.erase(sealed_order_.begin() + static_cast<std::ptrdiff_t>(i));
+  // mu_ held by the caller.  Least recently used first; blocks that are
+  // leased or being loaded (someone else holds a reference) stay.
+  for (auto it = lru_.begin(); it != lru_.end(); ++it) {
+    auto sit = sealed_.find(*it);
+    if (sit != sealed_.end() && sit->second.block.use_count() > 1) continue;
+    if (sit != sealed_.end()) sealed_.erase(sit);
+    lru_.erase(it);
     return true;
   }
   return false;
@@ -684,8 +684,7 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
   {
     std::lock_guard<std::mutex> lock(mu_);
     auto seal = [&](const BlockKey& key, InflightBlock* b) {
-      sealed_[key] = b->seal();
-      sealed_order_.push_back(key);
+      seal_insert(key, b->seal());
     };
     if (page_first) {
       const SaveList& l = lists[ctxs[0].list];
@@ -753,7 +752,8 @@ int Engine::query_prefix(const std::string& instance_id, const std::vector<std::
   for (const std::string& h : hashes) {
     auto it = sealed_.find(BlockKey{instance->ns(), h});
     if (it == sealed_.end()) break;
-    lease.blocks.push_back(it->second);
+    lease.blocks.push_back(it->second.block);
+    lru_.splice(lru_.end(), lru_, it->second.pos);  // most recently used
   }
   *out_hits = lease.blocks.size();
   *out_lease = 0;

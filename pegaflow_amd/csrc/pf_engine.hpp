@@ -9,6 +9,7 @@
 
 #include <cstdint>
 #include <future>
+#include <list>
 #include <map>
 #include <memory>
 #include <mutex>
@@ -146,8 +147,16 @@ class Engine {
   std::mutex mu_;  // instances, store, leases
   std::map<std::string, std::shared_ptr<InstanceContext>> instances_;
   std::map<BlockKey, InflightBlock> inflight_;
-  std::map<BlockKey, std::shared_ptr<SealedBlock>> sealed_;
-  std::vector<BlockKey> sealed_order_;  // insertion order, for oldest-first eviction
+  // The read cache: sealed blocks in least-recently-used order (front = next
+  // to go; a prefix query moves its hits to the back), storage/mod.rs:482-554
+  // and storage/read_cache.rs of the reference without its admission policy.
+  struct SealedEntry {
+    std::shared_ptr<SealedBlock> block;
+    std::list<BlockKey>::iterator pos;
+  };
+  std::map<BlockKey, SealedEntry> sealed_;
+  std::list<BlockKey> lru_;
+  void seal_insert(const BlockKey& key, std::shared_ptr<SealedBlock> block);
   struct Lease {
     std::string instance_id;
     std::vector<std::shared_ptr<SealedBlock>> blocks;

@@ -232,6 +232,28 @@ def test_pool_pressure_evicts_oldest_unleased_blocks(gpu):
     e.close()
 
 
+def test_eviction_is_least_recently_used(gpu):
+    """A prefix query makes its hits the most recently used blocks
+    (storage/read_cache.rs): the batch that was not touched goes first."""
+    e = PegaEngine(pool_size=64 * 1024)
+    layer = Layer("layer_0", 64, 4096)
+    register(e, "lru", [layer])
+    first, second, third = (make_block_hashes(8, s) for s in (1, 2, 3))
+    e.batch_save_kv_blocks("lru", 0, 0, 0, [LayerSave("layer_0", list(range(8)), first)])
+    e.batch_save_kv_blocks("lru", 0, 0, 0, [LayerSave("layer_0", list(range(8, 16)), second)])
+    hits, lease = e.query_prefix("lru", first)      # touch the older batch ...
+    assert hits == 8
+    e.release_query_lease(lease)                    # ... without keeping it pinned
+    e.batch_save_kv_blocks("lru", 0, 0, 0, [LayerSave("layer_0", list(range(16, 24)), third)])
+    assert e.query_prefix("lru", second)[0] == 0    # the untouched batch was evicted
+    h1, l1 = e.query_prefix("lru", first)
+    h3, l3 = e.query_prefix("lru", third)
+    assert (h1, h3) == (8, 8)
+    e.release_query_lease(l1)
+    e.release_query_lease(l3)
+    e.close()
+
+
 def test_blockwise_alloc_and_odd_segment_size(gpu):
     """--blockwise-alloc gives every block its own K and V allocation (the
     worker then falls back to per-fragment descriptors); 1000-byte segments in
