@@ -38,9 +38,9 @@ HBM_PEAK_GBPS = 8000.0      # MI355X published HBM3E bandwidth
 # WRITE_SIZE runs of this script: KiB per dispatch, scaled by what a plain copy
 # of exactly 1 GiB reads on the same counters (x2.000 and x1.000).
 MEASURED_TRAFFIC_STAGED = {
-    "llama8b": int((160184.2 * 2.000 + 320034.9 * 1.000) * 1024),
-    "llama70b_fp8": int((131358.9 * 2.000 + 262171.2 * 1.000) * 1024),
-    "dsv3_mla": int((249956.5 * 2.000 + 499880.8 * 1.000) * 1024),
+    "llama8b": int((160338.3 * 2.000 + 320000.0 * 1.000) * 1024),
+    "llama70b_fp8": int((131614.6 * 2.000 + 262144.0 * 1.000) * 1024),
+    "dsv3_mla": int((249963.3 * 2.000 + 499712.0 * 1.000) * 1024),
 }
 
 WORKLOADS = {
@@ -74,6 +74,9 @@ def parse_args():
     ap.add_argument("--slots", type=int, default=0)
     ap.add_argument("--unroll", type=int, default=0)
     ap.add_argument("--zc-max-wg", type=int, default=0)
+    ap.add_argument("--copy-stream", type=int, default=0, choices=[0, 1, 2],
+                    help="staged path: 0 default, 1 link copies on a side stream, 2 in order on "
+                         "the caller's stream (kernels then never overlap a copy)")
     ap.add_argument("--no-overlap", action="store_true", help="skip the GEMM-overlap section")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-engine", action="store_true", help="skip the save/query/load engine section")
@@ -209,7 +212,8 @@ def main():
     save_layers = layers_for(src_cache, save_ids)
     load_layers = layers_for(dst_cache, load_ids)
     xfer = BlockTransfer(staging_slot_bytes=args.slot_mb << 20, staging_slots=args.slots,
-                         tile_unroll=args.unroll, zerocopy_max_workgroups=args.zc_max_wg)
+                         tile_unroll=args.unroll, zerocopy_max_workgroups=args.zc_max_wg,
+                         copy_stream=args.copy_stream)
     stream = Stream()
     ev = [Event(timing=True) for _ in range(4)]
 
@@ -398,7 +402,8 @@ def main():
                    "layers": n_layers, "blocks": n, "fragment_bytes": seg,
                    "payload_bytes_per_direction": payload, "path": used_path,
                    "host_layout": "page-first" if w["page_first"] else "layer-first",
-                   "staging_slot_mb": args.slot_mb or 512, "staging_slots": args.slots or 2},
+                   "staging_slot_mb": args.slot_mb or 512, "staging_slots": args.slots or 2,
+                   "copy_stream": args.copy_stream},
         "save_gbps": round(save_gbps, 3),
         "step_save_load_ms": step_times[:16],
         "settle_steps": settle_steps,
