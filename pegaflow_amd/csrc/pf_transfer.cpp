@@ -195,7 +195,25 @@ hipError_t copy_range(const Range& r, bool host_is_src, hipStream_t s) {
 
 }  // namespace
 
+namespace {
+// A batch that failed half way may have left work on the stream that reads
+// the table slab or the staging buffer: drain it, keeping the message.
+int drained(int st, hipStream_t s) {
+  if (st == PF_OK) return st;
+  const std::string message = last_error();
+  (void)hipStreamSynchronize(s);
+  (void)hipGetLastError();
+  last_error() = message;
+  return st;
+}
+}  // namespace
+
 int MemcpyBackend::submit(const CopyDesc* copies, uint64_t n, bool host_is_src, hipStream_t s) {
+  return drained(submit_impl(copies, n, host_is_src, s), s);
+}
+
+int MemcpyBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_src,
+                               hipStream_t s) {
   const std::vector<Range> ranges = merge_ranges(copies, n);
   const char* what = host_is_src ? "hipMemcpyHtoDAsync" : "hipMemcpyDtoHAsync";
   if (ranges.size() <= kFewRanges) {
@@ -352,6 +370,11 @@ int MemcpyBackend::submit(const CopyDesc* copies, uint64_t n, bool host_is_src, 
 // ---------------------------------------------------------------------------
 
 int KernelBackend::submit(const CopyDesc* copies, uint64_t n, bool host_is_src, hipStream_t s) {
+  return drained(submit_impl(copies, n, host_is_src, s), s);
+}
+
+int KernelBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_src,
+                               hipStream_t s) {
   if (n == 0) return PF_OK;  // kernel.rs:85-87
   if (n > 0x7FFFFFFFull) {
     return fail(PF_ERR_INVALID_ARGUMENT, "descriptor batch of %llu exceeds the kernel limit",

@@ -86,6 +86,7 @@ class MemcpyBackend : public TransferBackend {
 
  private:
   int submit(const CopyDesc* copies, uint64_t n, bool host_is_src, hipStream_t s);
+  int submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_src, hipStream_t s);
   SlabPool slabs_;
   void* staging_ = nullptr;
   uint64_t staging_cap_ = 0;
@@ -105,6 +106,7 @@ class KernelBackend : public TransferBackend {
 
  private:
   int submit(const CopyDesc* copies, uint64_t n, bool host_is_src, hipStream_t s);
+  int submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_src, hipStream_t s);
   SlabPool slabs_;
 };
 

@@ -359,6 +359,7 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
     }
   }
 
+  began_ = true;
   PF_HIP(hipMemcpyAsync(slab->dev, slab->host, slab_bytes, hipMemcpyHostToDevice, s));
   hipStream_t side = use_side_stream(chunks.size()) ? side_ : s;
   if (side != s) {
@@ -410,6 +411,23 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
 
 int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save,
               hipStream_t s) {
+  began_ = false;
+  const int st = run_impl(layers, n_layers, path, save, s);
+  if (st != PF_OK && began_) {
+    // Something was already enqueued, possibly on the side stream, which the
+    // caller's synchronise of `s` would not cover: drain both before the
+    // caller learns of the failure and releases its buffers.
+    const std::string message = last_error();
+    (void)hipStreamSynchronize(side_);
+    (void)hipStreamSynchronize(s);
+    (void)hipGetLastError();
+    last_error() = message;
+  }
+  return st;
+}
+
+int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save,
+                   hipStream_t s) {
   timing_used_ = 0;
   if (n_layers == 0) return PF_OK;
   if (!layers) return fail(PF_ERR_INVALID_ARGUMENT, "layers must not be null");
@@ -583,6 +601,7 @@ int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool s
   next_slot_ = slot_cursor;
 
   // ---- 4. enqueue ---------------------------------------------------------
+  began_ = true;
   PF_HIP(hipMemcpyAsync(slab->dev, slab->host, slab_bytes, hipMemcpyHostToDevice, s));
   // With kernel timing on, the DMA copies run on the caller's stream too, so
   // that every timed kernel executes alone (a measurement mode: no overlap).

@@ -105,6 +105,8 @@ class Xfer {
     return x;
   }
   int run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save, hipStream_t s);
+  int run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save,
+               hipStream_t s);
   int save(const pf_layer_blocks* layers, uint64_t n_layers, int path, hipStream_t s) {
     return run(layers, n_layers, path, true, s);
   }
@@ -168,6 +170,7 @@ class Xfer {
   int last_path_ = 0;
 
   bool timing_ = false;
+  bool began_ = false;  // the current call has enqueued work
   uint32_t copy_stream_ = 0;  // 0 = by unit count, 1 = side stream, 2 = caller's stream
   // A second stream pays off only when the copy of one unit can overlap the
   // gather of the next.  Measured on MI355X (Llama layer shape, one call then
