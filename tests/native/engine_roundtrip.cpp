@@ -1,0 +1,65 @@
+// A native consumer of the C ABI: the save -> query -> load cycle of
+// pegaflow-core's engine tests (tests/engine_basic.rs, hybrid_groups.rs) driven
+// from C++ with nothing but include/pegahip.h and the HIP runtime, over both
+// transfer modes, both worker forms (block ids / descriptors), blockwise
+// allocation, page-first pages small (zero-copy) and large (whole-page
+// staging), and a 20-layer task whose load is converted in two parts.
+// Built by `make -C pegaflow_amd/csrc native-tests`; run by
+// tests/test_gpu_native.py.  Exit status 0 and a last line "all ok" = pass.
+#include "../../include/pegahip.h"
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+#define OK(x) do{int st_=(x); if(st_!=0){printf("FAIL line %d: %s -> %d %s\n",__LINE__,#x,st_,pf_last_error()); return 1;}}while(0)
+int run(bool page_first,int mode,bool desc,bool blockwise,int nseg,int L,uint64_t nb,uint64_t seg,uint64_t n,uint64_t pool_mb){
+  printf("case page_first=%d mode=%d desc=%d blockwise=%d nseg=%d L=%d nb=%llu seg=%llu n=%llu\n",page_first,mode,desc,blockwise,nseg,L,(unsigned long long)nb,(unsigned long long)seg,(unsigned long long)n); fflush(stdout);
+  pf_engine_config cfg; memset(&cfg,0,sizeof cfg); cfg.pool_size=pool_mb<<20; cfg.pool_shards=1; cfg.blockwise_alloc=blockwise; cfg.use_descriptor_backends=desc;
+  pf_engine_t e=nullptr; OK(pf_engine_create(&cfg,&e));
+  const uint64_t layer_bytes=nseg*nb*seg;
+  std::vector<void*> src(L),dst(L); std::vector<std::vector<uint8_t>> host(L);
+  std::mt19937_64 rng(7);
+  for(int l=0;l<L;l++){ if(hipMalloc(&src[l],layer_bytes)||hipMalloc(&dst[l],layer_bytes)) return 2; host[l].resize(layer_bytes); for(auto& b:host[l]) b=(uint8_t)rng(); (void)hipMemcpy(src[l],host[l].data(),layer_bytes,hipMemcpyHostToDevice); (void)hipMemset(dst[l],0,layer_bytes);} 
+  std::vector<std::string> names(L); std::vector<const char*> cn(L); for(int l=0;l<L;l++){ names[l]="model.layers."+std::to_string(l)+".attn"; cn[l]=names[l].c_str(); }
+  std::vector<uint64_t> sz(L,layer_bytes),nbs(L,nb),bpb(L,seg),kvs(L,nseg==2?nb*seg:0),sg(L,nseg);
+  for(int which=0;which<2;which++){
+    std::vector<uint64_t> ptrs(L); for(int l=0;l<L;l++) ptrs[l]=(uint64_t)(which?dst[l]:src[l]);
+    OK(pf_engine_register_context_layer_batch(e,which?"dst":"src","ns",0,0,0,1,1,L,cn.data(),ptrs.data(),sz.data(),nbs.data(),bpb.data(),kvs.data(),sg.data(),nullptr,nullptr,mode,page_first));
+  }
+  std::vector<uint64_t> ids(nb); for(uint64_t i=0;i<nb;i++) ids[i]=i; std::shuffle(ids.begin(),ids.end(),rng); ids.resize(n);
+  std::vector<int64_t> dids(nb); for(uint64_t i=0;i<nb;i++) dids[i]=i; std::shuffle(dids.begin(),dids.end(),rng); dids.resize(n); if(n>3) dids[1]=-1;
+  for(int rep=0;rep<3;rep++){
+    std::vector<std::vector<uint8_t>> hs(n); std::vector<const uint8_t*> hp(n); std::vector<uint32_t> hl(n);
+    for(uint64_t i=0;i<n;i++){ hs[i].resize(8+ (i%3)); hs[i][0]=rep; memcpy(&hs[i][1],&i,4); hp[i]=hs[i].data(); hl[i]=hs[i].size(); }
+    std::vector<pf_layer_save> saves(L); for(int l=0;l<L;l++){ saves[l]={cn[l],ids.data(),hp.data(),hl.data(),n}; }
+    OK(pf_engine_batch_save(e,"src",0,0,0,saves.data(),L));
+    OK(pf_engine_batch_save(e,"src",0,0,0,saves.data(),L));  // dedupe
+    uint64_t hits=0,lease=0; OK(pf_engine_query_prefix(e,"dst",hp.data(),hl.data(),n,&hits,&lease)); if(hits!=n){printf("hits %llu\n",(unsigned long long)hits); return 3;}
+    const char* const* groups[1]={cn.data()}; uint64_t gs[1]={(uint64_t)L}; const int64_t* dd[1]={dids.data()};
+    pf_task_t t=nullptr; OK(pf_engine_batch_load(e,"dst",0,0,1,groups,gs,lease,dd,n,nullptr,&t));
+    pf_task_result r; OK(pf_task_wait(t,-1,&r)); OK(pf_task_destroy(t));
+    // verify
+    for(int l=0;l<L;l++){ std::vector<uint8_t> got(layer_bytes); (void)hipMemcpy(got.data(),dst[l],layer_bytes,hipMemcpyDeviceToHost);
+      for(uint64_t i=0;i<n;i++){ if(dids[i]<0) continue; for(int s=0;s<nseg;s++){ if(memcmp(&got[s*nb*seg+dids[i]*seg],&host[l][s*nb*seg+ids[i]*seg],seg)){ printf("MISMATCH layer %d pos %llu\n",l,(unsigned long long)i); return 4;} } } }
+    if(rep==1) pf_engine_evict_all(e);
+  }
+  OK(pf_engine_unregister_instance(e,"src")); OK(pf_engine_unregister_instance(e,"dst"));
+  OK(pf_engine_destroy(e));
+  for(int l=0;l<L;l++){ (void)hipFree(src[l]); (void)hipFree(dst[l]); }
+  return 0;
+}
+int main(){
+  int rc=0;
+  rc|=run(false,0,false,false,2,4,256,4096,100,64);
+  rc|=run(false,1,false,false,2,4,256,4096,100,64);
+  rc|=run(false,0,true,false,2,4,256,4096,100,64);
+  rc|=run(false,1,true,false,1,3,128,1000,50,64);
+  rc|=run(false,0,false,true,2,3,128,4096,40,64);
+  rc|=run(true,1,false,false,1,5,128,8192,60,64);
+  rc|=run(true,0,false,false,1,5,2048,65536,1500,1200);   // page-first, whole-page staging (>64 MiB)
+  rc|=run(false,0,false,false,2,20,4096,32768,2500,4000); // staged, two-part conversion on load
+  printf(rc?"FAILED\n":"all ok\n"); return rc;
+}
