@@ -419,9 +419,15 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
     bool per_block = false;
     for (const auto& l : task->layers) per_block |= !l.blocks.empty();
     size_t first_part = n_layers ? n_layers : 1;
-    if (xfer && per_block && n_layers >= 16) first_part = n_layers / 16 < 2 ? 2 : n_layers / 16;
+    // (Descriptor backends build one descriptor per fragment whatever the form.)
+    if ((!xfer || per_block) && n_layers >= 16) first_part = n_layers / 16 < 2 ? 2 : n_layers / 16;
     for (size_t begin = 0; begin < n_layers && st == PF_OK;) {
-      const size_t end = begin == 0 ? (first_part < n_layers ? first_part : n_layers) : n_layers;
+      // Block-ID form: the rest goes in one call (a call boundary drains the
+      // engine's copy pipeline).  Descriptor form: every part is that small;
+      // its copies are in order on one stream, so boundaries cost nothing.
+      const size_t end = (begin == 0 || !xfer)
+                             ? (begin + first_part < n_layers ? begin + first_part : n_layers)
+                             : n_layers;
       bool done_fast = false;
       if (xfer) {
         BlockForm form;
