@@ -9,13 +9,21 @@ Importing submodules that touch the library raises if it has not been built.
 
 from .connector import (  # noqa: F401
     KVCacheRegistrationInfo,
+    assemble_layer_saves,
+    block_shard,
     infer_kv_cache_registration,
+    register_kv_caches,
+    registration_tensor,
     resolve_transfer_backend,
 )
 
 __all__ = [
     "KVCacheRegistrationInfo",
+    "assemble_layer_saves",
+    "block_shard",
     "infer_kv_cache_registration",
+    "register_kv_caches",
+    "registration_tensor",
     "resolve_transfer_backend",
 ]
 __version__ = "0.1.0"

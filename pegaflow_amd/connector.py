@@ -108,3 +108,126 @@ def resolve_transfer_backend(is_mla: bool, override: str | None) -> str:
             f"Unsupported pegaflow.transfer_backend {override!r}; expected one of: {allowed}"
         )
     return normalized
+
+
+# ---------------------------------------------------------------------------
+# Worker-side callers of the path (python/pegaflow/connector/worker.py): how a
+# vLLM worker turns its KV tensors into a registration and its save intents
+# into per-layer block lists.  In-process forms over PegaEngine; the
+# reference sends the same values over gRPC with CUDA-IPC handles.
+# ---------------------------------------------------------------------------
+
+def registration_tensor(kv_cache):
+    """The tensor that represents a layer's cache (worker.py:154-176): the
+    tensor itself, or the first of a sequence of recurrent-state tensors that
+    share one allocation, block count and page stride."""
+    if not isinstance(kv_cache, (tuple, list)):
+        return kv_cache
+    states = tuple(kv_cache)
+    if not states or not all(hasattr(s, "untyped_storage") for s in states):
+        raise TypeError("KV cache must be a tensor or a non-empty sequence of state tensors")
+    first = states[0]
+    if first.storage_offset() != 0:
+        raise RuntimeError("the first recurrent-state tensor must start at storage offset zero")
+    storage_ptr = first.untyped_storage().data_ptr()
+    num_blocks = first.shape[0]
+    page_bytes = first.stride(0) * first.element_size()
+    for state in states:
+        if state.untyped_storage().data_ptr() != storage_ptr:
+            raise RuntimeError("recurrent-state tensors must share one CUDA allocation")
+        if state.shape[0] != num_blocks:
+            raise RuntimeError("recurrent-state tensors must have the same block count")
+        if state.stride(0) * state.element_size() != page_bytes:
+            raise RuntimeError("recurrent-state tensors must have one common page stride")
+    return first
+
+
+def register_kv_caches(engine, instance_id: str, namespace: str, device_id: int, kv_caches: dict,
+                       block_size: int, *, is_mla: bool = False, tp_rank: int = 0,
+                       pp_rank: int = 0, tp_size: int = 1, world_size: int = 1,
+                       transfer_backend: str | None = None, page_first: bool = False,
+                       recurrent_layer_names=(), layer_group_ids=None) -> list[str]:
+    """Register exactly the KV caches of this device (worker.py:261-412) with
+    an in-process engine.  Returns the registered layer names in order."""
+    from .transfer import TransferMode
+    if not kv_caches:
+        raise RuntimeError("No KV cache layers were selected for registration")
+    names, ptrs, sizes, num_blocks, bytes_per_block, kv_strides, segments = ([] for _ in range(7))
+    for layer_name, kv_cache in kv_caches.items():
+        recurrent = layer_name in recurrent_layer_names or isinstance(kv_cache, (tuple, list))
+        tensor = registration_tensor(kv_cache)
+        assert tensor.storage_offset() == 0, f"KV cache for {layer_name} must have zero storage offset"
+        reg = infer_kv_cache_registration(tensor, block_size, is_mla=is_mla,
+                                          is_recurrent_state=recurrent)
+        names.append(layer_name)
+        ptrs.append(tensor.data_ptr())
+        sizes.append(tensor.untyped_storage().nbytes())
+        num_blocks.append(reg.num_blocks)
+        bytes_per_block.append(reg.bytes_per_block)
+        kv_strides.append(reg.kv_stride_bytes)
+        segments.append(reg.segments)
+    mode = TransferMode.from_name(resolve_transfer_backend(is_mla, transfer_backend))
+    engine.register_context_layer_batch(
+        instance_id, namespace, device_id, tp_rank, pp_rank, tp_size, world_size, names, ptrs,
+        sizes, num_blocks, bytes_per_block, kv_strides, segments, transfer_mode=mode,
+        page_first=page_first, layer_group_ids=layer_group_ids)
+    return names
+
+
+def block_shard(block_ids, block_hashes, tp_rank: int, tp_size: int):
+    """The (block ids, hashes) one rank saves under page-first: the stripe
+    ``block_id % tp_size == tp_rank`` (worker.py:982-1005)."""
+    if tp_size <= 1:
+        return list(block_ids), list(block_hashes)
+    ids, hashes = [], []
+    for block_id, block_hash in zip(block_ids, block_hashes, strict=True):
+        if block_id % tp_size == tp_rank:
+            ids.append(block_id)
+            hashes.append(block_hash)
+    return ids, hashes
+
+
+def assemble_layer_saves(save_intents, registered_layers, *, layer_to_group=None,
+                         page_first: bool = False, stripe: tuple[int, int] | None = None,
+                         cross_layer_key: str | None = None):
+    """Per-layer save lists of a batch of save intents (worker.py:826-885).
+
+    Each intent carries ``block_ids_by_group`` and ``block_hashes``.  Every
+    registered layer (or the one cross-layer pseudo-layer) receives the ids of
+    its cache group; the vLLM null block (id 0) is dropped with its hash;
+    under page-first with ``stripe = (tp_rank, tp_size)`` each rank keeps its
+    block stripe.  Lists of several intents are concatenated per layer.
+    Returns ``[(layer_name, block_ids, block_hashes)]`` in first-seen order."""
+    layer_to_group = layer_to_group or {}
+    saves: dict[str, tuple[list, list]] = {}
+    for intent in save_intents:
+        if not any(intent.block_ids_by_group):
+            continue
+        if cross_layer_key is not None:
+            target_layers = (cross_layer_key,)
+        else:
+            assert registered_layers, "KV caches must be registered before submitting save intents"
+            target_layers = tuple(registered_layers)
+        for layer_name in target_layers:
+            group_index = layer_to_group.get(layer_name, 0)
+            try:
+                block_ids = intent.block_ids_by_group[group_index]
+            except IndexError as exc:
+                raise RuntimeError(
+                    f"save intent is missing cache group {group_index} for {layer_name}") from exc
+            block_hashes = intent.block_hashes
+            if len(block_ids) != len(block_hashes):
+                raise RuntimeError(
+                    f"save block/hash count mismatch for {layer_name}: "
+                    f"blocks={len(block_ids)} hashes={len(block_hashes)}")
+            non_null = [(b, h) for b, h in zip(block_ids, block_hashes, strict=True) if b != 0]
+            ids = [b for b, _ in non_null]
+            hashes = [h for _, h in non_null]
+            if page_first and stripe is not None:
+                ids, hashes = block_shard(ids, hashes, stripe[0], stripe[1])
+            if not ids:
+                continue
+            entry = saves.setdefault(layer_name, ([], []))
+            entry[0].extend(ids)
+            entry[1].extend(hashes)
+    return [(name, ids, hashes) for name, (ids, hashes) in saves.items()]

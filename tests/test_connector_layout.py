@@ -62,3 +62,76 @@ def test_resolve_transfer_backend():
     assert resolve_transfer_backend(False, "KERNEL") == "kernel"
     with pytest.raises(ValueError, match="expected one of: direct, kernel"):
         resolve_transfer_backend(False, "rdma")
+
+
+# ---------------------------------------------------------------------------
+# Worker-side save-list assembly (worker.py:826-885, 982-1005)
+# ---------------------------------------------------------------------------
+
+class _Intent:
+    def __init__(self, block_ids_by_group, block_hashes):
+        self.block_ids_by_group = block_ids_by_group
+        self.block_hashes = block_hashes
+
+
+def test_block_shard_stripes_are_disjoint_and_complete():
+    from pegaflow_amd.connector import block_shard
+    ids = [7, 0, 12, 5, 9, 4, 18]
+    hashes = [bytes([i]) for i in range(len(ids))]
+    assert block_shard(ids, hashes, 0, 1) == (ids, hashes)
+    seen = []
+    for rank in range(4):
+        got_ids, got_hashes = block_shard(ids, hashes, rank, 4)
+        assert all(b % 4 == rank for b in got_ids)
+        assert [hashes[ids.index(b)] for b in got_ids] == got_hashes     # hashes travel with ids
+        seen += got_ids
+    assert sorted(seen) == sorted(ids)
+    with pytest.raises(ValueError):
+        block_shard([1, 2], [b"a"], 0, 2)
+
+
+def test_assemble_layer_saves_drops_null_blocks_and_follows_groups():
+    from pegaflow_amd.connector import assemble_layer_saves
+    h = [b"h0", b"h1", b"h2"]
+    intents = [
+        _Intent([[4, 0, 6], [9, 8, 0]], h),       # group 0 and group 1 ids of one request
+        _Intent([[], []], []),                     # nothing to save: skipped
+        _Intent([[2], [3]], [b"x"]),
+    ]
+    got = assemble_layer_saves(intents, ["attn.0", "attn.1", "gdn.0"],
+                               layer_to_group={"attn.0": 0, "attn.1": 0, "gdn.0": 1})
+    assert got == [
+        ("attn.0", [4, 6, 2], [b"h0", b"h2", b"x"]),
+        ("attn.1", [4, 6, 2], [b"h0", b"h2", b"x"]),
+        ("gdn.0", [9, 8, 3], [b"h0", b"h1", b"x"]),
+    ]
+    # page-first: each rank keeps its stripe of the non-null blocks
+    got = assemble_layer_saves([_Intent([[4, 0, 6, 7]], [b"a", b"b", b"c", b"d"])], ["l0", "l1"],
+                               page_first=True, stripe=(1, 2))
+    assert got == [("l0", [7], [b"d"]), ("l1", [7], [b"d"])]
+    # cross-layer mode: one pseudo-layer whose block is all layers
+    got = assemble_layer_saves([_Intent([[1, 2]], [b"a", b"b"])], ["ignored"], cross_layer_key="ALL_LAYERS")
+    assert got == [("ALL_LAYERS", [1, 2], [b"a", b"b"])]
+    with pytest.raises(RuntimeError, match="save block/hash count mismatch for l0: blocks=2 hashes=1"):
+        assemble_layer_saves([_Intent([[1, 2]], [b"a"])], ["l0"])
+    with pytest.raises(RuntimeError, match="save intent is missing cache group 1 for l1"):
+        assemble_layer_saves([_Intent([[1]], [b"a"])], ["l1"], layer_to_group={"l1": 1})
+
+
+def test_registration_tensor_accepts_shared_recurrent_states():
+    import torch
+    from pegaflow_amd.connector import registration_tensor
+    t = torch.zeros(8, 16)
+    assert registration_tensor(t) is t
+    storage = torch.zeros(8 * 24)
+    conv = storage.as_strided((8, 16), (24, 1))
+    ssm = storage.as_strided((8, 8), (24, 1), 16)
+    assert registration_tensor((conv, ssm)) is conv
+    with pytest.raises(RuntimeError, match="share one CUDA allocation"):
+        registration_tensor((conv, torch.zeros(8, 8)))
+    with pytest.raises(RuntimeError, match="same block count"):
+        registration_tensor((conv, storage.as_strided((4, 8), (24, 1), 16)))
+    with pytest.raises(RuntimeError, match="one common page stride"):
+        registration_tensor((conv, storage.as_strided((8, 8), (12, 1), 16)))
+    with pytest.raises(TypeError):
+        registration_tensor(())
