@@ -30,16 +30,14 @@ typedef __attribute__((address_space(4))) const uint64_t c_u64;
 
 constexpr int kLanes = 256;
 
-// 16-byte global stores with an explicit cache policy.  Measured on MI355X at
-// the Llama shape (5000 x 2 x 32 KiB gathered or scattered per launch), all 49
-// load x store policy pairs: a dense destination is written fastest with
-// "sc1 nt" (6.35 TB/s against 6.30 for plain nt), a destination scattered over
-// the cache with "sc1" and no nt (6.13 TB/s against 5.72 for nt).
+// 16-byte global store with an explicit cache policy.  Measured on MI355X at
+// the Llama shape (5000 x 2 x 32 KiB gathered or scattered per launch) over
+// all 49 load x store policy pairs: a destination written in ascending
+// address order is written fastest with "sc1 nt" (gather 6.35 TB/s against
+// 6.30 for plain nt; scatter in ascending-id row order 6.17 against 5.63 for
+// "sc1" and 5.44 for an ordinary store).
 __device__ __forceinline__ void store16_sc1_nt(uint64_t dst, u32x4 v) {
   asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(dst), "v"(v) : "memory");
-}
-__device__ __forceinline__ void store16_sc1(uint64_t dst, u32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst), "v"(v) : "memory");
 }
 
 // Copy `bytes` <= U*4096 from src to dst; both 16-byte aligned.
@@ -187,7 +185,13 @@ __global__ __launch_bounds__(LT) void block_tiles_kernel(const BlockUnit* __rest
   constexpr uint32_t kTile = LT * 16;
   const BlockUnit* __restrict__ up = units + (SEGS == 2 ? blockIdx.z >> 1 : blockIdx.z);
   const uint32_t seg = SEGS == 2 ? (blockIdx.z & 1u) : 0u;
-  const uint32_t pos = blockIdx.y;
+  if (blockIdx.y >= up->n_blocks) return;
+  // Rows may visit the list positions in another order (see launch_block_tiles).
+  uint32_t pos = blockIdx.y;
+  if (up->order != nullptr) {
+    c_u32* order = reinterpret_cast<c_u32*>(reinterpret_cast<uint64_t>(up->order));
+    pos = order[blockIdx.y];
+  }
   const uint64_t frag_bytes = up->frag_bytes;
   const uint64_t off = static_cast<uint64_t>(blockIdx.x) * kTile;
   if (seg >= up->n_seg || pos >= up->n_blocks || off >= frag_bytes) return;
@@ -212,16 +216,10 @@ __global__ __launch_bounds__(LT) void block_tiles_kernel(const BlockUnit* __rest
     const g_u32x4* __restrict__ s = reinterpret_cast<const g_u32x4*>(src);
     const uint32_t nvec = bytes >> 4;
     if (lane < nvec) {
-      // Gather: ordinary load of the scattered source, streaming store to the
-      // dense staging side.  Scatter: streaming load of the dense side,
-      // cached-scope store to the scattered destination.
-      if (TO_FAR) {
-        const u32x4 v = s[lane];
-        store16_sc1_nt(dst + lane * 16ull, v);
-      } else {
-        const u32x4 v = __builtin_nontemporal_load(s + lane);
-        store16_sc1(dst + lane * 16ull, v);
-      }
+      // Gather: ordinary load of the scattered source; scatter: streaming
+      // load of the staging side.  Both store streaming.
+      const u32x4 v = TO_FAR ? s[lane] : __builtin_nontemporal_load(s + lane);
+      store16_sc1_nt(dst + lane * 16ull, v);
     }
     const uint32_t j = (nvec << 4) + lane;
     if (j < bytes) reinterpret_cast<g_u8*>(dst)[j] = reinterpret_cast<const g_u8*>(src)[j];

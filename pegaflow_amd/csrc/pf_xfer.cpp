@@ -49,6 +49,10 @@ struct LayerPlan {
   bool vec_ok = false;
   uint64_t ids_slab_off = 0;    // byte offset of the id list inside the slab
   uint64_t table_slab_off = 0;  // byte offset of the page table inside the slab
+  uint64_t order_slab_off = 0;  // byte offset of the row order inside the slab (staged loads)
+  uint64_t per_unit = 0;        // list positions per staged unit
+  bool ordered = false;
+  bool order_owner = false;     // this plan fills the order region
   uint64_t layer_bytes = 0;
   size_t src_index = 0;         // index in the caller's layer array
 };
@@ -298,6 +302,21 @@ bool Xfer::plan_page_pack(const std::vector<LayerPlan>& plans, bool save, PagePa
   return true;
 }
 
+namespace {
+// For every unit-sized range of the list: the positions of the range, relative
+// to its start, in ascending order of their block id.
+void fill_row_order(const uint32_t* ids, uint64_t n, uint64_t per_unit, uint32_t* out) {
+  std::vector<uint64_t> keys;
+  for (uint64_t first = 0; first < n; first += per_unit) {
+    const uint64_t count = std::min(per_unit, n - first);
+    keys.resize(count);
+    for (uint64_t i = 0; i < count; ++i) keys[i] = (static_cast<uint64_t>(ids[first + i]) << 32) | i;
+    std::sort(keys.begin(), keys.end());
+    for (uint64_t i = 0; i < count; ++i) out[first + i] = static_cast<uint32_t>(keys[i]);
+  }
+}
+}  // namespace
+
 int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uint64_t n_layers,
                         bool save, hipStream_t s) {
   const LayerPlan& first = plans.front();
@@ -326,13 +345,19 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
   }
   // Slab: one BlockUnit per (chunk, layer), then the shared id list.
   const uint64_t units_bytes = (chunks.size() * n_plans * sizeof(BlockUnit) + 255) & ~255ull;
-  const uint64_t slab_bytes = units_bytes + ((n * sizeof(uint32_t) + 255) & ~255ull);
+  const uint64_t ids_bytes = (n * sizeof(uint32_t) + 255) & ~255ull;
+  // Loads visit the pages of a chunk in ascending destination id (launch_block_tiles).
+  const uint64_t slab_bytes = units_bytes + ids_bytes + (save ? 0 : ids_bytes);
   SlabPool::Slab* slab = nullptr;
   int st = slabs_.acquire(slab_bytes, &slab);
   if (st != PF_OK) return st;
   uint8_t* slab_host = static_cast<uint8_t*>(slab->host);
   const uint64_t slab_dev = reinterpret_cast<uint64_t>(slab->dev);
   std::memcpy(slab_host + units_bytes, first.ids, n * sizeof(uint32_t));
+  if (!save) {
+    uint32_t* order_host = reinterpret_cast<uint32_t*>(slab_host + units_bytes + ids_bytes);
+    for (const Chunk& c : chunks) fill_row_order(first.ids + c.first, c.count, c.count, order_host + c.first);
+  }
   BlockUnit* units_host = reinterpret_cast<BlockUnit*>(slab_host);
   const BlockUnit* units_dev = reinterpret_cast<const BlockUnit*>(slab_dev);
   std::vector<uint32_t> chunk_slot(chunks.size());
@@ -351,6 +376,10 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
       u.far_base[0] = base + (p.page_offset - pack.lo);
       u.far_stride = pack.page_bytes;
       u.ids = reinterpret_cast<const uint32_t*>(slab_dev + units_bytes) + chunks[ci].first;
+      if (!save && chunks[ci].count > 1) {
+        u.order = reinterpret_cast<const uint32_t*>(slab_dev + units_bytes + ids_bytes) +
+                  chunks[ci].first;
+      }
       u.n_blocks = static_cast<uint32_t>(chunks[ci].count);
       u.n_seg = 1;
       u.tiles_per_frag = 1;
@@ -499,6 +528,7 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     const uint64_t block_bytes = p.frag_bytes * p.n_seg;
     uint64_t per_unit = std::max<uint64_t>(slot_bytes_ / block_bytes, 1);
     per_unit = std::min<uint64_t>(per_unit, kMaxTileBlocks);
+    p.per_unit = per_unit;
     for (uint64_t first = 0; first < p.n_blocks; first += per_unit) {
       uint64_t count = std::min(per_unit, p.n_blocks - first);
       unit_refs.push_back({pi, first, count});
@@ -512,7 +542,9 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     // Layers that pass the very same id array share one upload.
     bool shared = false;
     for (size_t pj = 0; pj < pi; ++pj) {
-      if (plans[pj].ids == p.ids && plans[pj].n_blocks == p.n_blocks) {
+      if (plans[pj].n_blocks == p.n_blocks &&
+          (plans[pj].ids == p.ids ||
+           std::memcmp(plans[pj].ids, p.ids, p.n_blocks * sizeof(uint32_t)) == 0)) {
         p.ids_slab_off = plans[pj].ids_slab_off;
         shared = true;
         break;
@@ -521,6 +553,23 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     if (!shared) {
       p.ids_slab_off = slab_bytes;
       slab_bytes += (p.n_blocks * sizeof(uint32_t) + 255) & ~255ull;
+    }
+    // Staged loads visit each unit's positions in ascending destination id
+    // (launch_block_tiles); layers with the same ids and unit size share it.
+    if (!save && p.staged && p.n_blocks > 1) {
+      p.ordered = true;
+      for (size_t pj = 0; pj < pi; ++pj) {
+        if (plans[pj].ordered && plans[pj].ids_slab_off == p.ids_slab_off &&
+            plans[pj].per_unit == p.per_unit) {
+          p.order_slab_off = plans[pj].order_slab_off;
+          break;
+        }
+      }
+      if (p.order_slab_off == 0) {
+        p.order_owner = true;
+        p.order_slab_off = slab_bytes;
+        slab_bytes += (p.n_blocks * sizeof(uint32_t) + 255) & ~255ull;
+      }
     }
     if (p.page_dev) {
       bool tshared = false;
@@ -548,6 +597,10 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     if (p.page_dev) {
       std::memcpy(slab_host + p.table_slab_off, p.page_dev, p.n_blocks * sizeof(uint64_t));
     }
+    if (p.order_owner) {
+      fill_row_order(p.ids, p.n_blocks, p.per_unit,
+                     reinterpret_cast<uint32_t*>(slab_host + p.order_slab_off));
+    }
   }
 
   // ---- 3. staging slots ---------------------------------------------------
@@ -571,6 +624,9 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     u.kv_stride = p.layout.kv_stride_bytes();
     u.frag_bytes = p.frag_bytes;
     u.ids = reinterpret_cast<const uint32_t*>(slab_dev + p.ids_slab_off) + r.first;
+    if (p.ordered) {
+      u.order = reinterpret_cast<const uint32_t*>(slab_dev + p.order_slab_off) + r.first;
+    }
     u.n_blocks = static_cast<uint32_t>(r.count);
     u.n_seg = p.n_seg;
     u.tiles_per_frag = static_cast<uint32_t>((p.frag_bytes + tile - 1) / tile);
