@@ -429,6 +429,11 @@ int pf_topology_seal(const pf_worker_layers* workers, uint32_t n_workers, uint32
 int pf_topology_destroy(pf_topology_t t);
 uint64_t pf_topology_num_layers(pf_topology_t t);
 uint64_t pf_topology_total_slots(pf_topology_t t);
+/* Storage groups (hybrid models), instance.rs:197-220: number of groups, the
+ * group of a layer id, and the slots a block of that group needs to seal. */
+uint64_t pf_topology_num_groups(pf_topology_t t);
+int pf_topology_group_of_layer(pf_topology_t t, uint64_t layer_id, uint32_t* out_group);
+int pf_topology_group_total_slots(pf_topology_t t, uint32_t group, uint64_t* out_slots);
 int pf_topology_is_page_first(pf_topology_t t);
 /* Layer ids are ranks of the byte-wise sorted layer names. */
 int pf_topology_layer_id(pf_topology_t t, const char* layer_name, uint64_t* out_id);

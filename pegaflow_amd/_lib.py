@@ -219,6 +219,9 @@ PROTOTYPES = {
     "pf_topology_destroy": (C.c_int, [vp]),
     "pf_topology_num_layers": (u64, [vp]),
     "pf_topology_total_slots": (u64, [vp]),
+    "pf_topology_num_groups": (u64, [vp]),
+    "pf_topology_group_of_layer": (C.c_int, [vp, u64, C.POINTER(u32)]),
+    "pf_topology_group_total_slots": (C.c_int, [vp, u32, C.POINTER(u64)]),
     "pf_topology_is_page_first": (C.c_int, [vp]),
     "pf_topology_layer_id": (C.c_int, [vp, C.c_char_p, C.POINTER(u64)]),
     "pf_topology_slot_index": (C.c_int, [vp, u64, u64, C.POINTER(u64)]),

@@ -307,6 +307,34 @@ uint64_t pf_topology_total_slots(pf_topology_t t) {
   return t ? reinterpret_cast<pf::LayerTopology*>(t)->total_slots() : 0;
 }
 
+uint64_t pf_topology_num_groups(pf_topology_t t) {
+  return t ? reinterpret_cast<pf::LayerTopology*>(t)->num_groups() : 0;
+}
+
+int pf_topology_group_of_layer(pf_topology_t t, uint64_t layer_id, uint32_t* out_group) {
+  PF_REQUIRE_PTR(t);
+  PF_REQUIRE_PTR(out_group);
+  auto* topo = reinterpret_cast<pf::LayerTopology*>(t);
+  if (layer_id >= topo->num_layers()) {
+    return pf::fail(PF_ERR_INVALID_ARGUMENT, "layer_id %llu out of range (%zu layers)",
+                    static_cast<unsigned long long>(layer_id), topo->num_layers());
+  }
+  *out_group = topo->group_of_layer(layer_id);
+  return PF_OK;
+}
+
+int pf_topology_group_total_slots(pf_topology_t t, uint32_t group, uint64_t* out_slots) {
+  PF_REQUIRE_PTR(t);
+  PF_REQUIRE_PTR(out_slots);
+  size_t n = 0;
+  std::string err;
+  if (!reinterpret_cast<pf::LayerTopology*>(t)->group_total_slots(group, &n, &err)) {
+    return pf::fail(PF_ERR_INVALID_ARGUMENT, "%s", err.c_str());
+  }
+  *out_slots = n;
+  return PF_OK;
+}
+
 int pf_topology_is_page_first(pf_topology_t t) {
   return t && reinterpret_cast<pf::LayerTopology*>(t)->is_page_first();
 }

@@ -245,6 +245,20 @@ class LayerTopology:
     def is_page_first(self) -> bool:
         return bool(self._lib.pf_topology_is_page_first(self.handle))
 
+    @property
+    def num_groups(self) -> int:
+        return self._lib.pf_topology_num_groups(self.handle)
+
+    def group_of_layer(self, layer_id: int) -> int:
+        out = C.c_uint32()
+        check(self._lib.pf_topology_group_of_layer(self.handle, layer_id, C.byref(out)))
+        return out.value
+
+    def group_total_slots(self, group: int) -> int:
+        out = C.c_uint64()
+        check(self._lib.pf_topology_group_total_slots(self.handle, group, C.byref(out)))
+        return out.value
+
     def layer_id(self, name: str) -> int:
         out = C.c_uint64()
         check(self._lib.pf_topology_layer_id(self.handle, name.encode(), C.byref(out)))

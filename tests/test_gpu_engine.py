@@ -413,3 +413,18 @@ def test_packed_saves_are_reusable_and_share_hash_lists(engine):
         for src, dst in zip([4, 0, 2], [1, 3, 5]):
             want[dst * 512:(dst + 1) * 512] = l.expected[src * 512:(src + 1) * 512]
         l.assert_gpu_matches(want)
+
+
+def test_unsealed_instance_rejects_topology_access(gpu):
+    """instance/tests.rs:269-286: with one of two workers registered nothing can
+    be saved, and the same device cannot register twice."""
+    e = PegaEngine(pool_size=1 << 20)
+    layer = Layer("layer_0", 4, 1024)
+    e.register_context_layer_batch("partial", "partial-ns", 0, 0, 0, 2, 2, ["layer_0"],
+                                   [layer.gpu.ptr], [layer.expected.nbytes], [4], [1024], [0], [1])
+    with pytest.raises(_lib.PegaHipError, match="registration incomplete: 1/2"):
+        e.batch_save_kv_blocks("partial", 0, 0, 0, [LayerSave("layer_0", [0], make_block_hashes(1, 1))])
+    with pytest.raises(_lib.PegaHipError, match="already exists"):
+        e.register_context_layer_batch("partial", "partial-ns", 0, 0, 0, 2, 2, ["layer_0"],
+                                       [layer.gpu.ptr], [layer.expected.nbytes], [4], [1024], [0], [1])
+    e.close()

@@ -244,3 +244,117 @@ def test_topology_rejections():
     ids = {n: topo.layer_id(n) for n in ("att0", "att1", "gdn0")}
     assert [topo.slot_index(ids[n], 0) for n in ("att0", "att1", "gdn0")] == [0, 1, 0]
     topo.close()
+
+
+# ---------------------------------------------------------------------------
+# The remaining cases of pegaflow-core/src/instance/tests.rs, one test each,
+# with the reference's inputs and assertions (the reference needs two CUDA
+# devices for several of them; sealing itself touches no device).
+# ---------------------------------------------------------------------------
+
+def _workers(*specs):
+    """specs: (device_id, tp_rank, pp_rank, [layer names] or [(name, group)], segment_bytes)."""
+    out = []
+    for device_id, tp_rank, pp_rank, layers, seg in specs:
+        names = [l if isinstance(l, str) else l[0] for l in layers]
+        groups = {l[0]: l[1] for l in layers if not isinstance(l, str)} or None
+        out.append(WorkerLayers(device_id, tp_rank, {n: _layout(i, seg) for i, n in enumerate(names)},
+                                pp_rank=pp_rank, groups=groups))
+    return out
+
+
+def test_seal_derives_layer_space_from_union_of_workers():
+    """instance/tests.rs:311-343: pipeline stages register disjoint layers
+    (stage 1 also a speculative MTP layer); ids span the union."""
+    topo = LayerTopology(_workers(
+        (0, 0, 0, ["model.layers.0.self_attn.attn"], 1024),
+        (1, 0, 1, ["model.layers.1.self_attn.attn", "model.layers.2.self_attn.attn"], 1024)),
+        tp_size=1)
+    assert topo.num_layers == 3
+    assert topo.layer_id("model.layers.2.self_attn.attn") == 2
+    topo.close()
+
+
+def test_mla_replica_registration_seals():
+    """instance/tests.rs:360-378: MLA replicas collapse to tp_rank 0; several
+    owners per slot are valid."""
+    layers = ["model.layers.0.self_attn.attn", "model.layers.0.self_attn.indexer.k_cache",
+              "model.layers.1.self_attn.attn", "model.layers.1.self_attn.indexer.k_cache"]
+    topo = LayerTopology(_workers((0, 0, 0, layers, 1024), (1, 0, 0, layers, 1024)), tp_size=1)
+    assert topo.num_layers == 4 and topo.total_slots == 4
+    topo.close()
+
+
+def test_seal_rejects_replicas_across_pipeline_stages():
+    """instance/tests.rs:385-409."""
+    layers = ["model.layers.0.self_attn.attn"]
+    with pytest.raises(_lib.InvalidArgument, match="different pipeline stages"):
+        LayerTopology(_workers((0, 0, 0, layers, 1024), (1, 0, 1, layers, 1024)), tp_size=1)
+
+
+def test_seal_rejects_missing_slot_owner():
+    """instance/tests.rs:415-437: every rank must register every layer; the
+    complete worker set then seals."""
+    with pytest.raises(_lib.InvalidArgument, match="incomplete KV registration") as exc:
+        LayerTopology(_workers((0, 0, 0, ["layer_0", "layer_1"], 1024), (1, 1, 0, ["layer_0"], 1024)),
+                      tp_size=2)
+    assert "layer_1" in str(exc.value)
+    topo = LayerTopology(_workers((0, 0, 0, ["layer_0", "layer_1"], 1024),
+                                  (1, 1, 0, ["layer_0", "layer_1"], 1024)), tp_size=2)
+    assert topo.total_slots == 4
+    topo.close()
+
+
+def test_seal_rejects_inconsistent_layer_geometry():
+    """instance/tests.rs:443-468."""
+    with pytest.raises(_lib.InvalidArgument, match="inconsistent geometry"):
+        LayerTopology(_workers((0, 0, 0, ["layer_0"], 1024), (1, 0, 0, ["layer_0"], 2048)), tp_size=1)
+
+
+def test_hybrid_topology_seals_per_group_slot_spaces():
+    """instance/tests.rs:476-512."""
+    topo = LayerTopology(_workers(
+        (0, 0, 0, [("attn_a", 0), ("attn_b", 0), ("recurrent_c", 1), ("recurrent_d", 1)], 1024)))
+    assert topo.num_layers == 4 and topo.num_groups == 2
+    assert [topo.group_of_layer(i) for i in range(4)] == [0, 0, 1, 1]
+    assert topo.group_total_slots(0) == 2 and topo.group_total_slots(1) == 2
+    assert topo.total_slots == 4
+    assert [topo.slot_index(i, 0) for i in range(4)] == [0, 1, 0, 1]
+    topo.close()
+
+
+def test_default_groups_keep_global_slot_layout():
+    """instance/tests.rs:520-535."""
+    topo = LayerTopology(_workers((0, 0, 0, ["layer_a", "layer_b", "layer_c"], 1024)))
+    assert topo.num_groups == 1 and topo.group_total_slots(0) == 3
+    for layer_id in range(3):
+        assert topo.group_of_layer(layer_id) == 0
+        assert topo.slot_index(layer_id, 0) == layer_id
+    with pytest.raises(_lib.InvalidArgument):
+        topo.group_total_slots(1)
+    topo.close()
+
+
+def test_seal_rejects_inconsistent_layer_group_across_devices():
+    """instance/tests.rs:541-560."""
+    with pytest.raises(_lib.InvalidArgument, match="storage group"):
+        LayerTopology(_workers((0, 0, 0, [("layer_0", 0)], 1024), (1, 0, 0, [("layer_0", 1)], 1024)),
+                      tp_size=1)
+
+
+def test_seal_rejects_sparse_group_ids():
+    """instance/tests.rs:565-576."""
+    with pytest.raises(_lib.InvalidArgument, match="dense"):
+        LayerTopology(_workers((0, 0, 0, [("layer_a", 0), ("layer_b", 2)], 1024)))
+
+
+def test_page_first_rejects_multiple_groups():
+    """instance/tests.rs:581-592."""
+    with pytest.raises(_lib.InvalidArgument, match="page-first"):
+        LayerTopology(_workers((0, 0, 0, [("layer_a", 0), ("layer_b", 1)], 1024)), page_first=True)
+
+
+def test_registration_without_layers_is_rejected():
+    """instance/tests.rs:291-300."""
+    with pytest.raises(_lib.InvalidArgument, match="no KV cache layers"):
+        LayerTopology([WorkerLayers(0, 0, {})])
