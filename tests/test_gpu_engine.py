@@ -428,3 +428,102 @@ def test_unsealed_instance_rejects_topology_access(gpu):
         e.register_context_layer_batch("partial", "partial-ns", 0, 0, 0, 2, 2, ["layer_0"],
                                        [layer.gpu.ptr], [layer.expected.nbytes], [4], [1024], [0], [1])
     e.close()
+
+
+# ---------------------------------------------------------------------------
+# pegaflow-core/tests/prefix_semantics.rs and eviction.rs, one test each
+# ---------------------------------------------------------------------------
+
+def _one_layer_engine(instance, num_blocks, block_bytes, **engine_kw):
+    e = PegaEngine(**engine_kw)
+    layer = Layer("layer_0", num_blocks, block_bytes)
+    register(e, instance, [layer])
+    return e, layer
+
+
+def _save(e, instance, hashes, ids=None):
+    ids = list(range(len(hashes))) if ids is None else ids
+    e.batch_save_kv_blocks(instance, 0, 0, 0, [LayerSave("layer_0", ids, hashes)])
+
+
+def _hits_then_release(e, instance, hashes):
+    hits, lease = e.query_prefix(instance, hashes)
+    if lease:
+        e.release_query_lease(lease)
+    return hits
+
+
+def test_partial_prefix_reports_contiguous_hit_count(gpu):
+    """prefix_semantics.rs:13-30: 3 of 5 saved -> 3 hits, 2 missing."""
+    e, _ = _one_layer_engine("test-partial-prefix", 3, 1024, pool_size=1 << 20)
+    _save(e, "test-partial-prefix", make_block_hashes(3, 10))
+    assert _hits_then_release(e, "test-partial-prefix", make_block_hashes(5, 10)) == 3
+    e.close()
+
+
+def test_gap_in_cached_blocks_breaks_prefix(gpu):
+    """prefix_semantics.rs:33-57: h0, h2, h3 cached -> the prefix stops at h1."""
+    e, _ = _one_layer_engine("test-gap-prefix", 3, 1024, pool_size=1 << 20)
+    h = make_block_hashes(4, 20)
+    _save(e, "test-gap-prefix", [h[0], h[2], h[3]])
+    assert _hits_then_release(e, "test-gap-prefix", h) == 1
+    e.close()
+
+
+def test_first_block_missing_yields_zero_prefix_hit(gpu):
+    """prefix_semantics.rs:60-82: no lease is created for zero hits."""
+    e, _ = _one_layer_engine("test-no-prefix", 3, 1024, pool_size=1 << 20)
+    h = make_block_hashes(4, 30)
+    _save(e, "test-no-prefix", [h[1], h[2], h[3]])
+    assert e.query_prefix("test-no-prefix", h) == (0, 0)
+    e.close()
+
+
+def test_miss_does_not_poison_later_hit_and_empty_query(gpu):
+    """prefix_semantics.rs:86-127: a miss leaves no state behind; an empty
+    query is zero hits."""
+    e, _ = _one_layer_engine("test-ram-miss-then-hit", 4, 1024, pool_size=1 << 20)
+    h = make_block_hashes(4, 40)
+    assert e.query_prefix("test-ram-miss-then-hit", h) == (0, 0)
+    _save(e, "test-ram-miss-then-hit", h)
+    assert _hits_then_release(e, "test-ram-miss-then-hit", h) == 4
+    assert e.query_prefix("test-ram-miss-then-hit", []) == (0, 0)
+    e.close()
+
+
+@pytest.mark.parametrize("shards", [1, 2], ids=["one_pool", "two_shards"])
+def test_eviction_reclaims_old_blocks_for_new(gpu, shards):
+    """eviction.rs:27-48,87-107: the pool fits two batches of 4 x 4096 B; the new
+    batch round-trips with the overwritten data, also with a sharded pool."""
+    e, layer = _one_layer_engine("inst-evict", 4, 4096, pool_size=4 * 4096 * 2, pool_shards=shards)
+    _save(e, "inst-evict", make_block_hashes(4, 1))
+    overwritten = (layer.expected.astype(np.uint16) + 42).astype(np.uint8)
+    layer.gpu.copy_from_host(overwritten)
+    new = make_block_hashes(4, 2)
+    _save(e, "inst-evict", new)
+    _save(e, "inst-evict", make_block_hashes(4, 3))          # a third batch must evict the first
+    assert _hits_then_release(e, "inst-evict", make_block_hashes(4, 1)) == 0
+    layer.zero_gpu()
+    hits, lease = e.query_prefix("inst-evict", new)
+    assert hits == 4
+    e.batch_load_kv_blocks_multi_layer("inst-evict", 0, 0, [["layer_0"]], lease, [[0, 1, 2, 3]]).wait()
+    layer.assert_gpu_matches(overwritten)
+    e.close()
+
+
+def test_leased_blocks_survive_eviction_pressure(gpu):
+    """eviction.rs:52-84: a lease pins the blocks and their place in the cache."""
+    e, layer = _one_layer_engine("inst-lease", 4, 4096, pool_size=4 * 4096 * 2)
+    hashes = make_block_hashes(4, 10)
+    _save(e, "inst-lease", hashes)
+    hits, lease = e.query_prefix("inst-lease", hashes)
+    assert hits == 4
+    reclaimed = make_block_hashes(4, 20)
+    _save(e, "inst-lease", reclaimed)
+    _save(e, "inst-lease", make_block_hashes(4, 21))          # pressure: reclaims the unleased batch
+    assert _hits_then_release(e, "inst-lease", reclaimed) == 0
+    assert _hits_then_release(e, "inst-lease", hashes) == 4   # still the same prefix
+    layer.zero_gpu()
+    e.batch_load_kv_blocks_multi_layer("inst-lease", 0, 0, [["layer_0"]], lease, [[0, 1, 2, 3]]).wait()
+    layer.assert_gpu_matches(layer.expected)
+    e.close()
