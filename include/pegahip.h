@@ -564,6 +564,31 @@ int pf_engine_batch_load(pf_engine_t e, const char* instance_id, uint64_t tp_ran
                          const uint64_t* group_sizes, uint64_t lease,
                          const int64_t* const* dest_block_ids, uint64_t n_blocks,
                          const char* load_state_shm, pf_task_t* out_task);
+/* The same with several leases in one task (lib.rs:654-898: `loads` is a list
+ * of (lease, destinations per group)); dest_block_ids[g] has n_blocks entries,
+ * one per block of that lease, -1 = skip. */
+typedef struct pf_load_request {
+  uint64_t lease;
+  const int64_t* const* dest_block_ids;
+  uint64_t n_blocks;
+} pf_load_request;
+int pf_engine_batch_load_multi(pf_engine_t e, const char* instance_id, uint64_t tp_rank,
+                               int device_id, uint64_t n_groups,
+                               const char* const* const* group_layer_names,
+                               const uint64_t* group_sizes, const pf_load_request* loads,
+                               uint64_t n_loads, const char* load_state_shm, pf_task_t* out_task);
+/* query_group_membership, lib.rs:593-611: out_present[i] = 1 when hashes[i] is
+ * sealed in storage group `group` (every position on its own; no prefix rule).
+ * An unknown group is an error. */
+int pf_engine_query_group_membership(pf_engine_t e, const char* instance_id, uint32_t group,
+                                     const uint8_t* const* hashes, const uint32_t* hash_lens,
+                                     uint64_t n, uint8_t* out_present);
+/* create_query_lease, lib.rs:614-628, naming the blocks by (group, hash): a
+ * lease over exactly these blocks, in this order.  n == 0 is an error; a hash
+ * that is no longer resident is PF_ERR_STORAGE. */
+int pf_engine_create_group_lease(pf_engine_t e, const char* instance_id, uint32_t group,
+                                 const uint8_t* const* hashes, const uint32_t* hash_lens,
+                                 uint64_t n, uint64_t* out_lease);
 int pf_engine_pool_usage(pf_engine_t e, uint64_t* out_used, uint64_t* out_total);
 uint64_t pf_engine_cached_blocks(pf_engine_t e);
 /* Drop every cached block that is not leased; returns how many. */

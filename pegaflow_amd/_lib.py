@@ -128,6 +128,11 @@ class PfLayerSave(C.Structure):
                 ("block_hash_lens", C.POINTER(u32)), ("n_blocks", u64)]
 
 
+class PfLoadRequest(C.Structure):
+    _fields_ = [("lease", u64), ("dest_block_ids", C.POINTER(C.POINTER(C.c_int64))),
+                ("n_blocks", u64)]
+
+
 class PfSaveProfile(C.Structure):
     _fields_ = [("validate_ms", C.c_double), ("filter_ms", C.c_double), ("alloc_ms", C.c_double),
                 ("assemble_ms", C.c_double), ("transfer_ms", C.c_double),
@@ -258,6 +263,16 @@ PROTOTYPES = {
                                        C.POINTER(C.POINTER(C.c_int64)), u64, C.c_char_p,
                                        C.POINTER(vp)]),
     "pf_engine_last_save_profile": (C.c_int, [vp, C.POINTER(PfSaveProfile)]),
+    "pf_engine_batch_load_multi": (C.c_int, [vp, C.c_char_p, u64, C.c_int, u64,
+                                             C.POINTER(C.POINTER(C.c_char_p)), C.POINTER(u64),
+                                             C.POINTER(PfLoadRequest), u64, C.c_char_p,
+                                             C.POINTER(vp)]),
+    "pf_engine_query_group_membership": (C.c_int, [vp, C.c_char_p, u32,
+                                                   C.POINTER(C.POINTER(C.c_uint8)),
+                                                   C.POINTER(u32), u64, C.POINTER(C.c_uint8)]),
+    "pf_engine_create_group_lease": (C.c_int, [vp, C.c_char_p, u32,
+                                               C.POINTER(C.POINTER(C.c_uint8)), C.POINTER(u32),
+                                               u64, C.POINTER(u64)]),
     "pf_engine_pool_usage": (C.c_int, [vp, C.POINTER(u64), C.POINTER(u64)]),
     "pf_engine_cached_blocks": (u64, [vp]),
     "pf_engine_evict_all": (u64, [vp]),

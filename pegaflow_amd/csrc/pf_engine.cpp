@@ -737,6 +737,55 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
   return PF_OK;
 }
 
+int Engine::query_group_membership(const std::string& instance_id, uint32_t group,
+                                   const std::vector<std::string>& hashes,
+                                   std::vector<uint8_t>* present, std::string* err) {
+  auto instance = get_instance(instance_id, err);
+  if (!instance) return PF_ERR_INSTANCE_MISSING;
+  auto topo = instance->sealed_topology(err);
+  if (!topo) return PF_ERR_INVALID_ARGUMENT;
+  size_t slots = 0;
+  std::string cause;
+  if (!topo->group_total_slots(group, &slots, &cause)) return bad(err, PF_ERR_INVALID_ARGUMENT, cause);
+  present->assign(hashes.size(), 0);
+  std::lock_guard<std::mutex> lock(mu_);
+  for (size_t i = 0; i < hashes.size(); ++i) {
+    (*present)[i] = sealed_.count(BlockKey{instance->ns(), group_hash(hashes[i], group)}) ? 1 : 0;
+  }
+  return PF_OK;
+}
+
+int Engine::create_group_lease(const std::string& instance_id, uint32_t group,
+                               const std::vector<std::string>& hashes, uint64_t* out_lease,
+                               std::string* err) {
+  auto instance = get_instance(instance_id, err);
+  if (!instance) return PF_ERR_INSTANCE_MISSING;
+  auto topo = instance->sealed_topology(err);
+  if (!topo) return PF_ERR_INVALID_ARGUMENT;
+  size_t slots = 0;
+  std::string cause;
+  if (!topo->group_total_slots(group, &slots, &cause)) return bad(err, PF_ERR_INVALID_ARGUMENT, cause);
+  if (hashes.empty()) {
+    return bad(err, PF_ERR_INVALID_ARGUMENT, "query lease requires at least one block");
+  }
+  std::lock_guard<std::mutex> lock(mu_);
+  Lease lease;
+  lease.instance_id = instance_id;
+  for (size_t i = 0; i < hashes.size(); ++i) {
+    auto it = sealed_.find(BlockKey{instance->ns(), group_hash(hashes[i], group)});
+    if (it == sealed_.end()) {
+      return bad(err, PF_ERR_STORAGE,
+                 "block " + std::to_string(i) + " of the lease is not resident in group " +
+                     std::to_string(group));
+    }
+    lease.blocks.push_back(it->second.block);
+    lru_.splice(lru_.end(), lru_, it->second.pos);
+  }
+  *out_lease = next_lease_++;
+  leases_[*out_lease] = std::move(lease);
+  return PF_OK;
+}
+
 SaveProfile Engine::last_save_profile() {
   std::lock_guard<std::mutex> lock(mu_);
   return last_save_profile_;

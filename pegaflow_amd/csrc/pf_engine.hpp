@@ -117,6 +117,17 @@ class Engine {
   // blocks (lib.rs:506-546,614-629).
   int query_prefix(const std::string& instance_id, const std::vector<std::string>& hashes,
                    uint64_t* out_hits, uint64_t* out_lease, std::string* err);
+  // lib.rs:593-611: per-position membership of `hashes` in one storage group
+  // (no prefix rule, no lease).  An unknown group is an error.
+  int query_group_membership(const std::string& instance_id, uint32_t group,
+                             const std::vector<std::string>& hashes, std::vector<uint8_t>* present,
+                             std::string* err);
+  // lib.rs:614-628 over hashes instead of block handles: a lease that pins the
+  // sealed blocks of exactly these hashes in `group`.  Fails when one of them
+  // is not resident (it may have been evicted since the membership query).
+  int create_group_lease(const std::string& instance_id, uint32_t group,
+                         const std::vector<std::string>& hashes, uint64_t* out_lease,
+                         std::string* err);
   bool release_query_lease(uint64_t lease);
   // lib.rs:654-898.  On success *out is fulfilled when the load settles (at
   // once when nothing is to be loaded).

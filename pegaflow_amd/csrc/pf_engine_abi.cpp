@@ -411,6 +411,94 @@ int pf_engine_batch_load(pf_engine_t e, const char* instance_id, uint64_t tp_ran
   return PF_OK;
 }
 
+int pf_engine_batch_load_multi(pf_engine_t e, const char* instance_id, uint64_t tp_rank,
+                               int device_id, uint64_t n_groups,
+                               const char* const* const* group_layer_names,
+                               const uint64_t* group_sizes, const pf_load_request* loads,
+                               uint64_t n_loads, const char* load_state_shm, pf_task_t* out_task) {
+  PF_REQUIRE_PTR(e);
+  PF_REQUIRE_PTR(instance_id);
+  PF_REQUIRE_PTR(out_task);
+  if (n_loads != 0) PF_REQUIRE_PTR(loads);
+  std::vector<std::vector<std::string>> groups(n_groups);
+  for (uint64_t g = 0; g < n_groups; ++g) {
+    for (uint64_t i = 0; i < group_sizes[g]; ++i) groups[g].emplace_back(group_layer_names[g][i]);
+  }
+  std::vector<pf::LoadRequest> reqs(n_loads);
+  for (uint64_t l = 0; l < n_loads; ++l) {
+    reqs[l].lease = loads[l].lease;
+    reqs[l].block_ids_by_group.resize(n_groups);
+    for (uint64_t g = 0; g < n_groups; ++g) {
+      if (loads[l].n_blocks != 0 && (!loads[l].dest_block_ids || !loads[l].dest_block_ids[g])) {
+        return pf::fail(PF_ERR_INVALID_ARGUMENT, "load %llu has no destination list for group %llu",
+                        static_cast<unsigned long long>(l), static_cast<unsigned long long>(g));
+      }
+      if (loads[l].n_blocks != 0) {
+        reqs[l].block_ids_by_group[g].assign(loads[l].dest_block_ids[g],
+                                             loads[l].dest_block_ids[g] + loads[l].n_blocks);
+      }
+    }
+  }
+  auto h = std::make_unique<TaskHandle>();
+  std::string err;
+  std::string shm = load_state_shm ? load_state_shm : "";
+  int st = reinterpret_cast<pf::Engine*>(e)->batch_load_kv_blocks_multi_layer(
+      instance_id, tp_rank, device_id, groups, reqs, shm, &h->fut, &err);
+  if (st != PF_OK) {
+    pf::last_error() = err;
+    if (!shm.empty()) {
+      std::string aerr;
+      if (auto ls = pf::LoadState::attach(shm, &aerr)) ls->set_error();
+    }
+    return st;
+  }
+  *out_task = reinterpret_cast<pf_task_t>(h.release());
+  return PF_OK;
+}
+
+int pf_engine_query_group_membership(pf_engine_t e, const char* instance_id, uint32_t group,
+                                     const uint8_t* const* hashes, const uint32_t* hash_lens,
+                                     uint64_t n, uint8_t* out_present) {
+  PF_REQUIRE_PTR(e);
+  PF_REQUIRE_PTR(instance_id);
+  if (n != 0) {
+    PF_REQUIRE_PTR(hashes);
+    PF_REQUIRE_PTR(hash_lens);
+    PF_REQUIRE_PTR(out_present);
+  }
+  std::vector<std::string> h;
+  for (uint64_t i = 0; i < n; ++i) h.push_back(hash_of(hashes[i], hash_lens[i]));
+  std::vector<uint8_t> present;
+  std::string err;
+  int st = reinterpret_cast<pf::Engine*>(e)->query_group_membership(instance_id, group, h, &present,
+                                                                    &err);
+  if (st != PF_OK) {
+    pf::last_error() = err;
+    return st;
+  }
+  for (uint64_t i = 0; i < n; ++i) out_present[i] = present[i];
+  return PF_OK;
+}
+
+int pf_engine_create_group_lease(pf_engine_t e, const char* instance_id, uint32_t group,
+                                 const uint8_t* const* hashes, const uint32_t* hash_lens,
+                                 uint64_t n, uint64_t* out_lease) {
+  PF_REQUIRE_PTR(e);
+  PF_REQUIRE_PTR(instance_id);
+  PF_REQUIRE_PTR(out_lease);
+  if (n != 0) {
+    PF_REQUIRE_PTR(hashes);
+    PF_REQUIRE_PTR(hash_lens);
+  }
+  std::vector<std::string> h;
+  for (uint64_t i = 0; i < n; ++i) h.push_back(hash_of(hashes[i], hash_lens[i]));
+  std::string err;
+  int st = reinterpret_cast<pf::Engine*>(e)->create_group_lease(instance_id, group, h, out_lease,
+                                                                &err);
+  if (st != PF_OK) pf::last_error() = err;
+  return st;
+}
+
 int pf_engine_pool_usage(pf_engine_t e, uint64_t* out_used, uint64_t* out_total) {
   PF_REQUIRE_PTR(e);
   PF_REQUIRE_PTR(out_used);

@@ -307,6 +307,66 @@ class PegaEngine:
                                              C.byref(t)))
         return Task(t, keep)
 
+    def query_group_membership(self, instance_id: str, group: int,
+                               hashes: Sequence[bytes]) -> list[bool]:
+        """Which of ``hashes`` are sealed in storage group ``group``, position by
+        position (no prefix rule)."""
+        ptrs, lens, _bufs = _pack_hashes(hashes)
+        out = (C.c_uint8 * max(len(hashes), 1))()
+        check(self._lib.pf_engine_query_group_membership(self.handle, instance_id.encode(), group,
+                                                         ptrs, lens, len(hashes), out))
+        return [bool(out[i]) for i in range(len(hashes))]
+
+    def create_group_lease(self, instance_id: str, group: int, hashes: Sequence[bytes]) -> int:
+        """A lease over exactly the blocks of ``hashes`` in ``group``."""
+        ptrs, lens, _bufs = _pack_hashes(hashes)
+        lease = C.c_uint64()
+        check(self._lib.pf_engine_create_group_lease(self.handle, instance_id.encode(), group,
+                                                     ptrs, lens, len(hashes), C.byref(lease)))
+        return lease.value
+
+    def batch_load_multi(self, instance_id: str, tp_rank: int, device_id: int,
+                         layer_groups: Sequence[Sequence[str]],
+                         loads: Sequence[tuple[int, Sequence[Sequence[int | None]]]],
+                         load_state: LoadState | None = None) -> Task:
+        """Several leases in one load task: ``loads`` = [(lease, destinations
+        per layer group)], each destination list as long as the lease."""
+        g = len(layer_groups)
+        keep = []
+        group_ptrs = (C.POINTER(C.c_char_p) * max(g, 1))()
+        sizes = (C.c_uint64 * max(g, 1))()
+        for i, names in enumerate(layer_groups):
+            arr = (C.c_char_p * max(len(names), 1))(*[s.encode() for s in names])
+            keep.append(arr)
+            group_ptrs[i] = arr
+            sizes[i] = len(names)
+        reqs = (_lib.PfLoadRequest * max(len(loads), 1))()
+        for li, (lease, dests) in enumerate(loads):
+            if len(dests) != g:
+                raise _lib.InvalidArgument(
+                    _lib.PF_ERR_INVALID_ARGUMENT,
+                    f"load group count {len(dests)} does not match layer group count {g}")
+            n_blocks = len(dests[0]) if g else 0
+            ptrs = (C.POINTER(C.c_int64) * max(g, 1))()
+            for gi, ids in enumerate(dests):
+                if len(ids) != n_blocks:
+                    raise _lib.InvalidArgument(
+                        _lib.PF_ERR_INVALID_ARGUMENT,
+                        "every load group needs one destination per leased block")
+                d = (C.c_int64 * max(n_blocks, 1))(*[-1 if v is None else int(v) for v in ids])
+                keep.append(d)
+                ptrs[gi] = d
+            keep.append(ptrs)
+            reqs[li].lease = lease
+            reqs[li].dest_block_ids = ptrs
+            reqs[li].n_blocks = n_blocks
+        t = C.c_void_p()
+        shm = load_state.shm_name.encode() if load_state is not None else None
+        check(self._lib.pf_engine_batch_load_multi(self.handle, instance_id.encode(), tp_rank,
+                                                   device_id, g, group_ptrs, sizes, reqs, len(loads),
+                                                   shm, C.byref(t)))
+        return Task(t, keep)
+
     def last_save_profile(self) -> dict:
         """Milliseconds per phase of the last successful save (and its bytes)."""
         p = _lib.PfSaveProfile()

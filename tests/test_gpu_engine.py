@@ -527,3 +527,74 @@ def test_leased_blocks_survive_eviction_pressure(gpu):
     e.batch_load_kv_blocks_multi_layer("inst-lease", 0, 0, [["layer_0"]], lease, [[0, 1, 2, 3]]).wait()
     layer.assert_gpu_matches(layer.expected)
     e.close()
+
+
+def test_recurrent_group_seals_final_block_save(engine):
+    """hybrid_groups.rs:14-176: the recurrent group seals a tail-only checkpoint
+    save, membership is per group, and one load with two leases restores the
+    attention prefix and the recurrent state block (5 -> 7)."""
+    attn_block, recur_block = 1024, 2048
+    layers = [Layer("attn_0", 8, attn_block), Layer("attn_1", 8, attn_block, overwrite=3),
+              Layer("recurrent_state", 8, recur_block, overwrite=9)]
+    register(engine, "hybrid-hma", layers, ns="hybrid-hma-ns", groups=[0, 0, 1])
+    hashes = make_block_hashes(8, 10)
+    prefix = hashes[:3]
+    engine.batch_save_kv_blocks("hybrid-hma", 0, 0, 0, [LayerSave("attn_0", [0, 1, 2], prefix),
+                                                        LayerSave("attn_1", [0, 1, 2], prefix)])
+    engine.batch_save_kv_blocks("hybrid-hma", 0, 0, 0, [LayerSave("recurrent_state", [5], [hashes[2]])])
+    assert engine.query_group_membership("hybrid-hma", 0, prefix) == [True, True, True]
+    assert engine.query_group_membership("hybrid-hma", 1, prefix) == [False, False, True]
+    with pytest.raises(_lib.InvalidArgument):
+        engine.query_group_membership("hybrid-hma", 2, prefix)       # unknown group: an error
+    hits, attn_lease = engine.query_prefix("hybrid-hma", prefix)     # classic prefix query: group 0
+    assert hits == 3
+    recur_lease = engine.create_group_lease("hybrid-hma", 1, [hashes[2]])
+    with pytest.raises(_lib.InvalidArgument, match="query lease requires at least one block"):
+        engine.create_group_lease("hybrid-hma", 1, [])
+    with pytest.raises(_lib.StorageError, match="not resident"):
+        engine.create_group_lease("hybrid-hma", 1, [hashes[0]])
+    for l in layers:
+        l.zero_gpu()
+    state = LoadState()
+    engine.batch_load_multi("hybrid-hma", 0, 0, [["attn_0", "attn_1"], ["recurrent_state"]], [
+        (attn_lease, [[0, 1, 2], [None, None, None]]),
+        (recur_lease, [[None], [7]]),
+    ], state).wait()
+    assert state.get() == LOAD_STATE_SUCCESS
+    for l in layers[:2]:
+        want = np.zeros_like(l.expected)
+        want[:3 * attn_block] = l.expected[:3 * attn_block]
+        l.assert_gpu_matches(want)
+    want = np.zeros_like(layers[2].expected)
+    want[7 * recur_block:8 * recur_block] = layers[2].expected[5 * recur_block:6 * recur_block]
+    layers[2].assert_gpu_matches(want)
+    state.close()
+
+
+def test_namespace_isolation(engine):
+    """engine_basic.rs:254-271: blocks of one namespace are invisible to another."""
+    a, b = Layer("layer_0", 4, 1024), Layer("layer_0", 4, 1024)
+    register(engine, "inst-a", [a], ns="ns-a")
+    register(engine, "inst-b", [b], ns="ns-b")
+    hashes = make_block_hashes(4, 50)
+    engine.batch_save_kv_blocks("inst-a", 0, 0, 0, [LayerSave("layer_0", [0, 1, 2, 3], hashes)])
+    assert engine.query_prefix("inst-b", hashes) == (0, 0)
+    hits, lease = engine.query_prefix("inst-a", hashes)
+    assert hits == 4
+    engine.release_query_lease(lease)
+
+
+def test_load_requires_a_live_lease(engine):
+    """prefetch_lease.rs:11-27: a released (or unknown) lease cannot be loaded."""
+    layer = Layer("layer_0", 4, 1024)
+    register(engine, "inst-lease-gone", [layer])
+    hashes = make_block_hashes(4, 60)
+    engine.batch_save_kv_blocks("inst-lease-gone", 0, 0, 0, [LayerSave("layer_0", [0, 1, 2, 3], hashes)])
+    _hits, lease = engine.query_prefix("inst-lease-gone", hashes)
+    engine.release_query_lease(lease)
+    state = LoadState()
+    with pytest.raises(_lib.StorageError, match="query lease .* not found"):
+        engine.batch_load_kv_blocks_multi_layer("inst-lease-gone", 0, 0, [["layer_0"]], lease,
+                                                [[0, 1, 2, 3]], state)
+    assert state.get() == LOAD_STATE_ERROR
+    state.close()
