@@ -771,6 +771,7 @@ int Engine::create_group_lease(const std::string& instance_id, uint32_t group,
   std::lock_guard<std::mutex> lock(mu_);
   Lease lease;
   lease.instance_id = instance_id;
+  lease.remaining_consumers = std::max<size_t>(instance->world_size(), 1);
   for (size_t i = 0; i < hashes.size(); ++i) {
     auto it = sealed_.find(BlockKey{instance->ns(), group_hash(hashes[i], group)});
     if (it == sealed_.end()) {
@@ -798,6 +799,7 @@ int Engine::query_prefix(const std::string& instance_id, const std::vector<std::
   std::lock_guard<std::mutex> lock(mu_);
   Lease lease;
   lease.instance_id = instance_id;
+  lease.remaining_consumers = std::max<size_t>(instance->world_size(), 1);
   for (const std::string& h : hashes) {
     auto it = sealed_.find(BlockKey{instance->ns(), h});
     if (it == sealed_.end()) break;
@@ -867,14 +869,23 @@ int Engine::batch_load_kv_blocks_multi_layer(
     std::vector<std::shared_ptr<SealedBlock>> blocks;
     {
       std::lock_guard<std::mutex> lock(mu_);
+      // lease.rs:105-134.
       auto it = leases_.find(lr.lease);
-      if (it == leases_.end() || it->second.instance_id != instance_id) {
+      if (it == leases_.end()) {
+        return bad(err, PF_ERR_STORAGE, "query lease is unknown or expired");
+      }
+      if (it->second.instance_id != instance_id) {
         return bad(err, PF_ERR_STORAGE,
-                   "query lease " + std::to_string(lr.lease) + " not found for instance " +
+                   "query lease belongs to instance " + it->second.instance_id + ", got " +
                        instance_id);
       }
-      blocks = std::move(it->second.blocks);
-      leases_.erase(it);
+      if (it->second.remaining_consumers > 1) {
+        --it->second.remaining_consumers;
+        blocks = it->second.blocks;
+      } else {
+        blocks = std::move(it->second.blocks);
+        leases_.erase(it);
+      }
     }
     if (lr.block_ids_by_group.size() != layer_groups.size()) {
       return bad(err, PF_ERR_INVALID_ARGUMENT,

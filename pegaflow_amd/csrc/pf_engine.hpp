@@ -80,6 +80,7 @@ class InstanceContext {
   const std::string& id() const { return id_; }
   const std::string& ns() const { return ns_; }
   size_t tp_size() const { return tp_size_; }
+  size_t world_size() const { return world_size_; }
   // Validation that must precede the (expensive) GPU context construction.
   int check_accepting(int device_id, size_t tp_rank, std::string* err);
 
@@ -168,9 +169,12 @@ class Engine {
   std::map<BlockKey, SealedEntry> sealed_;
   std::list<BlockKey> lru_;
   void seal_insert(const BlockKey& key, std::shared_ptr<SealedBlock> block);
+  // lease.rs:40-134: a lease serves one load per worker of the instance's
+  // world size, then disappears.
   struct Lease {
     std::string instance_id;
     std::vector<std::shared_ptr<SealedBlock>> blocks;
+    size_t remaining_consumers = 1;
   };
   std::map<uint64_t, Lease> leases_;
   uint64_t next_lease_ = 1;

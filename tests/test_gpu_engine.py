@@ -593,8 +593,26 @@ def test_load_requires_a_live_lease(engine):
     _hits, lease = engine.query_prefix("inst-lease-gone", hashes)
     engine.release_query_lease(lease)
     state = LoadState()
-    with pytest.raises(_lib.StorageError, match="query lease .* not found"):
+    with pytest.raises(_lib.StorageError, match="query lease is unknown or expired"):
         engine.batch_load_kv_blocks_multi_layer("inst-lease-gone", 0, 0, [["layer_0"]], lease,
                                                 [[0, 1, 2, 3]], state)
     assert state.get() == LOAD_STATE_ERROR
     state.close()
+
+
+def test_lease_of_another_instance_is_refused_without_being_consumed(engine):
+    """lease.rs:192-219 through the load path (lib.rs:779-782)."""
+    a, b = Layer("layer_0", 4, 1024), Layer("layer_0", 4, 1024)
+    register(engine, "inst-a", [a], ns="shared-ns")
+    register(engine, "inst-b", [b], ns="shared-ns")
+    hashes = make_block_hashes(4, 70)
+    engine.batch_save_kv_blocks("inst-a", 0, 0, 0, [LayerSave("layer_0", [0, 1, 2, 3], hashes)])
+    _hits, lease = engine.query_prefix("inst-a", hashes)
+    with pytest.raises(_lib.StorageError, match="query lease belongs to instance inst-a, got inst-b"):
+        engine.batch_load_kv_blocks_multi_layer("inst-b", 0, 0, [["layer_0"]], lease, [[0, 1, 2, 3]])
+    a.zero_gpu()
+    engine.batch_load_kv_blocks_multi_layer("inst-a", 0, 0, [["layer_0"]], lease, [[0, 1, 2, 3]]).wait()
+    a.assert_gpu_matches(a.expected)
+    # consumed by its one worker (world size 1): a second load finds it gone
+    with pytest.raises(_lib.StorageError, match="query lease is unknown or expired"):
+        engine.batch_load_kv_blocks_multi_layer("inst-a", 0, 0, [["layer_0"]], lease, [[0, 1, 2, 3]])
