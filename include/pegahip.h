@@ -395,6 +395,9 @@ int pf_numa_pin_thread(int numa_node);
 int pf_numa_node_count(void);
 /* NUMA node of a PCI device under `sysfs_root` (NULL = /sys/bus/pci/devices). */
 int pf_numa_node_of_pci(const char* bdf, const char* sysfs_root);
+/* query_pages_numa, numa.rs:448-476: the NUMA node each address currently
+ * resides on (move_pages query), -1 where unknown. */
+int pf_numa_query_pages(const void* const* addrs, uint64_t n, int* out_nodes);
 
 /* ------------------------------------------------------------------------ */
 /* Layer topology and page-first placement                                   */

@@ -216,6 +216,7 @@ PROTOTYPES = {
     "pf_numa_parse_cpulist": (C.c_int, [C.c_char_p, C.POINTER(u64), u64, C.POINTER(u64)]),
     "pf_numa_pin_thread": (C.c_int, [C.c_int]),
     "pf_numa_node_count": (C.c_int, []),
+    "pf_numa_query_pages": (C.c_int, [C.POINTER(vp), u64, C.POINTER(C.c_int)]),
     "pf_numa_node_of_pci": (C.c_int, [C.c_char_p, C.c_char_p]),
     "pf_build_page_layout": (C.c_int, [C.POINTER(u64), C.POINTER(u64), u64, u64, C.POINTER(u64),
                                        C.POINTER(u64), C.POINTER(u64), C.POINTER(u64),

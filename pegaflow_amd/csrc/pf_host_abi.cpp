@@ -214,6 +214,18 @@ int pf_numa_node_count(void) {
   return static_cast<int>(topo.size());
 }
 
+int pf_numa_query_pages(const void* const* addrs, uint64_t n, int* out_nodes) {
+  if (n == 0) return PF_OK;
+  PF_REQUIRE_PTR(addrs);
+  PF_REQUIRE_PTR(out_nodes);
+  std::vector<const void*> v(addrs, addrs + n);
+  std::vector<pf::NumaNode> nodes = pf::query_pages_numa(v);
+  for (uint64_t i = 0; i < n; ++i) {
+    out_nodes[i] = i < nodes.size() && nodes[i].is_valid() ? static_cast<int>(nodes[i].id) : -1;
+  }
+  return PF_OK;
+}
+
 int pf_numa_node_of_pci(const char* bdf, const char* sysfs_root) {
   return pf::numa_node_of_pci_device(bdf, sysfs_root);
 }

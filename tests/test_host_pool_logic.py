@@ -358,3 +358,18 @@ def test_registration_without_layers_is_rejected():
     """instance/tests.rs:291-300."""
     with pytest.raises(_lib.InvalidArgument, match="no KV cache layers"):
         LayerTopology([WorkerLayers(0, 0, {})])
+
+
+def test_query_pages_numa():
+    """numa.rs:606-636: no addresses -> nothing; touched heap pages sit on a
+    valid node."""
+    import ctypes as C
+    lib = _lib.load()
+    assert lib.pf_numa_query_pages(None, 0, None) == 0
+    buf = np.zeros(8192 + 4096, dtype=np.uint8)
+    base = (buf.ctypes.data + 4095) & ~4095
+    buf[:] = 1
+    addrs = (C.c_void_p * 2)(base, base + 4096)
+    nodes = (C.c_int * 2)(-7, -7)
+    _lib.check(lib.pf_numa_query_pages(addrs, 2, nodes))
+    assert all(0 <= n < max(lib.pf_numa_node_count(), 1) for n in nodes), list(nodes)
