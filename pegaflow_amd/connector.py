@@ -118,28 +118,33 @@ def resolve_transfer_backend(is_mla: bool, override: str | None) -> str:
 # ---------------------------------------------------------------------------
 
 def registration_tensor(kv_cache):
-    """The tensor that represents a layer's cache (worker.py:154-176): the
-    tensor itself, or the first of a sequence of recurrent-state tensors that
-    share one allocation, block count and page stride."""
+    """The tensor that stands for a layer's cache (worker.py:154-176).  A plain
+    tensor stands for itself.  A sequence of recurrent-state tensors is one
+    page-strided allocation seen through several views: its first view is
+    returned after checking that every view starts in the same storage, has the
+    same number of blocks and steps from block to block by the same bytes."""
     if not isinstance(kv_cache, (tuple, list)):
         return kv_cache
-    states = tuple(kv_cache)
-    if not states or not all(hasattr(s, "untyped_storage") for s in states):
+    views = list(kv_cache)
+    if not views or any(not hasattr(v, "untyped_storage") for v in views):
         raise TypeError("KV cache must be a tensor or a non-empty sequence of state tensors")
-    first = states[0]
-    if first.storage_offset() != 0:
+    head = views[0]
+    if head.storage_offset() != 0:
         raise RuntimeError("the first recurrent-state tensor must start at storage offset zero")
-    storage_ptr = first.untyped_storage().data_ptr()
-    num_blocks = first.shape[0]
-    page_bytes = first.stride(0) * first.element_size()
-    for state in states:
-        if state.untyped_storage().data_ptr() != storage_ptr:
-            raise RuntimeError("recurrent-state tensors must share one CUDA allocation")
-        if state.shape[0] != num_blocks:
-            raise RuntimeError("recurrent-state tensors must have the same block count")
-        if state.stride(0) * state.element_size() != page_bytes:
-            raise RuntimeError("recurrent-state tensors must have one common page stride")
-    return first
+
+    def facts(view):
+        return (view.untyped_storage().data_ptr(), view.shape[0],
+                view.stride(0) * view.element_size())
+
+    complaints = ("recurrent-state tensors must share one CUDA allocation",
+                  "recurrent-state tensors must have the same block count",
+                  "recurrent-state tensors must have one common page stride")
+    expected = facts(head)
+    for view in views[1:]:
+        for got, want, complaint in zip(facts(view), expected, complaints):
+            if got != want:
+                raise RuntimeError(complaint)
+    return head
 
 
 def register_kv_caches(engine, instance_id: str, namespace: str, device_id: int, kv_caches: dict,
@@ -176,15 +181,14 @@ def register_kv_caches(engine, instance_id: str, namespace: str, device_id: int,
 
 def block_shard(block_ids, block_hashes, tp_rank: int, tp_size: int):
     """The (block ids, hashes) one rank saves under page-first: the stripe
-    ``block_id % tp_size == tp_rank`` (worker.py:982-1005)."""
-    if tp_size <= 1:
-        return list(block_ids), list(block_hashes)
-    ids, hashes = [], []
-    for block_id, block_hash in zip(block_ids, block_hashes, strict=True):
-        if block_id % tp_size == tp_rank:
-            ids.append(block_id)
-            hashes.append(block_hash)
-    return ids, hashes
+    ``block_id % tp_size == tp_rank`` (worker.py:982-1005); everything when
+    there is a single rank.  The stripes of all ranks are disjoint and cover
+    every block, so each page is written exactly once."""
+    pairs = list(zip(block_ids, block_hashes, strict=True))
+    if tp_size > 1:
+        pairs = [(block_id, block_hash) for block_id, block_hash in pairs
+                 if block_id % tp_size == tp_rank]
+    return [block_id for block_id, _ in pairs], [block_hash for _, block_hash in pairs]
 
 
 def assemble_layer_saves(save_intents, registered_layers, *, layer_to_group=None,
