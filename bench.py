@@ -80,6 +80,8 @@ def parse_args():
     ap.add_argument("--no-overlap", action="store_true", help="skip the GEMM-overlap section")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-engine", action="store_true", help="skip the save/query/load engine section")
+    ap.add_argument("--engine-child", action="store_true",
+                    help="(internal) run only the engine section and print its JSON")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--settle-max", type=int, default=8,
@@ -169,6 +171,11 @@ def main():
     dst_cache = [new_cache(False) for _ in range(n_layers)]
     save_ids = make_ids(np, w["ids"], nb, n, args.seed)
     load_ids = make_ids(np, "permutation", nb, n, args.seed + 1)
+    if args.engine_child:
+        torch.cuda.synchronize()
+        print(json.dumps(run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids,
+                                    payload)))
+        return
     t0 = time.time()
     pool = PinnedMemory(payload)
     pool_alloc_s = time.time() - t0
@@ -369,15 +376,29 @@ def main():
         duplex = run_duplex(xfer, save_layers, load_layers, stream, path, payload, args)
 
     # ---- the same workload through the save / query / load engine -----------
-    # The bench's own engine and stream are released first: a process gets few
-    # hardware queues (GPU_MAX_HW_QUEUES, 4 by default) and streams beyond that
-    # number share them, which would serialise the pool's two workers.
+    # In a process of its own, as the engine is deployed (a server that runs
+    # nothing else on the GPU): which link copies the runtime overlaps depends
+    # on the history of a process's streams, and this process has used many by
+    # now.  The child allocates its own caches, so this one releases its first.
     xfer.close()
     stream.close()
     pool.close()
     engine = None
     if not args.no_engine:
-        engine = run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, payload)
+        import subprocess
+        del src_cache, dst_cache, save_layers, load_layers, scratch, scratch2
+        torch.cuda.empty_cache()
+        cmd = [sys.executable, os.path.abspath(__file__), "--engine-child", "--workload",
+               args.workload, "--seed", str(args.seed)]
+        if args.layers:
+            cmd += ["--layers", str(args.layers)]
+        proc = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+        lines = [ln for ln in proc.stdout.splitlines() if ln.startswith("{")]
+        if proc.returncode == 0 and lines:
+            engine = json.loads(lines[-1])
+        else:
+            print("bench.py: engine section failed:\n" + proc.stderr[-2000:], file=sys.stderr)
+            sys.exit(1)
 
     # ---- CPU baseline: the oracle's memcpy executor on the host cores -----
     cpu = None

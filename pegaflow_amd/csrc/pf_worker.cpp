@@ -301,7 +301,41 @@ std::unique_ptr<GpuWorkerPool> GpuWorkerPool::spawn(int device_id, NumaNode numa
     if (status) *status = bad.status;
     return nullptr;  // destructor joins the threads
   }
+  pool->prime_copy_overlap();
   return pool;
+}
+
+// Measured on MI355X with this runtime: whether the link copies of the save
+// stream and of the load stream overlap is settled by their first large copies.
+// When the load stream's first host -> device copy is issued while a device ->
+// host copy of the save stream is in flight, the two directions overlap from
+// then on (a save and a load together: 88-107 GB/s); when that first copy runs
+// with nothing else in flight, every later pair is serialised (55 GB/s), and
+// so is a pool whose load stream was warmed up alone.  So the pool issues,
+// once, a few 32 MiB copies on the save stream and, while they run, the same
+// on the load stream.  Failure here only loses the overlap.
+void GpuWorkerPool::prime_copy_overlap() {
+  if (hipSetDevice(device_id_) != hipSuccess) return;
+  const size_t chunk = 32u << 20;
+  void* host = nullptr;
+  void* dev = nullptr;
+  if (hipHostMalloc(&host, 2 * chunk, hipHostMallocMapped) == hipSuccess &&
+      hipMalloc(&dev, 2 * chunk) == hipSuccess) {
+    std::memset(host, 0, 2 * chunk);
+    uint8_t* h = static_cast<uint8_t*>(host);
+    uint8_t* d = static_cast<uint8_t*>(dev);
+    for (int i = 0; i < 6; ++i) {
+      (void)hipMemcpyAsync(h, d, chunk, hipMemcpyDeviceToHost, save_.stream);
+    }
+    for (int i = 0; i < 3; ++i) {
+      (void)hipMemcpyAsync(d + chunk, h + chunk, chunk, hipMemcpyHostToDevice, load_.stream);
+    }
+    (void)hipStreamSynchronize(save_.stream);
+    (void)hipStreamSynchronize(load_.stream);
+  }
+  if (dev) (void)hipFree(dev);
+  if (host) (void)hipHostFree(host);
+  (void)hipGetLastError();
 }
 
 GpuWorkerPool::~GpuWorkerPool() {
@@ -370,13 +404,11 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
     backend = build_backend(mode_);
     if (!use_descriptors_) {
       // The pool always has a second engine (load next to save), so each
-      // worker keeps to one stream.  Whether the runtime overlaps the link
-      // copies of two streams depends on the history of the process's
-      // streams (measured: a save and a load together move 88-103 GB/s in
-      // some processes and 55-57 GB/s in others); with a side stream per
-      // engine the two directions were additionally seen on one hardware
-      // queue.  One stream per worker costs 1.4 % when one direction is
-      // active alone.
+      // worker keeps to one stream: with a side stream per engine the link
+      // copies of the two directions were seen on one hardware queue (a
+      // process gets 4 by default) and a save and a load together shared
+      // 56 GB/s.  One stream per worker costs 1.4 % when one direction is
+      // active alone (see also prime_copy_overlap).
       pf_xfer_config cfg;
       std::memset(&cfg, 0, sizeof(cfg));
       cfg.copy_stream = 2;
@@ -387,6 +419,7 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
       }
     }
   }
+  w->stream = stream;
   ready->set_value(init);
   if (init.status != PF_OK) {
     if (done) (void)hipEventDestroy(done);

@@ -117,7 +117,10 @@ class GpuWorkerPool {
     std::condition_variable cv;
     std::deque<std::unique_ptr<Task>> queue;
     bool stop = false;
+    hipStream_t stream = nullptr;  // set by the worker before it reports ready
   };
+  // One large copy in each direction, in flight together, before the first task.
+  void prime_copy_overlap();
   GpuWorkerPool() = default;
   void run(Worker* w, bool is_load, NumaNode numa, std::promise<TaskResult>* ready);
   std::future<TaskResult> push(Worker* w, std::unique_ptr<Task> t);
