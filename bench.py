@@ -785,9 +785,23 @@ def run_cpu_baseline(np, w, save_ids, load_ids, seconds, seed):
         qwen_pass()
         reps += 1
     q_gbps = 2 * q_layers * 2 * q_n * 32768 * reps / (time.perf_counter() - t0) / 1e9
+    # A plain copy of 1 GiB in 4 MiB pieces over the same threads (a STREAM-copy
+    # style yardstick for the host memory system; bytes counted once, as above).
+    big_src = np.full(1 << 30, 7, dtype=np.uint8)
+    big_dst = np.zeros(1 << 30, dtype=np.uint8)
+    piece = 4 << 20
+    rows = [(big_dst.ctypes.data + o, big_src.ctypes.data + o, big_src.ctypes.data + o, piece, 0, 0)
+            for o in range(0, 1 << 30, piece)]
+    O.exec_descs(rows, host_is_src=True, backend="kernel", threads=threads)
+    reps, t0 = 0, time.perf_counter()
+    while reps < 3 or time.perf_counter() - t0 < 1.0:
+        O.exec_descs(rows, host_is_src=True, backend="kernel", threads=threads)
+        reps += 1
+    stream_gbps = (1 << 30) * reps / (time.perf_counter() - t0) / 1e9
     return {"value": round(out["all"], 2), "unit": "GB/s", "cores": threads, "kind": "port",
             "single_thread_gbps": round(out["one"], 2),
             "configs0_qwen3_0p6b_gbps": round(q_gbps, 2),
+            "plain_copy_1gib_gbps": round(stream_gbps, 2),
             "sample": f"one layer [{nseg},{nb},{seg}B] host-resident, {n} blocks saved+loaded "
                       f"repeatedly for ~{seconds:.0f}s (oracle memcpy executor)"}
 
