@@ -49,3 +49,19 @@ def test_no_device_is_an_error_not_a_fallback():
     assert lib.pf_host_alloc(4096, _lib.PF_HOST_HIP_ALLOC, -1, C.byref(mem)) != 0
     p = C.c_uint64()
     assert lib.pf_dev_malloc(4096, C.byref(p)) != 0
+
+
+def test_header_is_plain_c(tmp_path):
+    """include/pegahip.h is the boundary for C, C++ and FFI generators alike: it
+    must compile as strict C99 and as C++11 with nothing else included."""
+    import shutil
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for compiler, std, name in (("gcc", "-std=c99", "hdr.c"), ("g++", "-std=c++11", "hdr.cpp")):
+        if shutil.which(compiler) is None:
+            pytest.skip(f"{compiler} not installed")
+        src = tmp_path / name
+        src.write_text('#include "include/pegahip.h"\nint main(void) { return 0; }\n')
+        proc = subprocess.run([compiler, std, "-Wall", "-Wextra", "-pedantic", "-Werror",
+                               "-fsyntax-only", str(src), "-I", root], capture_output=True, text=True)
+        assert proc.returncode == 0, proc.stderr
