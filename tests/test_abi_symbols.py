@@ -5,6 +5,8 @@ import ctypes as C
 import os
 import re
 
+import pytest
+
 from pegaflow_amd import _lib
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
