@@ -180,17 +180,22 @@ __global__ __launch_bounds__(kLanes) void block_units_kernel(const BlockUnit* __
 // keeps every SIMD full of waves, and the 3-D grid needs no division.
 // Remapping workgroups so that each XCD owns whole fragments changed nothing
 // (no data is reused, so there is no L2 locality to win).
-template <int LT, bool TO_FAR, int SEGS>
+// UNITS_INNER: grid.y walks the (unit, segment) pairs and grid.z the list
+// positions, so workgroups that are dispatched together belong to one
+// position; otherwise grid.y walks the positions of one (unit, segment).
+template <int LT, bool TO_FAR, int SEGS, bool UNITS_INNER>
 __global__ __launch_bounds__(LT) void block_tiles_kernel(const BlockUnit* __restrict__ units) {
   constexpr uint32_t kTile = LT * 16;
-  const BlockUnit* __restrict__ up = units + (SEGS == 2 ? blockIdx.z >> 1 : blockIdx.z);
-  const uint32_t seg = SEGS == 2 ? (blockIdx.z & 1u) : 0u;
-  if (blockIdx.y >= up->n_blocks) return;
+  const uint32_t unit_seg = UNITS_INNER ? blockIdx.y : blockIdx.z;
+  const uint32_t row = UNITS_INNER ? blockIdx.z : blockIdx.y;
+  const BlockUnit* __restrict__ up = units + (SEGS == 2 ? unit_seg >> 1 : unit_seg);
+  const uint32_t seg = SEGS == 2 ? (unit_seg & 1u) : 0u;
+  if (row >= up->n_blocks) return;
   // Rows may visit the list positions in another order (see launch_block_tiles).
-  uint32_t pos = blockIdx.y;
+  uint32_t pos = row;
   if (up->order != nullptr) {
     c_u32* order = reinterpret_cast<c_u32*>(reinterpret_cast<uint64_t>(up->order));
-    pos = order[blockIdx.y];
+    pos = order[row];
   }
   const uint64_t frag_bytes = up->frag_bytes;
   const uint64_t off = static_cast<uint64_t>(blockIdx.x) * kTile;
@@ -327,20 +332,47 @@ int launch_block_tiles(const BlockUnit* units, uint32_t n_units, uint32_t max_bl
                 "tile launch out of range: %u units, %u blocks, %llu-byte fragments", n_units,
                 max_blocks, static_cast<unsigned long long>(max_frag_bytes));
   }
-  dim3 grid(static_cast<uint32_t>(gx), max_blocks, max_seg * n_units), block(kTileLanes, 1, 1);
-  if (max_seg == 2) {
-    if (to_far) {
-      hipLaunchKernelGGL((block_tiles_kernel<kTileLanes, true, 2>), grid, block, 0, s, units);
+  // A launch over several units (the layers of page-first pages) makes the
+  // units the inner grid dimension: the staging side is then walked page after
+  // page and every cache in ascending position order.  Measured on the
+  // DeepSeek-V3 page-first shape (61 units x 119 pages per launch): gather
+  // 5.3 -> 5.9 TB/s, scatter 5.5 -> 6.2 TB/s against positions-inner.
+  const bool units_inner = n_units > 1;
+  const uint32_t unit_segs = max_seg * n_units;
+  dim3 grid(static_cast<uint32_t>(gx), units_inner ? unit_segs : max_blocks,
+            units_inner ? max_blocks : unit_segs);
+  dim3 block(kTileLanes, 1, 1);
+#define PF_LAUNCH_TILES(TO_FAR_, SEGS_, INNER_)                                                \
+  hipLaunchKernelGGL((block_tiles_kernel<kTileLanes, TO_FAR_, SEGS_, INNER_>), grid, block, 0, s, \
+                     units)
+  if (units_inner) {
+    if (max_seg == 2) {
+      if (to_far) {
+        PF_LAUNCH_TILES(true, 2, true);
+      } else {
+        PF_LAUNCH_TILES(false, 2, true);
+      }
     } else {
-      hipLaunchKernelGGL((block_tiles_kernel<kTileLanes, false, 2>), grid, block, 0, s, units);
+      if (to_far) {
+        PF_LAUNCH_TILES(true, 1, true);
+      } else {
+        PF_LAUNCH_TILES(false, 1, true);
+      }
+    }
+  } else if (max_seg == 2) {
+    if (to_far) {
+      PF_LAUNCH_TILES(true, 2, false);
+    } else {
+      PF_LAUNCH_TILES(false, 2, false);
     }
   } else {
     if (to_far) {
-      hipLaunchKernelGGL((block_tiles_kernel<kTileLanes, true, 1>), grid, block, 0, s, units);
+      PF_LAUNCH_TILES(true, 1, false);
     } else {
-      hipLaunchKernelGGL((block_tiles_kernel<kTileLanes, false, 1>), grid, block, 0, s, units);
+      PF_LAUNCH_TILES(false, 1, false);
     }
   }
+#undef PF_LAUNCH_TILES
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail_hip(e, "block_tiles_kernel launch");
   return PF_OK;
