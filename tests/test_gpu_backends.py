@@ -285,3 +285,63 @@ def test_direct_backend_run_longer_than_the_staging_buffer(stream, gpu):
         b.close()
         dev.close()
         host.close()
+
+
+def _random_batch(rng):
+    """Rows (device offset, host offset, size, host allocation) of a random
+    batch: host-dense runs of small pieces, isolated pieces, now and then a
+    large range; device slots are disjoint and visited in shuffled order."""
+    pieces = []           # (size, host_off, alloc)
+    host_cursor = int(rng.integers(0, 64))
+    alloc = 1
+    for _ in range(int(rng.integers(1, 6))):
+        kind = int(rng.integers(0, 3))
+        if kind == 0:     # a dense run
+            count = int(rng.integers(2, 400))
+            unit = int(rng.choice([16, 64, 1000, 4096, 4112]))
+            for _ in range(count):
+                size = unit if rng.integers(0, 4) else int(rng.integers(1, unit + 1))
+                pieces.append((size, host_cursor, alloc))
+                host_cursor += size
+        elif kind == 1:   # isolated pieces with gaps between them
+            for _ in range(int(rng.integers(1, 40))):
+                size = int(rng.integers(1, 6000))
+                host_cursor += int(rng.integers(1, 300))
+                pieces.append((size, host_cursor, alloc))
+                host_cursor += size
+        else:             # one large range
+            size = (4 << 20) + int(rng.integers(0, 4096))
+            host_cursor += int(rng.integers(0, 64))
+            pieces.append((size, host_cursor, alloc))
+            host_cursor += size
+        host_cursor += int(rng.integers(1, 5000))
+        alloc += int(rng.integers(0, 2))
+    # disjoint device slots, assigned in shuffled order
+    order = rng.permutation(len(pieces))
+    dev_cursor = int(rng.integers(0, 64))
+    dev_off = [0] * len(pieces)
+    for idx in order:
+        dev_off[idx] = dev_cursor
+        dev_cursor += pieces[idx][0] + int(rng.integers(0, 128))
+    rows = [(dev_off[i], p[1], p[0], p[2]) for i, p in enumerate(pieces)]
+    return rows, dev_cursor + 64, host_cursor + 64
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_descriptor_batches_match_oracle(backends, stream, seed):
+    """Both backends, both directions, on seeded random batches; bytes outside
+    the fragments must stay as they were."""
+    from pegaflow_amd.transfer import desc_array
+    rng = np.random.default_rng(7000 + seed)
+    rows4, dev_bytes, host_bytes = _random_batch(rng)
+    rows = [(d, h, s) for d, h, s, _a in rows4]
+    d = np.array([r[0] for r in rows4], dtype=np.uint64)
+    h = np.array([r[1] for r in rows4], dtype=np.uint64)
+    sz = np.array([r[2] for r in rows4], dtype=np.uint64)
+    al = np.array([r[3] for r in rows4], dtype=np.uint64)
+
+    def descs(dev, host):
+        return desc_array(dev.ptr + d, host.host_ptr + h, host.device_ptr + h, sz, 0, al)
+
+    for b in backends:
+        _run_both_directions(b, stream, descs, dev_bytes, host_bytes, rows, seed=seed)
