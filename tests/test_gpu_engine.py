@@ -616,3 +616,27 @@ def test_lease_of_another_instance_is_refused_without_being_consumed(engine):
     # consumed by its one worker (world size 1): a second load finds it gone
     with pytest.raises(_lib.StorageError, match="query lease is unknown or expired"):
         engine.batch_load_kv_blocks_multi_layer("inst-a", 0, 0, [["layer_0"]], lease, [[0, 1, 2, 3]])
+
+
+def test_partially_cached_save_stores_only_the_new_blocks(engine):
+    """engine_basic.rs:178-190 (dedupe) with a mixed list: hashes already in the
+    cache are skipped position by position, the rest keep their own block ids."""
+    layer = Layer("layer_0", 16, 1024)
+    register(engine, "partial-dedupe", [layer])
+    h = make_block_hashes(6, 80)
+    engine.batch_save_kv_blocks("partial-dedupe", 0, 0, 0, [LayerSave("layer_0", [0, 1, 2, 3], h[:4])])
+    used = engine.pool_usage()[0]
+    # h2, h3 again (from other device blocks: must NOT be re-read), h4, h5 new
+    engine.batch_save_kv_blocks("partial-dedupe", 0, 0, 0,
+                                [LayerSave("layer_0", [9, 8, 7, 6], [h[2], h[3], h[4], h[5]])])
+    assert engine.cached_blocks == 6
+    assert engine.pool_usage()[0] == used + 2 * 1024
+    layer.zero_gpu()
+    hits, lease = engine.query_prefix("partial-dedupe", h)
+    assert hits == 6
+    engine.batch_load_kv_blocks_multi_layer("partial-dedupe", 0, 0, [["layer_0"]], lease,
+                                            [[10, 11, 12, 13, 14, 15]]).wait()
+    want = np.zeros_like(layer.expected)
+    for dst, src in zip(range(10, 16), [0, 1, 2, 3, 7, 6]):
+        want[dst * 1024:(dst + 1) * 1024] = layer.expected[src * 1024:(src + 1) * 1024]
+    layer.assert_gpu_matches(want)
