@@ -22,6 +22,7 @@ line is the default workload).
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -537,11 +538,20 @@ def run_ref_transfer_bench(torch, np, args):
         for _ in range(warmup):
             fn()
             stream.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(iters):
-            fn()
-            stream.synchronize()
-        return nbytes * iters / (time.perf_counter() - t0) / 2 ** 30
+        # The interpreter's cyclic collector is paused while timing, as timeit does:
+        # with torch loaded one full collection takes about 40 ms, eight iterations
+        # of the largest case, and it falls into the same cell on every run.
+        gc.collect()
+        gc.disable()
+        try:
+            t0 = time.perf_counter()
+            for _ in range(iters):
+                fn()
+                stream.synchronize()
+            seconds = time.perf_counter() - t0
+        finally:
+            gc.enable()
+        return nbytes * iters / seconds / 2 ** 30
 
     rows = []
     for n in counts:

@@ -276,7 +276,8 @@ constexpr int kDescUnroll = 4;
 
 bool unroll_supported(int unroll) { return unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8; }
 
-int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipStream_t s);
+int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipStream_t s,
+                     uint32_t max_workgroups);
 
 int launch_block_units(const BlockUnit* units, uint32_t n_units, uint64_t max_tiles, bool to_far,
                        int unroll, uint32_t max_workgroups_x, hipStream_t s) {
@@ -415,13 +416,19 @@ int launch_plain_copy(void* dst, const void* src, uint64_t bytes, int unroll, hi
   return PF_OK;
 }
 
-int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipStream_t s) {
+int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipStream_t s,
+                     uint32_t max_workgroups) {
   if (n == 0) return PF_OK;
   constexpr uint64_t kTile = tile_bytes(kDescUnroll);
   uint64_t gx = n < kMaxGridX ? n : kMaxGridX;
   uint64_t gy = (max_size + kTile - 1) / kTile;
   if (gy < 1) gy = 1;
   if (gy > 64) gy = 64;
+  if (max_workgroups != 0) {
+    // The kernel strides over descriptors and tiles, so any grid covers the batch.
+    while (gx * gy > max_workgroups && gy > 1) gy >>= 1;
+    if (gx * gy > max_workgroups) gx = max_workgroups / gy ? max_workgroups / gy : 1;
+  }
   // Keep the launch to a few million workgroups; the kernel strides in both
   // dimensions, so a smaller grid only means more iterations per workgroup.
   while (gx * gy > (1ull << 22) && gy > 1) gy >>= 1;

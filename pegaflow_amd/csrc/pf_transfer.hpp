@@ -115,6 +115,8 @@ std::unique_ptr<TransferBackend> build_backend(TransferMode mode);
 
 // Launch the descriptor-table copy kernel: `table` is a device array of
 // 3*n u64 words [dst, src, size].  `max_size` is the largest size in it.
-int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipStream_t s);
+// `max_workgroups` caps the grid (0 = as many as the batch has tiles).
+int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipStream_t s,
+                     uint32_t max_workgroups = 0);
 
 }  // namespace pf
