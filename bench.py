@@ -84,6 +84,8 @@ def parse_args():
     ap.add_argument("--engine-child", action="store_true",
                     help="(internal) run only the engine section and print its JSON")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--ref-fragments", type=int, default=0,
+                    help="ref_transfer_bench: only this fragment count (default: 1024..65536)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--settle-max", type=int, default=8,
                     help="upper bound on the untimed passes run after the warmup until two agree")
@@ -317,6 +319,30 @@ def main():
                                      stream.handle))
     hbm_copy_gbps = 2 * time_copy(plain, reps=20)
 
+    # The same yardstick over the memory the gather and the scatter touch: one
+    # plain copy of a layer's payload from the head of each layer's cache into
+    # a staging-sized buffer, and back into each destination cache -- what the
+    # kernels would do if the block ids were 0..n-1 and the layout one segment.
+    # Copying one buffer pair over and over (above) is placement-dependent and
+    # comes out 5-10 % faster than a walk over 32 different caches.
+    def plain_over_layers(to_cache):
+        def once():
+            for li in range(n_layers):
+                cache = (dst_cache if to_cache else src_cache)[li].data_ptr()
+                a, b = (cache, scratch.data_ptr()) if to_cache else (scratch.data_ptr(), cache)
+                _lib.check(lib.pf_plain_copy(a, b, payload_per_layer, 0, stream.handle))
+        once()
+        stream.synchronize()
+        ev[0].record(stream)
+        for _ in range(3):
+            once()
+        ev[1].record(stream)
+        ev[1].synchronize()
+        return 2 * payload * 3 / (ev[0].elapsed_ms(ev[1]) / 1e3) / 1e9
+    assert payload_per_layer <= link_bytes
+    plain_gather_form = plain_over_layers(False)
+    plain_scatter_form = plain_over_layers(True)
+
     # ---- roofline of the dominant kernel (separate, untimed pass; in this pass
     # the copies share the kernels' stream, so every timed launch runs alone) ---
     xfer.set_kernel_timing(True)
@@ -344,7 +370,9 @@ def main():
                     "alg_bytes_per_launch": int(alg_bytes),
                     "save_kernel_gbps": round(2 * payload / (k_save_ms / 1e3) / 1e9, 1),
                     "load_kernel_gbps": round(2 * payload / (k_load_ms / 1e3) / 1e9, 1),
-                    "plain_copy_same_tile_gbps": round(hbm_copy_gbps, 1)}
+                    "plain_copy_same_tile_gbps": round(hbm_copy_gbps, 1),
+                    "plain_copy_over_layers_gbps": {"from_caches": round(plain_gather_form, 1),
+                                                    "into_caches": round(plain_scatter_form, 1)}}
     else:
         # zero-copy: the kernel touches HBM once per payload byte and is
         # bounded by the host link, not by HBM
@@ -511,7 +539,7 @@ def run_ref_transfer_bench(torch, np, args):
     from pegaflow_amd.transfer import (BlockTransfer, KernelBackend, LayerBlocks, MemcpyBackend,
                                        TransferPath, desc_array)
     seg, stride_factor, warmup, iters = 4096, 2, 3, 20
-    counts = [1024, 4096, 16384, 65536]
+    counts = [args.ref_fragments] if args.ref_fragments else [1024, 4096, 16384, 65536]
     dev = torch.device("cuda:0")
     max_n = max(counts)
     device_buf = torch.full((max_n * seg * stride_factor,), 0xA5, device=dev, dtype=torch.uint8)
@@ -587,7 +615,7 @@ def run_ref_transfer_bench(torch, np, args):
     if not np.array_equal(got, host.as_numpy()[:max_n * seg]):
         print("bench.py: device bytes differ from the host image", file=sys.stderr)
         sys.exit(1)
-    headline = next(r for r in rows if r["fragments"] == 65536 and r["layout"] == "shuffled")
+    headline = next(r for r in rows if r["fragments"] == max_n and r["layout"] == "shuffled")
     print(json.dumps({
         "metric": "descriptor backends at the shapes of the reference's transfer bench "
                   "(4 KiB fragments), GiB/s",
@@ -595,8 +623,8 @@ def run_ref_transfer_bench(torch, np, args):
         "warmup": warmup, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": "benches/transfer_h2d.rs shapes: 4 KiB fragments, "
-                               "1024..65536 per batch, contiguous/strided/shuffled, "
-                               "value = kernel backend, shuffled, 65536 fragments, H2D"},
+                               f"{counts[0]}..{max_n} per batch, contiguous/strided/shuffled, "
+                               f"value = kernel backend, shuffled, {max_n} fragments, H2D"},
         "table": rows}))
 
 
