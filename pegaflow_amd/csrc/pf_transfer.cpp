@@ -396,6 +396,13 @@ int KernelBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_
   uint64_t max_size = 0;
   for (uint64_t i = 0; i < n; ++i) {
     const CopyDesc& c = copies[i];
+    if (c.size != 0 && (c.device == 0 || c.host_device == 0)) {
+      // The kernel dereferences both addresses; a null one would fault the GPU.
+      return fail(PF_ERR_INVALID_ARGUMENT,
+                  "descriptor %llu: the kernel backend needs a device address and a "
+                  "device-visible host address",
+                  static_cast<unsigned long long>(i));
+    }
     table[3 * i + 0] = host_is_src ? c.device : c.host_device;
     table[3 * i + 1] = host_is_src ? c.host_device : c.device;
     table[3 * i + 2] = c.size;

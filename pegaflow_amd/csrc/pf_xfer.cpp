@@ -202,7 +202,11 @@ int Xfer::plan_layer(const pf_layer_blocks& in, size_t index, int path, LayerPla
         return fail(PF_ERR_INVALID_ARGUMENT, "layer %s: host segment %u is null", p.name.c_str(),
                     sgm);
       }
-      uint64_t need = (p.n_blocks - 1) * in.host_stride + p.frag_bytes;
+      uint64_t need = 0;
+      if (__builtin_mul_overflow(p.n_blocks - 1, in.host_stride, &need) ||
+          __builtin_add_overflow(need, p.frag_bytes, &need)) {
+        return fail(PF_ERR_INVALID_ARGUMENT, "layer %s: host image size overflows", p.name.c_str());
+      }
       if (need > in.host_len[sgm]) {
         return fail(PF_ERR_INVALID_ARGUMENT,
                     "layer %s: host segment %u needs %llu bytes, has %llu", p.name.c_str(), sgm,

@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 
 from oracle import oracle as O
+from pegaflow_amd import _lib
 from pegaflow_amd.runtime import DeviceBuffer, PinnedMemory, Stream
 from pegaflow_amd.transfer import CopyDesc, KernelBackend, MemcpyBackend
 from tests.helpers import kernel_test_pattern, random_bytes, xorshift_shuffle
@@ -59,6 +60,23 @@ def test_empty_batch_is_a_no_op(backends, stream):
         b.h2d([], stream)
         b.d2h([], stream)
     stream.synchronize()
+
+
+def test_kernel_backend_refuses_null_addresses(stream, gpu):
+    """A descriptor the kernel would dereference at address 0 is refused on the
+    host; zero-size descriptors carry no addresses worth checking."""
+    b = KernelBackend()
+    host = PinnedMemory(4096)
+    dev = DeviceBuffer(4096)
+    for desc in (CopyDesc(0, host.host_ptr, host.device_ptr, 64, 0, 1),
+                 CopyDesc(dev.ptr, host.host_ptr, 0, 64, 0, 1)):
+        with pytest.raises(_lib.InvalidArgument, match="descriptor 1: the kernel backend needs"):
+            b.d2h([CopyDesc(dev.ptr, host.host_ptr, host.device_ptr, 64, 0, 1), desc], stream)
+    b.d2h([CopyDesc(0, 0, 0, 0, 0, 0)], stream)
+    stream.synchronize()
+    b.close()
+    host.close()
+    dev.close()
 
 
 def _oracle_expect(dev0, host0, rows, host_is_src):

@@ -327,6 +327,39 @@ def test_worker_pool_matches_oracle(gpu, mode, use_desc):
     dev.close()
 
 
+@pytest.mark.parametrize("use_desc", [False, True], ids=["block_ids", "descriptors"])
+def test_worker_pool_split_cache_with_single_segment_host_blocks(gpu, use_desc):
+    """gpu_worker.rs:373-379: a split K/V cache moved to or from host blocks of
+    one segment puts V right behind K (`k_ptr + k.bytes`)."""
+    rng = np.random.default_rng(41)
+    nb, seg, n = 48, 4112, 17
+    cache0 = random_bytes(rng, 2 * nb * seg)
+    dev = DeviceBuffer(cache0.nbytes)
+    dev.copy_from_host(cache0)
+    host = PinnedMemory(2 * n * seg)
+    host.as_numpy()[:] = 0x5A
+    layout = KVCacheLayout(dev.ptr, cache0.nbytes, nb, seg, nb * seg, 2)
+    ids = rng.choice(nb, n, replace=False)
+    blocks = [HostBlock((host.host_ptr + i * 2 * seg,), (host.device_ptr + i * 2 * seg,), (7,),
+                        (2 * seg,)) for i in range(n)]
+    pool = GpuWorkerPool(0, -1, TransferMode.DIRECT, use_descriptor_backends=use_desc)
+    res = pool.batch_save([LayerTransferData("kv", layout, ids, blocks)]).wait()
+    assert res.done and res.bytes == 2 * n * seg
+    img = host.as_numpy().reshape(n, 2, seg)
+    kv = cache0.reshape(2, nb, seg)
+    assert np.array_equal(img[:, 0], kv[0, ids]) and np.array_equal(img[:, 1], kv[1, ids])
+    dest = rng.choice(nb, n, replace=False)
+    dev.fill(0x22)
+    pool.submit_load([LayerTransferData("kv", layout, dest, blocks)], None).wait()
+    want = np.full_like(kv, 0x22)
+    want[0, dest] = kv[0, ids]
+    want[1, dest] = kv[1, ids]
+    assert np.array_equal(dev.copy_to_host().reshape(2, nb, seg), want)
+    pool.close()
+    host.close()
+    dev.close()
+
+
 def test_worker_pool_init_failure_is_synchronous(gpu):
     with pytest.raises(_lib.PegaHipError, match="Failed to initialise GPU worker on device 99"):
         GpuWorkerPool(99)
