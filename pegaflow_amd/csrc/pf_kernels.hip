@@ -7,7 +7,7 @@
 //     loads before the first store so U global_load_dwordx4 are in flight per
 //     lane, and consecutive lanes touch consecutive 16-byte words, so each
 //     wavefront's access is one 1 KiB contiguous burst;
-//   * loads and stores are non-temporal: the data is touched once;
+//   * loads are non-temporal and stores "sc1 nt": the data is touched once;
 //   * all per-tile address arithmetic is wave-uniform (scalar registers).
 #include "pf_kernels.hpp"
 
@@ -30,14 +30,44 @@ typedef __attribute__((address_space(4))) const uint64_t c_u64;
 
 constexpr int kLanes = 256;
 
-// 16-byte global store with an explicit cache policy.  Measured on MI355X at
-// the Llama shape (5000 x 2 x 32 KiB gathered or scattered per launch) over
-// all 49 load x store policy pairs: a destination written in ascending
-// address order is written fastest with "sc1 nt" (gather 6.35 TB/s against
-// 6.30 for plain nt; scatter in ascending-id row order 6.17 against 5.63 for
-// "sc1" and 5.44 for an ordinary store).
-__device__ __forceinline__ void store16_sc1_nt(uint64_t dst, u32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(dst), "v"(v) : "memory");
+// 16-byte store with the cache policy "sc1 nt".  Measured on MI355X at the
+// Llama shape (5000 x 2 x 32 KiB gathered or scattered per launch) over all 49
+// load x store policy pairs: a destination written in ascending address order
+// is written fastest with "sc1 nt" (gather 6.35 TB/s against 6.30 for plain
+// nt; scatter in ascending-id row order 6.17 against 5.63 for "sc1" and 5.44
+// for an ordinary store).  Stores into mapped host memory want the same: every
+// policy with sc1 moves the Llama layer over the link at 56.3 GB/s (64
+// workgroups; hipMemcpyAsync on the same box 56.1), plain and sc0 stores at
+// 54.2, nt alone at 53.9; loads from host memory do not care (56.6 with any
+// policy).
+//
+// The policy bits are not reachable from a plain C++ store, and the store must
+// not be inline assembly: the compiler cannot see that an asm statement is a
+// 16-byte store, so it neither keeps the data registers alive for the wait
+// states such a store needs nor counts it for s_waitcnt.  (With the store
+// written as asm, a four-store tile loop had the address of the fourth store
+// computed into the data registers of the first two instructions after that
+// one was issued, and the first store wrote address bits into lanes 12-15 of
+// every 16-lane row.)  A raw buffer store carries the bits in its `aux`
+// operand and is an ordinary instruction to the compiler.  The descriptor
+// covers exactly the tile (wave-uniform base and byte count, no stride), so a
+// store beyond the tile would be dropped by the hardware's range check.
+constexpr int kAuxSc1Nt = (1 << 4) | (1 << 1);  // gfx940+: bit 4 = sc1, bit 1 = nt
+constexpr int kRawBufferWord3 = 0x00020000;     // untyped 32-bit data, no swizzle, no tid
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_descriptor(uint64_t base, uint32_t bytes) {
+  // The base is wave-uniform by construction; say so, or the compiler would
+  // loop over the lanes to build one descriptor per distinct value.
+  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(base));
+  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(base >> 32));
+  return __builtin_amdgcn_make_buffer_rsrc(
+      reinterpret_cast<void*>((static_cast<uint64_t>(hi) << 32) | lo), 0,
+      static_cast<int>(__builtin_amdgcn_readfirstlane(bytes)), kRawBufferWord3);
+}
+
+__device__ __forceinline__ void store16_sc1_nt(__amdgpu_buffer_rsrc_t tile, uint32_t offset,
+                                               u32x4 v) {
+  __builtin_amdgcn_raw_buffer_store_b128(v, tile, static_cast<int>(offset), 0, kAuxSc1Nt);
 }
 
 // Copy `bytes` <= U*4096 from src to dst; both 16-byte aligned.
@@ -46,13 +76,13 @@ __device__ __forceinline__ void copy_tile_vec(uint64_t dst, uint64_t src, uint32
   constexpr uint32_t kTile = U * kLanes * 16;
   const uint32_t lane = threadIdx.x;
   const g_u32x4* __restrict__ s = reinterpret_cast<const g_u32x4*>(src);
-  g_u32x4* __restrict__ d = reinterpret_cast<g_u32x4*>(dst);
   u32x4 v[U];
+  const __amdgpu_buffer_rsrc_t tile = tile_descriptor(dst, bytes & ~15u);
   if (bytes == kTile) {
 #pragma unroll
     for (int k = 0; k < U; ++k) v[k] = __builtin_nontemporal_load(s + lane + k * kLanes);
 #pragma unroll
-    for (int k = 0; k < U; ++k) __builtin_nontemporal_store(v[k], d + lane + k * kLanes);
+    for (int k = 0; k < U; ++k) store16_sc1_nt(tile, (lane + k * kLanes) * 16u, v[k]);
     return;
   }
   const uint32_t nvec = bytes >> 4;
@@ -64,7 +94,7 @@ __device__ __forceinline__ void copy_tile_vec(uint64_t dst, uint64_t src, uint32
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const uint32_t idx = lane + k * kLanes;
-    if (idx < nvec) __builtin_nontemporal_store(v[k], d + idx);
+    if (idx < nvec) store16_sc1_nt(tile, idx * 16u, v[k]);
   }
   // Fewer than 16 trailing bytes (fragment size not a multiple of 16).
   const uint32_t j = (nvec << 4) + lane;
@@ -220,11 +250,12 @@ __global__ __launch_bounds__(LT) void block_tiles_kernel(const BlockUnit* __rest
   if (up->vec_ok) {
     const g_u32x4* __restrict__ s = reinterpret_cast<const g_u32x4*>(src);
     const uint32_t nvec = bytes >> 4;
+    const __amdgpu_buffer_rsrc_t tile = tile_descriptor(dst, nvec << 4);
     if (lane < nvec) {
       // Gather: ordinary load of the scattered source; scatter: streaming
       // load of the staging side.  Both store streaming.
       const u32x4 v = TO_FAR ? s[lane] : __builtin_nontemporal_load(s + lane);
-      store16_sc1_nt(dst + lane * 16ull, v);
+      store16_sc1_nt(tile, lane * 16u, v);
     }
     const uint32_t j = (nvec << 4) + lane;
     if (j < bytes) reinterpret_cast<g_u8*>(dst)[j] = reinterpret_cast<const g_u8*>(src)[j];

@@ -43,7 +43,20 @@ int run(bool page_first,int mode,bool desc,bool blockwise,int nseg,int L,uint64_
     pf_task_result r; OK(pf_task_wait(t,-1,&r)); OK(pf_task_destroy(t));
     // verify
     for(int l=0;l<L;l++){ std::vector<uint8_t> got(layer_bytes); (void)hipMemcpy(got.data(),dst[l],layer_bytes,hipMemcpyDeviceToHost);
-      for(uint64_t i=0;i<n;i++){ if(dids[i]<0) continue; for(int s=0;s<nseg;s++){ if(memcmp(&got[s*nb*seg+dids[i]*seg],&host[l][s*nb*seg+ids[i]*seg],seg)){ printf("MISMATCH layer %d pos %llu\n",l,(unsigned long long)i); return 4;} } } }
+      uint64_t bad=0;
+      for(uint64_t i=0;i<n;i++){ if(dids[i]<0) continue; for(int s=0;s<nseg;s++){ const uint8_t* g=&got[s*nb*seg+dids[i]*seg]; const uint8_t* w=&host[l][s*nb*seg+ids[i]*seg];
+        if(memcmp(g,w,seg)){ if(bad++<4){ uint64_t at=0; while(g[at]==w[at]) ++at; uint64_t last=seg-1; while(g[last]==w[last]) --last;
+            // whose bytes are these?  another position of this layer, or nothing at all
+            long long other=-1; int other_seg=-1; for(uint64_t j=0;j<n&&other<0;j++) for(int t=0;t<nseg;t++) if(!memcmp(g+at,&host[l][t*nb*seg+ids[j]*seg+at],last-at+1)){ other=(long long)j; other_seg=t; break; }
+            bool zero=true; for(uint64_t k=at;k<=last;k++) if(g[k]){ zero=false; break; }
+            { printf("  dword map from byte %llu (one char per 16-byte lane word, bit i set = dword i differs):", (unsigned long long)(at&~15ull));
+              for(uint64_t k=at&~15ull;k<=last;k+=16){ int m=0; for(int d=0;d<4;d++) if(memcmp(g+k+4*d,w+k+4*d,4)) m|=1<<d; printf("%x",m);} printf("\n");
+              // does the first differing 16-byte word hold another fragment's bytes at the same offset?
+              uint64_t k0=at&~15ull; int d0=0; while(!memcmp(g+k0+4*d0,w+k0+4*d0,4)) ++d0;
+              for(int l2=0;l2<L;l2++) for(uint64_t j=0;j<nb;j++) for(int t=0;t<nseg;t++) if(!memcmp(g+k0+4*d0,&host[l2][t*nb*seg+j*seg+k0+4*d0],4)) printf("  first wrong dword equals source layer %d block id %llu segment %d at the same offset\n",l2,(unsigned long long)j,t);
+              printf("  first wrong dword %02x%02x%02x%02x wanted %02x%02x%02x%02x\n",g[k0+4*d0],g[k0+4*d0+1],g[k0+4*d0+2],g[k0+4*d0+3],w[k0+4*d0],w[k0+4*d0+1],w[k0+4*d0+2],w[k0+4*d0+3]); }
+            printf("MISMATCH rep %d layer %d segment %d pos %llu (src id %llu -> dst id %lld): bytes [%llu, %llu] differ; they are %s (pos %lld seg %d)\n",rep,l,s,(unsigned long long)i,(unsigned long long)ids[i],(long long)dids[i],(unsigned long long)at,(unsigned long long)last, zero?"zero":(other>=0?"another position's":"unknown"),other,other_seg); } } } }
+      if(bad){ printf("MISMATCH: %llu fragments of layer %d differ in rep %d\n",(unsigned long long)bad,l,rep); return 4; } }
     if(rep==1) pf_engine_evict_all(e);
   }
   OK(pf_engine_unregister_instance(e,"src")); OK(pf_engine_unregister_instance(e,"dst"));
