@@ -39,9 +39,9 @@ HBM_PEAK_GBPS = 8000.0      # MI355X published HBM3E bandwidth
 # WRITE_SIZE runs of this script: KiB per dispatch, scaled by what a plain copy
 # of exactly 1 GiB reads on the same counters (x2.000 and x1.000).
 MEASURED_TRAFFIC_STAGED = {
-    "llama8b": int((160401.7 * 2.000 + 320000.0 * 1.000) * 1024),
-    "llama70b_fp8": int((131713.4 * 2.000 + 262144.0 * 1.000) * 1024),
-    "dsv3_mla": int((249972.8 * 2.000 + 499712.0 * 1.000) * 1024),
+    "llama8b": int((160399.4 * 2.000 + 320000.0 * 1.000) * 1024),
+    "llama70b_fp8": int((131709.5 * 2.000 + 262144.0 * 1.000) * 1024),
+    "dsv3_mla": int((249954.4 * 2.000 + 499712.0 * 1.000) * 1024),
 }
 
 WORKLOADS = {
