@@ -58,3 +58,91 @@ def test_register_save_query_load_on_torch_tensors(kind, gpu):
             assert torch.equal(dst[n].view(torch.int16), want.view(torch.int16)), n
     finally:
         eng.close()
+
+
+@pytest.mark.parametrize("kind", ["kv_first", "mla_page_first"])
+def test_worker_connector_steps_over_a_real_engine(kind, gpu):
+    """Two workers (a prefill and a decode instance of one namespace) driven the
+    way vLLM drives them: metadata in, start_load_kv / wait_for_save per step,
+    get_finished polled until the requests are reported."""
+    import time
+
+    import torch
+
+    from pegaflow_amd.worker_connector import (ConnectorContext, InProcessEngineClient, LoadIntent,
+                                               PegaConnectorMetadata, SaveIntent, WorkerConnector)
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(11)
+    names = [f"model.layers.{i}.self_attn.attn" for i in range(4)]
+    if kind == "kv_first":
+        shape, is_mla, block_size, block_dim = (2, 96, 16, 8, 128), False, 16, 1
+    else:
+        shape, is_mla, block_size, block_dim = (96, 64, 576), True, 64, 0
+    src = {n: torch.randn(shape, device=dev, dtype=torch.bfloat16, generator=gen) for n in names}
+    dst = {n: torch.zeros(shape, device=dev, dtype=torch.bfloat16) for n in names}
+    torch.cuda.synchronize()
+    eng = PegaEngine(pool_size=64 << 20)
+    client = InProcessEngineClient(eng)
+
+    def worker_for(instance):
+        ctx = ConnectorContext(instance_id=instance, namespace="ns", block_size=block_size,
+                               tp_size=1, world_size=1, tp_rank=0, device_id=0,
+                               engine_client=client, is_mla=is_mla)
+        return WorkerConnector(ctx, device_synchronize=torch.cuda.synchronize)
+
+    def poll(worker, finished, which, want, seconds=20.0):
+        deadline = time.time() + seconds
+        seen = set()
+        while time.time() < deadline:
+            got = worker.get_finished(finished)[which]
+            finished = set()
+            seen |= got or set()
+            if seen == want:
+                return
+            time.sleep(0.002)
+        raise AssertionError(f"{want - seen} never reported")
+
+    prefill, decode = worker_for("prefill"), worker_for("decode")
+    try:
+        prefill.register_kv_caches(src)
+        decode.register_kv_caches(dst)
+        assert prefill._registered_layers == names and prefill._page_first == is_mla
+        # step 1: two requests finish prefill; request b holds the null block
+        hashes_a = [b"a%d" % i + bytes(6) for i in range(5)]
+        hashes_b = [b"b%d" % i + bytes(6) for i in range(3)]
+        step = PegaConnectorMetadata(save_intents={
+            "a": SaveIntent(((7, 3, 50, 51, 9),), tuple(hashes_a)),
+            "b": SaveIntent(((0, 20, 21),), tuple(hashes_b))})
+        prefill.start_load_kv(step)
+        prefill.save_kv_layer(step, names[0], src[names[0]], None)     # per-layer hook: nothing
+        prefill.wait_for_save()
+        poll(prefill, {"a", "b"}, 0, {"a", "b"})
+        assert eng.cached_blocks == 7                                # b's null block was dropped
+        # step 2: the scheduler side queries, the decode worker loads
+        hits, lease = client.query("decode", hashes_a)
+        assert hits == 5
+        hits_b, lease_b = client.query("decode", hashes_b)
+        assert hits_b == 0 and lease_b == b""                          # b's first block was never stored
+        dest = (60, 61, None, 63, 64)
+        decode.start_load_kv(PegaConnectorMetadata(load_intents={
+            "a": LoadIntent((dest,), (lease,), num_tokens=5 * block_size)}))
+        decode.wait_for_layer_load(names[0])
+        poll(decode, set(), 1, {"a"})
+        assert decode.get_block_ids_with_load_errors() == set()
+        src_ids = torch.tensor([7, 3, 51, 9], device=dev)
+        dst_ids = torch.tensor([60, 61, 63, 64], device=dev)
+        for n in names:
+            want = torch.zeros_like(src[n])
+            want.index_copy_(block_dim, dst_ids, src[n].index_select(block_dim, src_ids))
+            assert torch.equal(dst[n].view(torch.int16), want.view(torch.int16)), n
+        # step 3: a lease the engine does not know fails the load call; vLLM is told to recompute
+        decode.start_load_kv(PegaConnectorMetadata(load_intents={
+            "c": LoadIntent(((70, 71),), (client.lease_token(987654),), num_tokens=2 * block_size)}))
+        assert decode.get_block_ids_with_load_errors() == {70, 71}
+        assert decode.get_finished(set())[1] == {"c"}
+    finally:
+        prefill.shutdown()
+        decode.shutdown()
+        eng.close()
