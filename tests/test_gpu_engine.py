@@ -604,6 +604,65 @@ def test_recurrent_group_seals_final_block_save(engine):
     state.close()
 
 
+def test_single_group_instances_are_unaffected(engine):
+    """hybrid_groups.rs:181-211: membership on an instance without layer groups
+    answers for group 0; a group the instance does not have is an error, not an
+    all-miss answer."""
+    layers = [Layer("layer_0", 4, 1024), Layer("layer_1", 4, 1024)]
+    register(engine, "hybrid-compat", layers, ns="hybrid-compat-ns")
+    hashes = make_block_hashes(4, 7)
+    engine.batch_save_kv_blocks("hybrid-compat", 0, 0, 0,
+                                [LayerSave(l.name, [0, 1], hashes[:2]) for l in layers])
+    assert engine.query_group_membership("hybrid-compat", 0, hashes) == [True, True, False, False]
+    with pytest.raises(_lib.InvalidArgument):
+        engine.query_group_membership("hybrid-compat", 7, hashes[:1])
+
+
+def test_recurrent_membership_is_an_exact_want_set(engine):
+    """hybrid_groups.rs:221-322: a recurrent want-set resolves only when every
+    member is stored in that group; a set with an absent member comes back
+    short and cannot be leased; a hash stored under the attention group alone
+    never satisfies the recurrent set."""
+    layers = [Layer("attn_0", 8, 1024), Layer("recurrent_state", 8, 2048, overwrite=5)]
+    register(engine, "hybrid-pd", layers, ns="hybrid-pd-ns", groups=[0, 1])
+    hashes = make_block_hashes(8, 21)
+    engine.batch_save_kv_blocks("hybrid-pd", 0, 0, 0, [LayerSave("attn_0", [0, 1, 2], hashes[:3])])
+    engine.batch_save_kv_blocks("hybrid-pd", 0, 0, 0,
+                                [LayerSave("recurrent_state", [4, 5], [hashes[1], hashes[2]])])
+    want = [hashes[1], hashes[2]]
+    assert engine.query_group_membership("hybrid-pd", 1, want) == [True, True]
+    lease = engine.create_group_lease("hybrid-pd", 1, want)          # complete set: leasable
+    short = [hashes[1], hashes[5], hashes[2]]
+    assert engine.query_group_membership("hybrid-pd", 1, short) == [True, False, True]
+    with pytest.raises(_lib.StorageError, match="block 1 of the lease is not resident in group 1"):
+        engine.create_group_lease("hybrid-pd", 1, short)
+    assert engine.query_group_membership("hybrid-pd", 1, [hashes[0]]) == [False]
+    assert engine.query_group_membership("hybrid-pd", 0, [hashes[0]]) == [True]
+    # the leased checkpoints load in the requested order
+    layers[1].zero_gpu()
+    engine.batch_load_multi("hybrid-pd", 0, 0, [["attn_0"], ["recurrent_state"]],
+                            [(lease, [[None, None], [6, 7]])]).wait()
+    want_bytes = np.zeros_like(layers[1].expected)
+    want_bytes[6 * 2048:8 * 2048] = layers[1].expected[4 * 2048:6 * 2048]
+    layers[1].assert_gpu_matches(want_bytes)
+
+
+def test_save_query_load_roundtrip_with_numa(gpu):
+    """engine_basic.rs:160-176: the same round trip with one pinned pool per NUMA node."""
+    e = PegaEngine(pool_size=64 << 20, numa_aware=True)
+    layer = Layer("layer_0", 4, 1024)
+    register(e, "test-roundtrip-numa", [layer])
+    hashes = make_block_hashes(4, 0)
+    e.batch_save_kv_blocks("test-roundtrip-numa", 0, 0, 0, [LayerSave("layer_0", [0, 1, 2, 3], hashes)])
+    layer.zero_gpu()
+    hits, lease = e.query_prefix("test-roundtrip-numa", hashes)
+    assert hits == 4
+    e.batch_load_kv_blocks_multi_layer("test-roundtrip-numa", 0, 0, [["layer_0"]], lease,
+                                       [[0, 1, 2, 3]]).wait()
+    layer.assert_gpu_matches(layer.expected)
+    e.close()
+
+
 def test_namespace_isolation(engine):
     """engine_basic.rs:254-271: blocks of one namespace are invisible to another."""
     a, b = Layer("layer_0", 4, 1024), Layer("layer_0", 4, 1024)
