@@ -11,19 +11,25 @@ from .connector import (  # noqa: F401
     KVCacheRegistrationInfo,
     assemble_layer_saves,
     block_shard,
+    derive_namespace,
     infer_kv_cache_registration,
+    reconcile_hybrid_hit,
     register_kv_caches,
     registration_tensor,
     resolve_transfer_backend,
+    storage_group_ids,
 )
 
 __all__ = [
     "KVCacheRegistrationInfo",
     "assemble_layer_saves",
     "block_shard",
+    "derive_namespace",
     "infer_kv_cache_registration",
+    "reconcile_hybrid_hit",
     "register_kv_caches",
     "registration_tensor",
     "resolve_transfer_backend",
+    "storage_group_ids",
 ]
 __version__ = "0.1.0"

@@ -235,3 +235,73 @@ def assemble_layer_saves(save_intents, registered_layers, *, layer_to_group=None
             entry[0].extend(ids)
             entry[1].extend(hashes)
     return [(name, ids, hashes) for name, (ids, hashes) in saves.items()]
+
+
+# ---------------------------------------------------------------------------
+# Scheduler-side facts that decide what the worker is asked to move
+# (python/pegaflow/connector/common.py): the storage namespace, the storage
+# group of each cache group, and how a hybrid model's per-group query results
+# combine into one resumable prefix.
+# ---------------------------------------------------------------------------
+
+def storage_group_ids(group_is_recurrent) -> tuple[int, ...]:
+    """Engine storage group of every connector cache group (common.py:405-415):
+    attention-like groups share storage group 0, recurrent groups are numbered
+    1, 2, ... in cache-group order, wherever the attention group sits."""
+    ids, next_recurrent = [], 1
+    for recurrent in group_is_recurrent:
+        if recurrent:
+            ids.append(next_recurrent)
+            next_recurrent += 1
+        else:
+            ids.append(0)
+    return tuple(ids)
+
+
+def reconcile_hybrid_hit(attention_hit_blocks: int, recurrent_hits):
+    """One hit for a hybrid (attention + recurrent state) model
+    (common.py:252-286).  ``recurrent_hits[g][s]`` = query positions whose
+    checkpoint is stored in recurrent group ``g`` on TP shard ``s``.  A position
+    is a legal resume point when it lies inside the attention prefix and every
+    group holds it on every shard; the hit is the rightmost such position plus
+    one block.  Returns ``(hit_blocks, checkpoint, usable_positions)``;
+    ``(0, None, frozenset())`` when the prefix cannot be resumed."""
+    nothing = (0, None, frozenset())
+    if attention_hit_blocks <= 0 or not recurrent_hits:
+        return nothing
+    shard_sets = [frozenset(p for p in shard if p < attention_hit_blocks)
+                  for group in recurrent_hits for shard in group]
+    if not shard_sets:
+        return nothing
+    usable = frozenset.intersection(*shard_sets)
+    if not usable:
+        return nothing
+    checkpoint = max(usable)
+    return checkpoint + 1, checkpoint, usable
+
+
+def derive_namespace(vllm_config, tp_size: int, dcp_world_size: int = 1, pcp_world_size: int = 1,
+                     cross_layer_blocks: bool = False) -> str:
+    """Storage namespace of a deployment (common.py:519-566): eight hex digits
+    of SHA-256 over every setting that changes how a block is laid out in
+    storage, so that two incompatible layouts can never answer each other's
+    queries.  ``vllm_config`` is vLLM's config object (only attributes are read)."""
+    import hashlib
+    model, cache = vllm_config.model_config, vllm_config.cache_config
+    extra = getattr(vllm_config, "additional_config", None) or {}
+    factors = {
+        "model": model.model,
+        "dtype": str(model.dtype),
+        "tp_size": tp_size,
+        "pp_size": vllm_config.parallel_config.pipeline_parallel_size,
+        "num_kv_heads": model.get_total_num_kv_heads(),
+        "head_size": model.get_head_size(),
+        "num_hidden_layers": model.get_total_num_hidden_layers(),
+        "cache_dtype": str(cache.cache_dtype),
+        "is_hma_enabled": not vllm_config.scheduler_config.disable_hybrid_kv_cache_manager,
+        "dcp_world_size": dcp_world_size,
+        "pcp_world_size": pcp_world_size,
+        "cross_layer_blocks": cross_layer_blocks,
+        "mla_layer_split_kv_cache": bool(extra.get("mla_layer_split_kv_cache", False)),
+    }
+    return hashlib.sha256(str(sorted(factors.items())).encode()).hexdigest()[:8]

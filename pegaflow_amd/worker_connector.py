@@ -26,7 +26,7 @@ import time
 from dataclasses import dataclass, field
 from typing import Any, Iterable, Sequence
 
-from .connector import assemble_layer_saves, register_kv_caches
+from .connector import assemble_layer_saves, register_kv_caches, storage_group_ids
 from .engine import LayerSave, LoadState, PegaEngine
 
 logger = logging.getLogger("pegaflow_amd.connector")
@@ -86,6 +86,20 @@ class CacheGroups:
     @property
     def has_recurrent_state(self) -> bool:
         return bool(self.recurrent_group_indices)
+
+    @property
+    def storage_group_ids(self) -> tuple[int, ...]:
+        return storage_group_ids(index in self.recurrent_group_indices
+                                 for index in range(self.group_count))
+
+    def storage_group_of(self, group_index: int) -> int:
+        return self.storage_group_ids[group_index]
+
+    @property
+    def hash_group_index(self) -> int:
+        """The attention group, whose block hashes key the whole request."""
+        return next(index for index in range(self.group_count)
+                    if index not in self.recurrent_group_indices)
 
     def layer_to_group(self) -> dict[str, int]:
         owner: dict[str, int] = {}

@@ -135,3 +135,68 @@ def test_registration_tensor_accepts_shared_recurrent_states():
         registration_tensor((conv, storage.as_strided((8, 8), (12, 1), 16)))
     with pytest.raises(TypeError):
         registration_tensor(())
+
+
+# ---- hybrid hit, storage groups, namespace ------------------------------------
+# python/tests/test_hybrid_reconcile.py:38-140 and test_derive_namespace.py:48-72
+
+from types import SimpleNamespace  # noqa: E402
+
+from pegaflow_amd.connector import (derive_namespace, reconcile_hybrid_hit,  # noqa: E402
+                                    storage_group_ids)
+
+
+@pytest.mark.parametrize("attn,recurrent,want", [
+    (3, (((2,),),), (3, 2, {2})),                       # rightmost checkpoint within the prefix
+    (2, (((2,),),), (0, None, set())),                  # checkpoint beyond the attention prefix
+    (3, (((),),), (0, None, set())),                    # attention alone cannot resume
+    (4, (((1, 2), (2, 3)),), (3, 2, {2})),              # shards must agree on the boundary
+    (3, (((0, 2),), ((1, 2),)), (3, 2, {2})),           # every recurrent group must hold it
+    (3, (((0, 2),), ((1,),)), (0, None, set())),
+    (3, (((0, 2),),), (3, 2, {0, 2})),                  # a gap below the rightmost hit is fine
+    (0, (((0,),),), (0, None, set())),                  # no attention prefix, no hit
+    (4, (((1, 3),),), (4, 3, {1, 3})),                  # earlier boundary kept for re-derivation
+    (3, (), (0, None, set())),
+])
+def test_reconcile_hybrid_hit(attn, recurrent, want):
+    hit, checkpoint, usable = reconcile_hybrid_hit(attn, recurrent)
+    assert (hit, checkpoint, set(usable)) == want
+    assert isinstance(usable, frozenset)
+
+
+def test_storage_group_ids():
+    assert storage_group_ids([False, True]) == (0, 1)            # attention first
+    assert storage_group_ids([True, False]) == (1, 0)            # recurrent group can come first
+    assert storage_group_ids([False]) == (0,)
+    assert storage_group_ids([False, True, True]) == (0, 1, 2)   # dense ids for several recurrent groups
+    from pegaflow_amd.worker_connector import CacheGroups
+    groups = CacheGroups((("mamba",), ("attn",)), frozenset({0}))
+    assert groups.storage_group_ids == (1, 0) and groups.hash_group_index == 1
+    assert groups.storage_group_of(0) == 1
+
+
+def _vllm_config(pp_size=1, mla_layer_split=False, disable_hma=False):
+    model = SimpleNamespace(model="/data/models/GLM-5.2-FP8", dtype="bfloat16",
+                            get_total_num_kv_heads=lambda: 1, get_head_size=lambda: 576,
+                            get_total_num_hidden_layers=lambda: 78)
+    return SimpleNamespace(
+        model_config=model, cache_config=SimpleNamespace(cache_dtype="fp8"),
+        scheduler_config=SimpleNamespace(disable_hybrid_kv_cache_manager=disable_hma),
+        parallel_config=SimpleNamespace(pipeline_parallel_size=pp_size),
+        additional_config={"mla_layer_split_kv_cache": mla_layer_split})
+
+
+def test_namespace_separates_incompatible_layouts():
+    ns = lambda **kw: derive_namespace(_vllm_config(**kw), tp_size=8)  # noqa: E731
+    assert ns(pp_size=1) != ns(pp_size=8)
+    assert ns(mla_layer_split=False) != ns(mla_layer_split=True)
+    assert ns(disable_hma=False) != ns(disable_hma=True)
+    assert ns(pp_size=4, mla_layer_split=True) == ns(pp_size=4, mla_layer_split=True)
+    cfg = _vllm_config(pp_size=4)
+    cfg.additional_config = None
+    assert derive_namespace(cfg, tp_size=8) == ns(pp_size=4, mla_layer_split=False)
+    assert derive_namespace(_vllm_config(), tp_size=8) != derive_namespace(_vllm_config(), tp_size=4)
+    assert derive_namespace(_vllm_config(), 8, dcp_world_size=2) != ns()
+    assert derive_namespace(_vllm_config(), 8, cross_layer_blocks=True) != ns()
+    value = ns()
+    assert len(value) == 8 and int(value, 16) >= 0
