@@ -209,3 +209,68 @@ def test_full_size_round_trip_properties(name, path, torch_dev):
         pool.close()
         del src, dst
         torch.cuda.empty_cache()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", ["llama8b", "llama70b_fp8", "dsv3_mla"])
+@pytest.mark.parametrize("backend_name", ["kernel", "direct"])
+def test_full_fragment_sizes_through_the_descriptor_backends(backend_name, shape, torch_dev):
+    """The reference-compatible backends at the fragment sizes and counts of
+    the benchmark shapes (8 layers of each): one descriptor per fragment, K
+    before V, device -> host, then host -> device into other slots; every
+    block of every layer is compared on the device."""
+    from pegaflow_amd.transfer import KernelBackend, MemcpyBackend, desc_array
+    torch = torch_dev
+    _, nb, seg, nseg, n, id_kind, _ = FULL[shape]
+    layers = 8
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(4321)
+    src = [torch.empty(nseg * nb * seg, device=dev, dtype=torch.uint8).random_(0, 256, generator=gen)
+           for _ in range(layers)]
+    dst = [torch.zeros(nseg * nb * seg, device=dev, dtype=torch.uint8) for _ in range(layers)]
+    save_ids = make_ids(np, id_kind, nb, n, 0).astype(np.uint64)
+    load_ids = make_ids(np, "permutation", nb, n, 1).astype(np.uint64)
+    pool = PinnedMemory(layers * nseg * n * seg)
+    torch.cuda.synchronize()
+    stream = Stream()
+    backend = KernelBackend() if backend_name == "kernel" else MemcpyBackend()
+    pos = np.arange(n, dtype=np.uint64)
+
+    def descriptors(tensors, ids):
+        """[layer][block][segment] order, as build_copy_descs emits them."""
+        per_layer = []
+        for li, t in enumerate(tensors):
+            rows = np.empty((n, nseg, 6), dtype=np.uint64)
+            for s in range(nseg):
+                host_off = (li * nseg + s) * n * seg + pos * seg
+                rows[:, s, 0] = t.data_ptr() + s * nb * seg + ids * seg
+                rows[:, s, 1] = pool.host_ptr + host_off
+                rows[:, s, 2] = pool.device_ptr + host_off
+                rows[:, s, 3] = seg
+                rows[:, s, 4] = li
+                rows[:, s, 5] = 1 + li * nseg + s       # one allocation per layer segment
+            per_layer.append(rows.reshape(n * nseg, 6))
+        rows = np.concatenate(per_layer)
+        return desc_array(rows[:, 0], rows[:, 1], rows[:, 2], rows[:, 3], rows[:, 4], rows[:, 5])
+
+    try:
+        backend.d2h(descriptors(src, save_ids), stream)
+        backend.h2d(descriptors(dst, load_ids), stream)
+        stream.synchronize()
+        sid = torch.from_numpy(save_ids.astype(np.int64)).to(dev)
+        lid = torch.from_numpy(load_ids.astype(np.int64)).to(dev)
+        untouched = torch.ones(nb, dtype=torch.bool, device=dev)
+        untouched[lid] = False
+        rest = torch.nonzero(untouched).reshape(-1)
+        for li in range(layers):
+            s = src[li].view(nseg, nb, seg)
+            d = dst[li].view(nseg, nb, seg)
+            assert torch.equal(d[:, lid], s[:, sid]), f"{shape} layer {li}: moved blocks differ"
+            assert not bool(d[:, rest].any()), f"{shape} layer {li}: a block outside the list changed"
+    finally:
+        backend.close()
+        stream.close()
+        pool.close()
+        del src, dst
+        torch.cuda.empty_cache()
