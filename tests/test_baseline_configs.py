@@ -274,3 +274,74 @@ def test_full_fragment_sizes_through_the_descriptor_backends(backend_name, shape
         pool.close()
         del src, dst
         torch.cuda.empty_cache()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("config,path", [
+    (dict(tile_unroll=1), TransferPath.ZEROCOPY),
+    (dict(tile_unroll=2), TransferPath.ZEROCOPY),
+    (dict(tile_unroll=8), TransferPath.ZEROCOPY),
+    (dict(zerocopy_max_workgroups=8), TransferPath.ZEROCOPY),
+    (dict(zerocopy_max_workgroups=4096), TransferPath.ZEROCOPY),
+    (dict(staging_slot_bytes=48 << 20), TransferPath.STAGED),               # five units per layer
+    (dict(staging_slot_bytes=48 << 20, staging_slots=3, copy_stream=1), TransferPath.STAGED),
+    (dict(staging_slot_bytes=48 << 20, copy_stream=2), TransferPath.STAGED),
+    (dict(copy_stream=1), TransferPath.STAGED),
+    (dict(auto_staged_min_bytes=1 << 40), TransferPath.AUTO),               # never staged
+    (dict(auto_staged_min_bytes=1 << 20), TransferPath.AUTO),               # staged from 1 MiB
+], ids=lambda v: ",".join(f"{k}={x}" for k, x in v.items()) if isinstance(v, dict) else str(int(v)))
+def test_engine_options_do_not_change_the_bytes(config, path, torch_dev):
+    """Every option of the block-ID engine (tile size of the zero-copy kernel,
+    its workgroup cap, staging slot size and count, where the link copies run,
+    the AUTO threshold) on 4 layers x 3000 blocks of the Llama shape: the same
+    blocks land in the same places."""
+    torch = torch_dev
+    layers, nb, seg, nseg, n = 4, 8192, 32768, 2, 3000
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(99)
+    src = [torch.empty(nseg * nb * seg, device=dev, dtype=torch.uint8).random_(0, 256, generator=gen)
+           for _ in range(layers)]
+    dst = [torch.zeros(nseg * nb * seg, device=dev, dtype=torch.uint8) for _ in range(layers)]
+    save_ids = make_ids(np, "permutation", nb, n, 5)
+    load_ids = make_ids(np, "permutation", nb, n, 6)
+    buf = n * seg
+    pool = PinnedMemory(layers * nseg * buf)
+    torch.cuda.synchronize()
+    stream, xfer = Stream(), BlockTransfer(**config)
+
+    def blocks(tensors, ids):
+        return [LayerBlocks(
+            layout=KVCacheLayout(t.data_ptr(), nseg * nb * seg, nb, seg, nb * seg, nseg),
+            block_ids=ids,
+            host=tuple(pool.host_ptr + (li * nseg + s) * buf for s in range(nseg)),
+            host_device=tuple(pool.device_ptr + (li * nseg + s) * buf for s in range(nseg)),
+            host_len=(buf, buf), host_stride=seg, layer_name=f"layer{li}")
+            for li, t in enumerate(tensors)]
+
+    try:
+        xfer.save(blocks(src, save_ids), stream, path)
+        xfer.load(blocks(dst, load_ids), stream, path)
+        stream.synchronize()
+        if "auto_staged_min_bytes" in config:
+            staged = config["auto_staged_min_bytes"] <= nseg * buf
+            assert xfer.last_path == (TransferPath.STAGED if staged else TransferPath.ZEROCOPY)
+        sid = torch.from_numpy(save_ids.astype(np.int64)).to(dev)
+        lid = torch.from_numpy(load_ids.astype(np.int64)).to(dev)
+        untouched = torch.ones(nb, dtype=torch.bool, device=dev)
+        untouched[lid] = False
+        rest = torch.nonzero(untouched).reshape(-1)
+        img = torch.from_numpy(pool.as_numpy())
+        for li in range(layers):
+            s = src[li].view(nseg, nb, seg)
+            d = dst[li].view(nseg, nb, seg)
+            assert torch.equal(d[:, lid], s[:, sid]), f"layer {li}: moved blocks differ"
+            assert not bool(d[:, rest].any()), f"layer {li}: a block outside the list changed"
+            got = img[li * nseg * buf:(li + 1) * nseg * buf].view(nseg, n, seg)
+            assert torch.equal(got, s[:, sid].cpu()), f"layer {li}: host image"
+    finally:
+        xfer.close()
+        stream.close()
+        pool.close()
+        del src, dst
+        torch.cuda.empty_cache()
