@@ -3,7 +3,8 @@
 // from C++ with nothing but include/pegahip.h and the HIP runtime, over both
 // transfer modes, both worker forms (block ids / descriptors), blockwise
 // allocation, page-first pages small (zero-copy) and large (whole-page
-// staging), and a 20-layer task whose load is converted in two parts.
+// staging), a 20-layer task whose load is converted in two parts, and 160 MiB
+// layers through every worker form.
 // Built by `make -C pegaflow_amd/csrc native-tests`; run by
 // tests/test_gpu_native.py.  Exit status 0 and a last line "all ok" = pass.
 #include "../../include/pegahip.h"
@@ -74,5 +75,8 @@ int main(){
   rc|=run(true,1,false,false,1,5,128,8192,60,64);
   rc|=run(true,0,false,false,1,5,2048,65536,1500,1200);   // page-first, whole-page staging (>64 MiB)
   rc|=run(false,0,false,false,2,20,4096,32768,2500,4000); // staged, two-part conversion on load
+  rc|=run(false,1,false,false,2,8,4096,32768,2500,2000);  // kernel mode at the same size: zero-copy both ways
+  rc|=run(false,0,true,false,2,8,4096,32768,2500,2000);   // per-fragment descriptors, direct backend, 40 000 per task
+  rc|=run(false,1,true,false,2,8,4096,32768,2500,2000);   // per-fragment descriptors, kernel backend
   printf(rc?"FAILED\n":"all ok\n"); return rc;
 }
