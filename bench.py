@@ -227,6 +227,12 @@ def main():
     stream = Stream()
     ev = [Event(timing=True) for _ in range(4)]
 
+    # Every gather / scatter launch of the timed steps is bracketed by HIP events
+    # on the stream it runs on (the streams are left as they are); the figures
+    # add up over a step and are read after the step's synchronise.
+    xfer.set_kernel_timing(2)
+    live = {"ms": 0.0, "launches": 0}
+
     def one_step():
         """save pass + load pass; returns (save_ms, load_ms) from stream events."""
         ev[0].record(stream)
@@ -235,6 +241,8 @@ def main():
         xfer.load(load_layers, stream, path)
         ev[2].record(stream)
         ev[2].synchronize()
+        k_ms, k_n = xfer.last_kernel_ms()
+        live["ms"], live["launches"] = live["ms"] + k_ms, live["launches"] + k_n
         return ev[0].elapsed_ms(ev[1]), ev[1].elapsed_ms(ev[2])
 
     for _ in range(args.warmup):
@@ -254,6 +262,7 @@ def main():
     stream.synchronize()
     save_ms = load_ms = 0.0
     step_times = []
+    live["ms"], live["launches"] = 0.0, 0
     t_start = time.perf_counter()
     for _ in range(args.steps):
         s_ms, l_ms = one_step()
@@ -263,6 +272,9 @@ def main():
     stream.synchronize()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t_start
+    xfer.set_kernel_timing(0)
+    live_launch_ms = live["ms"] / max(live["launches"], 1)
+    live_launches_per_step = live["launches"] // max(args.steps, 1)
     used_path = "staged" if xfer.last_path == TransferPath.STAGED else "zerocopy"
 
     step_bytes = 2 * payload
@@ -343,47 +355,49 @@ def main():
     plain_gather_form = plain_over_layers(False)
     plain_scatter_form = plain_over_layers(True)
 
-    # ---- roofline of the dominant kernel (separate, untimed pass; in this pass
-    # the copies share the kernels' stream, so every timed launch runs alone) ---
-    xfer.set_kernel_timing(True)
+    # ---- roofline of the dominant kernel ------------------------------------
+    # `achieved` comes from the events around every launch of the timed steps
+    # (above).  A second, untimed pass times the launches running alone (the link
+    # copies share the kernels' stream in that mode) and splits them by direction.
+    xfer.set_kernel_timing(1)
     xfer.save(save_layers, stream, path)
     stream.synchronize()
     k_save_ms, k_save_n = xfer.last_kernel_ms()
     xfer.load(load_layers, stream, path)
     stream.synchronize()
     k_load_ms, k_load_n = xfer.last_kernel_ms()
-    xfer.set_kernel_timing(False)
-    launches = k_save_n + k_load_n
-    avg_launch_ms = (k_save_ms + k_load_ms) / max(launches, 1)
+    xfer.set_kernel_timing(0)
+    alone_launches = k_save_n + k_load_n
+    alone_launch_ms = (k_save_ms + k_load_ms) / max(alone_launches, 1)
+    launches = live_launches_per_step
+    assert launches == alone_launches, (launches, alone_launches)
     bytes_per_launch = 2 * payload / max(launches, 1)          # payload bytes one launch moves
     default_shape = not args.layers and not args.slot_mb
-    if used_path == "staged":
-        # device gather/scatter: every payload byte is read once and written
-        # once in HBM -> 2 x payload algorithmic bytes per launch
-        alg_bytes = 2 * bytes_per_launch
-        achieved = alg_bytes / (avg_launch_ms / 1e3) / 1e9
-        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                    "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                    "traffic": MEASURED_TRAFFIC_STAGED[args.workload] if default_shape else None,
-                    "kernel": "block_tiles_kernel (staged gather/scatter)",
-                    "launches": launches, "avg_launch_us": round(avg_launch_ms * 1e3, 2),
-                    "alg_bytes_per_launch": int(alg_bytes),
-                    "save_kernel_gbps": round(2 * payload / (k_save_ms / 1e3) / 1e9, 1),
-                    "load_kernel_gbps": round(2 * payload / (k_load_ms / 1e3) / 1e9, 1),
-                    "plain_copy_same_tile_gbps": round(hbm_copy_gbps, 1),
-                    "plain_copy_over_layers_gbps": {"from_caches": round(plain_gather_form, 1),
-                                                    "into_caches": round(plain_scatter_form, 1)}}
-    else:
-        # zero-copy: the kernel touches HBM once per payload byte and is
-        # bounded by the host link, not by HBM
-        alg_bytes = bytes_per_launch
-        achieved = alg_bytes / (avg_launch_ms / 1e3) / 1e9
-        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                    "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                    "kernel": "block_units_kernel (zero-copy, host-link bound)",
-                    "launches": launches, "avg_launch_us": round(avg_launch_ms * 1e3, 2),
-                    "alg_bytes_per_launch": int(alg_bytes),
-                    "plain_copy_same_tile_gbps": round(hbm_copy_gbps, 1)}
+    # staged: every payload byte is read once and written once in HBM -> 2 x
+    # payload algorithmic bytes per launch; zero-copy: the kernel touches HBM
+    # once per payload byte and is bounded by the host link, not by HBM
+    staged_path = used_path == "staged"
+    alg_bytes = (2 if staged_path else 1) * bytes_per_launch
+    achieved = alg_bytes / (live_launch_ms / 1e3) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                "traffic": (MEASURED_TRAFFIC_STAGED[args.workload]
+                            if staged_path and default_shape else None),
+                "kernel": ("block_tiles_kernel (staged gather/scatter)" if staged_path
+                           else "block_units_kernel (zero-copy, host-link bound)"),
+                "measured": f"HIP events around each of the {live['launches']} launches of the "
+                            f"{args.steps} timed steps",
+                "launches": launches, "avg_launch_us": round(live_launch_ms * 1e3, 2),
+                "alg_bytes_per_launch": int(alg_bytes),
+                "launches_alone": {
+                    "avg_launch_us": round(alone_launch_ms * 1e3, 2),
+                    "achieved": round(alg_bytes / (alone_launch_ms / 1e3) / 1e9, 1),
+                    "save_kernel_gbps": round(alg_bytes * k_save_n / (k_save_ms / 1e3) / 1e9, 1),
+                    "load_kernel_gbps": round(alg_bytes * k_load_n / (k_load_ms / 1e3) / 1e9, 1)},
+                "plain_copy_same_tile_gbps": round(hbm_copy_gbps, 1)}
+    if staged_path:
+        roofline["plain_copy_over_layers_gbps"] = {"from_caches": round(plain_gather_form, 1),
+                                                   "into_caches": round(plain_scatter_form, 1)}
 
     link = {"bound": "pcie_gen5_x16", "theoretical_gbps": PCIE_GEN5_X16_GBPS,
             "measured_d2h_gbps": round(d2h_peak, 2), "measured_h2d_gbps": round(h2d_peak, 2),

@@ -300,9 +300,13 @@ int pf_xfer_load(pf_xfer_t x, const pf_layer_blocks* layers, uint64_t n_layers,
 int pf_xfer_set_layer_events(pf_xfer_t x, pf_event_t* events, uint64_t n);
 /* Path the last call took for layer 0 (PF_PATH_ZEROCOPY or PF_PATH_STAGED). */
 int pf_xfer_last_path(pf_xfer_t x);
-/* Timing of the device-side gather/scatter kernels of the last call: total
- * milliseconds and launches, measured with events on the stream the kernels
- * ran on.  Blocks until those events have completed. */
+/* Timing of the device-side gather/scatter kernels, measured with events on
+ * the stream the kernels ran on: total milliseconds and launches.  Blocks until
+ * those events have completed.  pf_xfer_set_kernel_timing: 0 = off; 1 = every
+ * launch is timed running alone (the link copies of the staged path share the
+ * kernels' stream while this is on) and the figures are those of the last call;
+ * 2 = launches are timed where they run, streams unchanged, and the figures add
+ * up over calls until pf_xfer_last_kernel_ms reads (and clears) them. */
 int pf_xfer_last_kernel_ms(pf_xfer_t x, float* out_ms, uint32_t* out_launches);
 int pf_xfer_set_kernel_timing(pf_xfer_t x, int enable);
 

@@ -123,6 +123,7 @@ int Xfer::last_kernel_ms(float* out_ms, uint32_t* out_launches) {
   }
   *out_ms = total;
   *out_launches = static_cast<uint32_t>(timing_used_);
+  if (timing_in_place_) timing_used_ = 0;
   return PF_OK;
 }
 
@@ -510,7 +511,7 @@ int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool s
 
 int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save,
                    hipStream_t s) {
-  timing_used_ = 0;
+  if (!timing_in_place_) timing_used_ = 0;
   if (n_layers == 0) return PF_OK;
   if (!layers) return fail(PF_ERR_INVALID_ARGUMENT, "layers must not be null");
   if (!layer_events_.empty() && layer_events_.size() < n_layers) {
@@ -899,7 +900,10 @@ int pf_plain_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t tile_unro
 
 int pf_xfer_set_kernel_timing(pf_xfer_t x, int enable) {
   PF_REQUIRE_PTR(x);
-  reinterpret_cast<pf::Xfer*>(x)->set_timing(enable != 0);
+  if (enable < 0 || enable > 2) {
+    return pf::fail(PF_ERR_INVALID_ARGUMENT, "kernel timing mode %d (expected 0, 1 or 2)", enable);
+  }
+  reinterpret_cast<pf::Xfer*>(x)->set_timing(enable);
   return PF_OK;
 }
 

@@ -121,7 +121,15 @@ class Xfer {
     }
   }
   int last_path() const { return last_path_; }
-  void set_timing(bool on) { timing_ = on; }
+  // 0 = off; 1 = time every launch alone (the link copies share the kernels'
+  // stream meanwhile) and restart the figures with every call; 2 = time the
+  // launches where they run, leaving the streams as they are, and add up over
+  // calls until last_kernel_ms() is read.
+  void set_timing(int mode) {
+    timing_ = mode != 0;
+    timing_in_place_ = mode == 2;
+    timing_used_ = 0;
+  }
   int last_kernel_ms(float* out_ms, uint32_t* out_launches);
 
  private:
@@ -170,6 +178,7 @@ class Xfer {
   int last_path_ = 0;
 
   bool timing_ = false;
+  bool timing_in_place_ = false;
   bool began_ = false;  // the current call has enqueued work
   uint32_t copy_stream_ = 0;  // 0 = by unit count, 1 = side stream, 2 = caller's stream
   // A second stream pays off only when the copy of one unit can overlap the
@@ -179,7 +188,7 @@ class Xfer {
   // 44.4 / 52.8 / 55.6 GB/s with the hand-off to a side stream; from two
   // units on the side stream wins (56.6 against 55.8 GB/s at 32 units).
   bool use_side_stream(size_t staged_units) const {
-    if (timing_ || copy_stream_ == 2) return false;
+    if ((timing_ && !timing_in_place_) || copy_stream_ == 2) return false;
     if (copy_stream_ == 1) return true;
     return staged_units > 1;
   }

@@ -285,8 +285,10 @@ class BlockTransfer:
     def last_path(self) -> int:
         return self._lib.pf_xfer_last_path(self.handle)
 
-    def set_kernel_timing(self, enable: bool) -> None:
-        check(self._lib.pf_xfer_set_kernel_timing(self.handle, 1 if enable else 0))
+    def set_kernel_timing(self, enable) -> None:
+        """False/0 = off; True/1 = launches timed alone, figures per call; 2 =
+        launches timed in place, figures add up until ``last_kernel_ms`` reads them."""
+        check(self._lib.pf_xfer_set_kernel_timing(self.handle, int(enable)))
 
     def last_kernel_ms(self) -> tuple[float, int]:
         ms = C.c_float()
