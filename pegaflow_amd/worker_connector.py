@@ -315,7 +315,15 @@ class WorkerConnector:
         self._page_first = self._use_page_first()
         group_ids = None
         if self._cache_groups.group_count > 1:
-            group_ids = [self._layer_to_group.get(name, 0) for name in kv_caches]
+            strangers = [name for name in kv_caches if name not in self._layer_to_group]
+            if strangers:
+                raise RuntimeError(
+                    f"HMA registration contains layers outside cache groups: {strangers[:8]}")
+            # The engine is told the STORAGE group of each layer (attention 0,
+            # recurrent groups 1, 2, ...), which is not the cache-group index
+            # when a recurrent group comes first (worker.py:364-367).
+            storage_ids = self._cache_groups.storage_group_ids
+            group_ids = [storage_ids[self._layer_to_group[name]] for name in kv_caches]
         recurrent = {name for index in self._cache_groups.recurrent_group_indices
                      for name in self._cache_groups.layer_names[index]}
         self._registered_layers = register_kv_caches(
@@ -324,6 +332,15 @@ class WorkerConnector:
             tp_size=1 if ctx.is_mla else ctx.tp_size, world_size=ctx.world_size,
             transfer_backend=ctx.transfer_backend, page_first=self._page_first,
             recurrent_layer_names=recurrent, layer_group_ids=group_ids)
+
+    def register_cross_layers_kv_cache(self, kv_cache, attn_backend=None) -> None:
+        """One tensor holds every layer of a block: it is registered as a single
+        pseudo-layer, named per pipeline stage when there are several
+        (worker.py:414-420)."""
+        self._cross_layer_mode = True
+        self._cross_layer_key = (f"{CROSS_LAYER_KEY}_pp{self._ctx.pp_rank}"
+                                 if self._ctx.pp_size > 1 else CROSS_LAYER_KEY)
+        self.register_kv_caches({self._cross_layer_key: kv_cache})
 
     def _use_page_first(self) -> bool:
         # worker.py:967-980: only when one worker writes every layer of a page.

@@ -60,7 +60,7 @@ def test_register_save_query_load_on_torch_tensors(kind, gpu):
         eng.close()
 
 
-@pytest.mark.parametrize("kind", ["kv_first", "mla_page_first"])
+@pytest.mark.parametrize("kind", ["kv_first", "mla_page_first", "cross_layer"])
 def test_worker_connector_steps_over_a_real_engine(kind, gpu):
     """Two workers (a prefill and a decode instance of one namespace) driven the
     way vLLM drives them: metadata in, start_load_kv / wait_for_save per step,
@@ -78,8 +78,12 @@ def test_worker_connector_steps_over_a_real_engine(kind, gpu):
     names = [f"model.layers.{i}.self_attn.attn" for i in range(4)]
     if kind == "kv_first":
         shape, is_mla, block_size, block_dim = (2, 96, 16, 8, 128), False, 16, 1
-    else:
+    elif kind == "mla_page_first":
         shape, is_mla, block_size, block_dim = (96, 64, 576), True, 64, 0
+    else:
+        # one tensor for all layers: [blocks, layers, K/V, tokens, heads, head size]
+        shape, is_mla, block_size, block_dim = (96, 3, 2, 16, 4, 64), False, 16, 0
+        names = ["ALL_LAYERS"]
     src = {n: torch.randn(shape, device=dev, dtype=torch.bfloat16, generator=gen) for n in names}
     dst = {n: torch.zeros(shape, device=dev, dtype=torch.bfloat16) for n in names}
     torch.cuda.synchronize()
@@ -106,8 +110,12 @@ def test_worker_connector_steps_over_a_real_engine(kind, gpu):
 
     prefill, decode = worker_for("prefill"), worker_for("decode")
     try:
-        prefill.register_kv_caches(src)
-        decode.register_kv_caches(dst)
+        if kind == "cross_layer":
+            prefill.register_cross_layers_kv_cache(src["ALL_LAYERS"])
+            decode.register_cross_layers_kv_cache(dst["ALL_LAYERS"])
+        else:
+            prefill.register_kv_caches(src)
+            decode.register_kv_caches(dst)
         assert prefill._registered_layers == names and prefill._page_first == is_mla
         # step 1: two requests finish prefill; request b holds the null block
         hashes_a = [b"a%d" % i + bytes(6) for i in range(5)]

@@ -371,3 +371,57 @@ def test_recurrent_hold_adds_one_membership_load_per_recurrent_group():
         worker.start_load_kv(PegaConnectorMetadata(load_intents={"h": LoadIntent(
             block_ids_by_group=((11,), (31,)), leases=(b"prefix",), num_tokens=16,
             recurrent_hold=bad)}))
+
+
+# ---- registration (worker.py:261-420; test_connector_fault_tolerance.py:500-511) ----
+
+def registering_worker(monkeypatch, cache_groups=None, **ctx):
+    """A worker whose engine registration is captured instead of executed."""
+    calls = []
+
+    def fake_register(engine, instance_id, namespace, device_id, kv_caches, block_size, **kw):
+        calls.append(dict(instance_id=instance_id, namespace=namespace, device_id=device_id,
+                          layers=list(kv_caches), block_size=block_size, **kw))
+        return list(kv_caches)
+
+    monkeypatch.setattr(wc, "register_kv_caches", fake_register)
+    client = wc.InProcessEngineClient(engine=None)
+    fields = dict(instance_id="inst", namespace="ns", block_size=16, tp_size=1, world_size=1,
+                  tp_rank=0, device_id=0, engine_client=client)
+    fields.update(ctx)
+    worker = WorkerConnector(ConnectorContext(**fields), cache_groups, start_save_thread=False)
+    return worker, calls
+
+
+def test_registration_passes_storage_group_ids(monkeypatch):
+    groups = CacheGroups((("mamba.0", "mamba.1"), ("attn.0",)), frozenset({0}))
+    worker, calls = registering_worker(monkeypatch, groups)
+    worker.register_kv_caches({"attn.0": object(), "mamba.0": object(), "mamba.1": object()})
+    assert calls[0]["layer_group_ids"] == [0, 1, 1]          # attention is storage group 0
+    assert calls[0]["recurrent_layer_names"] == {"mamba.0", "mamba.1"}
+    assert calls[0]["page_first"] is False
+    assert worker._registered_layers == ["attn.0", "mamba.0", "mamba.1"]
+    with pytest.raises(RuntimeError, match="layers outside cache groups: \\['stray'\\]"):
+        worker.register_kv_caches({"attn.0": object(), "stray": object()})
+
+
+def test_single_group_registration_and_page_first_choice(monkeypatch):
+    worker, calls = registering_worker(monkeypatch, is_mla=True, tp_rank=3, tp_size=4)
+    worker.register_kv_caches({"l0": object()})
+    # MLA: stored once for all TP ranks, page-first when one worker writes whole pages
+    assert calls[0]["layer_group_ids"] is None and calls[0]["page_first"] is True
+    assert calls[0]["tp_rank"] == 0 and calls[0]["tp_size"] == 1
+    worker, calls = registering_worker(monkeypatch, is_mla=True, pp_size=2)
+    worker.register_kv_caches({"l0": object()})
+    assert calls[0]["page_first"] is False                    # a pipeline stage holds part of a page
+
+
+def test_cross_layer_registration_uses_pp_suffixed_name(monkeypatch):
+    worker, calls = registering_worker(monkeypatch, pp_rank=2, pp_size=4)
+    worker.register_cross_layers_kv_cache(object())
+    assert calls[0]["layers"] == ["ALL_LAYERS_pp2"]
+    assert worker._cross_layer_mode and worker._registered_layers == ["ALL_LAYERS_pp2"]
+    worker, calls = registering_worker(monkeypatch)
+    worker.register_cross_layers_kv_cache(object())
+    assert calls[0]["layers"] == ["ALL_LAYERS"]
+    assert worker._load_layer_groups() == [["ALL_LAYERS"]]    # loads then name the pseudo-layer
