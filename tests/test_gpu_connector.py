@@ -154,3 +154,93 @@ def test_worker_connector_steps_over_a_real_engine(kind, gpu):
         prefill.shutdown()
         decode.shutdown()
         eng.close()
+
+
+def test_hybrid_worker_resumes_attention_prefix_and_recurrent_checkpoint(gpu):
+    """A hybrid model (attention + recurrent state) through two workers: the
+    attention group saves a three-block prefix, the recurrent group only the
+    checkpoint at its end; the scheduler-side facts (prefix hit, per-group
+    membership, reconcile_hybrid_hit) turn into one load with a prefix lease and
+    a membership lease (worker.py:572-619, hybrid_groups.rs:14-176)."""
+    import time
+
+    import torch
+
+    from pegaflow_amd.connector import reconcile_hybrid_hit
+    from pegaflow_amd.worker_connector import (CacheGroups, ConnectorContext,
+                                               InProcessEngineClient, LoadIntent,
+                                               PegaConnectorMetadata, RecurrentLoadHold,
+                                               SaveIntent, WorkerConnector)
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(3)
+    blocks, page_elems = 32, 2048                          # one 4 KiB state page per block
+
+    def make_caches(fill):
+        caches = {}
+        for name in ("attn_0", "attn_1"):
+            caches[name] = (torch.randn((2, blocks, 16, 4, 64), device=dev, dtype=torch.bfloat16,
+                                        generator=gen) if fill
+                            else torch.zeros((2, blocks, 16, 4, 64), device=dev, dtype=torch.bfloat16))
+        page = (torch.randn(blocks * page_elems, device=dev, dtype=torch.float16, generator=gen)
+                if fill else torch.zeros(blocks * page_elems, device=dev, dtype=torch.float16))
+        # two state tensors viewing one page-strided allocation (conv state, ssm state)
+        caches["recurrent_state"] = (page.as_strided((blocks, 512), (page_elems, 1), 0),
+                                     page.as_strided((blocks, 1024), (page_elems, 1), 512))
+        return caches, page
+
+    src, src_page = make_caches(True)
+    dst, dst_page = make_caches(False)
+    torch.cuda.synchronize()
+    groups = CacheGroups((("attn_0", "attn_1"), ("recurrent_state",)), frozenset({1}))
+    eng = PegaEngine(pool_size=64 << 20)
+    client = InProcessEngineClient(eng)
+
+    def worker_for(instance):
+        ctx = ConnectorContext(instance_id=instance, namespace="hybrid", block_size=16, tp_size=1,
+                               world_size=1, tp_rank=0, device_id=0, engine_client=client)
+        return WorkerConnector(ctx, groups, device_synchronize=torch.cuda.synchronize)
+
+    prefill, decode = worker_for("prefill"), worker_for("decode")
+    try:
+        prefill.register_kv_caches(src)
+        decode.register_kv_caches(dst)
+        hashes = [bytes([40 + i]) * 8 for i in range(3)]
+        step = PegaConnectorMetadata(save_intents={"r": SaveIntent(
+            block_ids_by_group=((1, 2, 3), (0, 0, 9)), block_hashes=tuple(hashes))})
+        prefill.start_load_kv(step)
+        prefill.wait_for_save()                              # recurrent state: saved before returning
+        assert prefill.get_finished({"r"})[0] == {"r"}
+        # the scheduler's view
+        hits, lease = client.query("decode", hashes)
+        members = eng.query_group_membership("decode", groups.storage_group_of(1), hashes)
+        assert hits == 3 and members == [False, False, True]
+        positions = tuple(i for i, present in enumerate(members) if present)
+        hit_blocks, checkpoint, usable = reconcile_hybrid_hit(hits, ((positions,),))
+        assert (hit_blocks, checkpoint, usable) == (3, 2, frozenset({2}))
+        member_lease = client.lease_token(eng.create_group_lease(
+            "decode", groups.storage_group_of(1), [hashes[p] for p in positions]))
+        hold = RecurrentLoadHold(leases=((member_lease,),), hit_positions=((positions,),),
+                                 checkpoint=checkpoint)
+        decode.start_load_kv(PegaConnectorMetadata(load_intents={"r": LoadIntent(
+            block_ids_by_group=((11, 12, 13), (None, None, 21)), leases=(lease,), num_tokens=48,
+            recurrent_hold=hold)}))
+        deadline = time.time() + 20
+        done = None
+        while done is None and time.time() < deadline:
+            done = decode.get_finished(set())[1]
+            time.sleep(0.002)
+        assert done == {"r"} and decode.get_block_ids_with_load_errors() == set()
+        for name in ("attn_0", "attn_1"):
+            want = torch.zeros_like(src[name])
+            want[:, 11:14] = src[name][:, 1:4]
+            assert torch.equal(dst[name].view(torch.int16), want.view(torch.int16)), name
+        want_page = torch.zeros_like(src_page).view(blocks, page_elems)
+        want_page[21] = src_page.view(blocks, page_elems)[9]
+        assert torch.equal(dst_page.view(blocks, page_elems).view(torch.int16),
+                           want_page.view(torch.int16))
+    finally:
+        prefill.shutdown()
+        decode.shutdown()
+        eng.close()
