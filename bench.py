@@ -81,6 +81,8 @@ def parse_args():
     ap.add_argument("--no-overlap", action="store_true", help="skip the GEMM-overlap section")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-engine", action="store_true", help="skip the save/query/load engine section")
+    ap.add_argument("--engine-mode", choices=["direct", "kernel"], default="direct",
+                    help="transfer mode the engine section registers its instances with")
     ap.add_argument("--engine-child", action="store_true",
                     help="(internal) run only the engine section and print its JSON")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
@@ -177,7 +179,7 @@ def main():
     if args.engine_child:
         torch.cuda.synchronize()
         print(json.dumps(run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids,
-                                    payload)))
+                                    payload, args.engine_mode)))
         return
     t0 = time.time()
     pool = PinnedMemory(payload)
@@ -432,7 +434,7 @@ def main():
         del src_cache, dst_cache, save_layers, load_layers, scratch, scratch2
         torch.cuda.empty_cache()
         cmd = [sys.executable, os.path.abspath(__file__), "--engine-child", "--workload",
-               args.workload, "--seed", str(args.seed)]
+               args.workload, "--seed", str(args.seed), "--engine-mode", args.engine_mode]
         if args.layers:
             cmd += ["--layers", str(args.layers)]
         proc = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
@@ -642,7 +644,8 @@ def run_ref_transfer_bench(torch, np, args):
         "table": rows}))
 
 
-def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, payload):
+def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, payload,
+               mode_name="direct"):
     """End to end through pf_engine_*: registration, batch_save (host image
     allocation in the pinned pool, one worker task, block bookkeeping), prefix
     query, batch_load into a second instance of the same namespace.  Times are
@@ -658,11 +661,12 @@ def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, pa
         eng.register_context_layer_batch(
             inst, "bench", 0, 0, 0, 1, 1, names, [t.data_ptr() for t in caches],
             [nseg * nb * seg] * n_layers, [nb] * n_layers, [seg] * n_layers, [kv] * n_layers,
-            [nseg] * n_layers, transfer_mode=TransferMode.DIRECT, page_first=w["page_first"])
+            [nseg] * n_layers, transfer_mode=TransferMode.from_name(mode_name),
+            page_first=w["page_first"])
     for t in dst_cache:
         t.zero_()
     torch.cuda.synchronize()
-    out = {"transfer_mode": "direct"}
+    out = {"transfer_mode": mode_name}
     reps = 3
     save_s, load_s, query_s = [], [], []
     for rep in range(reps):

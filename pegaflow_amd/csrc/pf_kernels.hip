@@ -274,6 +274,25 @@ __global__ __launch_bounds__(LT) void block_tiles_kernel(const BlockUnit* __rest
   }
 }
 
+// The two halves of streams_run_concurrently().  The wait is bounded by the
+// constant-rate device clock (100 MHz), so the lane leaves whatever happens.
+__global__ __launch_bounds__(64) void probe_wait_kernel(uint32_t* word, uint32_t* seen,
+                                                        uint64_t max_ticks) {
+  if (threadIdx.x != 0) return;
+  const uint64_t begin = wall_clock64();
+  uint32_t value = 0;
+  for (;;) {
+    value = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (value != 0 || wall_clock64() - begin > max_ticks) break;
+    __builtin_amdgcn_s_sleep(16);
+  }
+  __hip_atomic_store(seen, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__global__ __launch_bounds__(64) void probe_post_kernel(uint32_t* word) {
+  if (threadIdx.x == 0) __hip_atomic_store(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 template <int U>
 __global__ __launch_bounds__(kLanes) void plain_copy_kernel(uint64_t dst, uint64_t src,
                                                             uint64_t bytes) {
@@ -408,6 +427,31 @@ int launch_block_tiles(const BlockUnit* units, uint32_t n_units, uint32_t max_bl
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail_hip(e, "block_tiles_kernel launch");
   return PF_OK;
+}
+
+int streams_run_concurrently(hipStream_t a, hipStream_t b, bool* out) {
+  *out = false;
+  uint32_t* words = nullptr;  // [0] the posted word, [1] what the waiter saw
+  PF_HIP(hipMalloc(reinterpret_cast<void**>(&words), 2 * sizeof(uint32_t)));
+  int st = PF_OK;
+  uint32_t seen = 0;
+  hipError_t e = hipMemset(words, 0, 2 * sizeof(uint32_t));
+  if (e == hipSuccess) e = hipDeviceSynchronize();
+  if (e == hipSuccess) {
+    constexpr uint64_t kMaxTicks = 200000;  // 2 ms of the 100 MHz clock
+    hipLaunchKernelGGL(probe_wait_kernel, dim3(1), dim3(64), 0, a, words, words + 1, kMaxTicks);
+    hipLaunchKernelGGL(probe_post_kernel, dim3(1), dim3(64), 0, b, words);
+    e = hipGetLastError();
+  }
+  // Wait for both whatever was launched, so that the words can be freed.
+  const hipError_t ea = hipStreamSynchronize(a);
+  const hipError_t eb = hipStreamSynchronize(b);
+  if (e == hipSuccess) e = ea != hipSuccess ? ea : eb;
+  if (e == hipSuccess) e = hipMemcpy(&seen, words + 1, sizeof(seen), hipMemcpyDeviceToHost);
+  if (e != hipSuccess) st = fail_hip(e, "stream concurrency probe");
+  (void)hipFree(words);
+  *out = seen != 0;
+  return st;
 }
 
 int launch_plain_copy(void* dst, const void* src, uint64_t bytes, int unroll, hipStream_t s) {

@@ -67,4 +67,12 @@ int launch_block_tiles(const BlockUnit* units, uint32_t n_units, uint32_t max_bl
 // unroll 0 selects the one-tile-per-workgroup form, 1/2/4/8 the grid-stride form.
 int launch_plain_copy(void* dst, const void* src, uint64_t bytes, int unroll, hipStream_t s);
 
+// Do kernels of stream `a` and stream `b` run at the same time?  The runtime
+// multiplexes a process's streams onto a few hardware queues, and two streams
+// that share one execute their kernels strictly one after the other.  A
+// one-lane kernel on `a` waits (for at most ~2 ms of the device's constant
+// clock, then gives up) for a word that a one-lane kernel on `b` writes; seeing
+// it proves the two ran concurrently.  Both streams are idle afterwards.
+int streams_run_concurrently(hipStream_t a, hipStream_t b, bool* out);
+
 }  // namespace pf

@@ -4,6 +4,7 @@
 #include <cstring>
 
 #include "pf_common.hpp"
+#include "pf_kernels.hpp"
 #include "pf_sync_state.hpp"
 #include "pf_xfer.hpp"
 
@@ -301,8 +302,77 @@ std::unique_ptr<GpuWorkerPool> GpuWorkerPool::spawn(int device_id, NumaNode numa
     if (status) *status = bad.status;
     return nullptr;  // destructor joins the threads
   }
+  pool->separate_worker_queues();
   pool->prime_copy_overlap();
   return pool;
+}
+
+// Worker streams must not share a hardware queue: a zero-copy save and a
+// zero-copy load are one long kernel each, and on one queue the second simply
+// waits for the first (seen with rocprofv3 --kernel-trace: the save worker of
+// one instance and the load worker of another both on queue 3, the load
+// starting the moment the save ended, 57 GB/s for the pair instead of 94).
+// The runtime decides which queue a stream gets and offers no way to ask, so
+// a new pool checks whether kernels of its streams overlap with each other
+// and with the idle worker streams of the other pools on the device, and
+// replaces a stream that does not by a fresh one, a few times at most, keeping
+// the candidate with the fewest clashes.  Rejected streams are destroyed at
+// the end (destroying one at once could hand its queue to the very next
+// stream).  No task has been accepted yet.
+namespace {
+std::mutex g_worker_streams_mu;
+std::vector<std::pair<int, hipStream_t>> g_worker_streams;  // (device, stream) of live pools
+
+size_t clashes(hipStream_t candidate, const std::vector<hipStream_t>& others) {
+  size_t n = 0;
+  for (hipStream_t other : others) {
+    bool concurrent = true;
+    // The waiting kernel goes on the candidate, which is idle by construction.
+    if (streams_run_concurrently(candidate, other, &concurrent) != PF_OK) return 0;
+    n += concurrent ? 0 : 1;
+  }
+  return n;
+}
+}  // namespace
+
+void GpuWorkerPool::separate_worker_queues() {
+  if (hipSetDevice(device_id_) != hipSuccess) return;
+  std::lock_guard<std::mutex> registry(g_worker_streams_mu);
+  std::vector<hipStream_t> others;
+  for (auto it = g_worker_streams.rbegin(); it != g_worker_streams.rend() && others.size() < 6;
+       ++it) {
+    // A stream that is busy would make the probe wait for its work: skip it.
+    if (it->first == device_id_ && hipStreamQuery(it->second) == hipSuccess) {
+      others.push_back(it->second);
+    }
+  }
+  (void)hipGetLastError();
+  std::vector<hipStream_t> rejected;
+  for (Worker* w : {&save_, &load_}) {
+    hipStream_t best = w->stream;
+    size_t best_clashes = clashes(best, others);
+    for (int attempt = 0; attempt < 6 && best_clashes != 0; ++attempt) {
+      hipStream_t fresh = nullptr;
+      if (hipStreamCreateWithFlags(&fresh, hipStreamNonBlocking) != hipSuccess) break;
+      const size_t c = clashes(fresh, others);
+      if (c < best_clashes) {
+        rejected.push_back(best);
+        best = fresh;
+        best_clashes = c;
+      } else {
+        rejected.push_back(fresh);
+      }
+    }
+    {
+      std::lock_guard<std::mutex> lock(w->mu);
+      w->stream = best;
+    }
+    others.push_back(best);
+  }
+  for (hipStream_t s : rejected) (void)hipStreamDestroy(s);
+  (void)hipGetLastError();
+  g_worker_streams.emplace_back(device_id_, save_.stream);
+  g_worker_streams.emplace_back(device_id_, load_.stream);
 }
 
 // Measured on MI355X with this runtime: whether the link copies of the save
@@ -339,6 +409,14 @@ void GpuWorkerPool::prime_copy_overlap() {
 }
 
 GpuWorkerPool::~GpuWorkerPool() {
+  {
+    // Out of the registry before the workers destroy their streams.
+    std::lock_guard<std::mutex> registry(g_worker_streams_mu);
+    for (auto it = g_worker_streams.begin(); it != g_worker_streams.end();) {
+      const bool mine = it->second == save_.stream || it->second == load_.stream;
+      it = mine ? g_worker_streams.erase(it) : it + 1;
+    }
+  }
   for (Worker* w : {&load_, &save_}) {
     {
       std::lock_guard<std::mutex> lock(w->mu);
@@ -436,6 +514,7 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
       if (w->queue.empty()) break;  // stop requested and drained
       task = std::move(w->queue.front());
       w->queue.pop_front();
+      stream = w->stream;  // the pool may have replaced it before the first task
     }
     // process_load_task / process_save_task, gpu_worker.rs:428-523.
     const auto t0 = std::chrono::steady_clock::now();
@@ -447,13 +526,20 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
     // (much larger) rest is still being converted.  Everything is only
     // enqueued; there is still one synchronisation.  Tasks described by host
     // images need no conversion work and go in one call, which also keeps the
-    // layers of page-first pages together for whole-page staging.
+    // layers of page-first pages together for whole-page staging.  Zero-copy
+    // tasks go in one call as well: a two-layer zero-copy launch that starts
+    // next to a zero-copy save of another worker crawled (124 ms instead of
+    // 11 ms, the save beside it at a quarter of its rate; a save and a load
+    // together 68 GB/s), while single launches share the link at 91-92 GB/s;
+    // alone, the one call costs 0.5-2 % of a load.
     const size_t n_layers = task->layers.size();
     bool per_block = false;
     for (const auto& l : task->layers) per_block |= !l.blocks.empty();
     size_t first_part = n_layers ? n_layers : 1;
     // (Descriptor backends build one descriptor per fragment whatever the form.)
-    if ((!xfer || per_block) && n_layers >= 16) first_part = n_layers / 16 < 2 ? 2 : n_layers / 16;
+    if ((!xfer || (per_block && path != PF_PATH_ZEROCOPY)) && n_layers >= 16) {
+      first_part = n_layers / 16 < 2 ? 2 : n_layers / 16;
+    }
     for (size_t begin = 0; begin < n_layers && st == PF_OK;) {
       // Block-ID form: the rest goes in one call (a call boundary drains the
       // engine's copy pipeline).  Descriptor form: every part is that small;
@@ -525,6 +611,10 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
   xfer.reset();
   backend.reset();
   (void)hipEventDestroy(done);
+  {
+    std::lock_guard<std::mutex> lock(w->mu);
+    stream = w->stream;
+  }
   (void)hipStreamDestroy(stream);
 }
 

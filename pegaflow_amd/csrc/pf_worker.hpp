@@ -121,6 +121,8 @@ class GpuWorkerPool {
   };
   // One large copy in each direction, in flight together, before the first task.
   void prime_copy_overlap();
+  // Make sure the two workers' streams execute kernels concurrently.
+  void separate_worker_queues();
   GpuWorkerPool() = default;
   void run(Worker* w, bool is_load, NumaNode numa, std::promise<TaskResult>* ready);
   std::future<TaskResult> push(Worker* w, std::unique_ptr<Task> t);

@@ -444,6 +444,9 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
 
   began_ = true;
   PF_HIP(hipMemcpyAsync(slab->dev, slab->host, slab_bytes, hipMemcpyHostToDevice, s));
+  if (use_side_stream(chunks.size()) && side_ == nullptr) {
+    PF_HIP(hipStreamCreateWithFlags(&side_, hipStreamNonBlocking));
+  }
   hipStream_t side = use_side_stream(chunks.size()) ? side_ : s;
   if (side != s) {
     PF_HIP(hipEventRecord(fork_, s));
@@ -501,7 +504,7 @@ int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool s
     // caller's synchronise of `s` would not cover: drain both before the
     // caller learns of the failure and releases its buffers.
     const std::string message = last_error();
-    (void)hipStreamSynchronize(side_);
+    if (side_ != nullptr) (void)hipStreamSynchronize(side_);
     (void)hipStreamSynchronize(s);
     (void)hipGetLastError();
     last_error() = message;
@@ -739,6 +742,9 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
   // that every timed kernel executes alone (a measurement mode: no overlap).
   size_t staged_units = 0;
   for (const UnitRef& r : unit_refs) staged_units += plans[r.plan].staged ? 1 : 0;
+  if (use_side_stream(staged_units) && side_ == nullptr) {
+    PF_HIP(hipStreamCreateWithFlags(&side_, hipStreamNonBlocking));
+  }
   hipStream_t side = use_side_stream(staged_units) ? side_ : s;
   bool side_used = false;
   auto fork_side = [&]() -> int {

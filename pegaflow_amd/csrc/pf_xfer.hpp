@@ -86,7 +86,8 @@ class Xfer {
       fail_hip(e, "hipGetDevice");
       return fail(PF_ERR_DEVICE_INIT, "transfer engine init failed: %s", last_error().c_str());
     }
-    PF_HIP(hipStreamCreateWithFlags(&side_, hipStreamNonBlocking));
+    // The side stream is created when a call first needs it: an engine whose
+    // link copies stay on the caller's stream never takes a hardware queue.
     PF_HIP(hipEventCreateWithFlags(&fork_, hipEventDisableTiming));
     PF_HIP(hipEventCreateWithFlags(&join_, hipEventDisableTiming));
     slots_.resize(n_slots_);
