@@ -76,6 +76,14 @@ int pf_stream_destroy(pf_stream_t s);
 int pf_stream_synchronize(pf_stream_t s);
 int pf_stream_wait_event(pf_stream_t s, pf_event_t e);
 void* pf_stream_native(pf_stream_t s);
+/* Do kernels of the two streams execute at the same time?  (The runtime
+ * multiplexes a process's streams onto a few hardware queues; streams that
+ * share one run their kernels strictly one after the other.)  *out = 1 when a
+ * one-lane kernel on `a` saw, within 2 ms, a word posted by a one-lane kernel
+ * on `b`.  Both streams are synchronised by the call.  The worker pools use
+ * this when they are spawned (no counterpart in the reference, whose two worker
+ * streams are never checked). */
+int pf_streams_run_concurrently(pf_stream_t a, pf_stream_t b, int* out);
 
 int pf_event_create(int enable_timing, pf_event_t* out);
 int pf_event_destroy(pf_event_t e);

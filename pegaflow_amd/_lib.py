@@ -153,6 +153,7 @@ PROTOTYPES = {
     "pf_stream_wrap": (C.c_int, [vp, C.POINTER(vp)]),
     "pf_stream_destroy": (C.c_int, [vp]),
     "pf_stream_synchronize": (C.c_int, [vp]),
+    "pf_streams_run_concurrently": (C.c_int, [vp, vp, C.POINTER(C.c_int)]),
     "pf_stream_wait_event": (C.c_int, [vp, vp]),
     "pf_stream_native": (vp, [vp]),
     "pf_event_create": (C.c_int, [C.c_int, C.POINTER(vp)]),

@@ -435,8 +435,9 @@ int streams_run_concurrently(hipStream_t a, hipStream_t b, bool* out) {
   PF_HIP(hipMalloc(reinterpret_cast<void**>(&words), 2 * sizeof(uint32_t)));
   int st = PF_OK;
   uint32_t seen = 0;
-  hipError_t e = hipMemset(words, 0, 2 * sizeof(uint32_t));
-  if (e == hipSuccess) e = hipDeviceSynchronize();
+  // Cleared on `a` and waited for there: no other stream of the device is touched.
+  hipError_t e = hipMemsetAsync(words, 0, 2 * sizeof(uint32_t), a);
+  if (e == hipSuccess) e = hipStreamSynchronize(a);
   if (e == hipSuccess) {
     constexpr uint64_t kMaxTicks = 200000;  // 2 ms of the 100 MHz clock
     hipLaunchKernelGGL(probe_wait_kernel, dim3(1), dim3(64), 0, a, words, words + 1, kMaxTicks);

@@ -4,6 +4,7 @@
 #include <fstream>
 
 #include "pf_common.hpp"
+#include "pf_kernels.hpp"
 #include "pf_numa.hpp"
 
 namespace pf {
@@ -113,6 +114,14 @@ int pf_stream_destroy(pf_stream_t s) {
   delete w;
   if (e != hipSuccess) return pf::fail_hip(e, "hipStreamDestroy");
   return PF_OK;
+}
+
+int pf_streams_run_concurrently(pf_stream_t a, pf_stream_t b, int* out) {
+  PF_REQUIRE_PTR(out);
+  bool concurrent = false;
+  const int st = pf::streams_run_concurrently(pf::native(a), pf::native(b), &concurrent);
+  *out = concurrent ? 1 : 0;
+  return st;
 }
 
 int pf_stream_synchronize(pf_stream_t s) {

@@ -61,6 +61,13 @@ class Stream:
     def synchronize(self) -> None:
         check(self._lib.pf_stream_synchronize(self.handle))
 
+    def runs_concurrently_with(self, other: "Stream") -> bool:
+        """Whether kernels of this stream and of ``other`` execute at the same
+        time (they do not when the runtime put both on one hardware queue)."""
+        out = C.c_int()
+        check(self._lib.pf_streams_run_concurrently(self.handle, other.handle, C.byref(out)))
+        return bool(out.value)
+
     def wait_event(self, event: "Event") -> None:
         check(self._lib.pf_stream_wait_event(self.handle, event.handle))
 

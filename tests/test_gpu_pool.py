@@ -111,3 +111,22 @@ def test_zero_size_and_bad_strategy(gpu):
         PinnedMemory(0)
     with pytest.raises(_lib.InvalidArgument, match="greater than zero"):
         PinnedAllocator(0)
+
+
+def test_stream_concurrency_probe(gpu):
+    """A stream cannot overlap with itself: the waiting kernel gives up after
+    its 2 ms and the answer is no.  For two streams the answer depends on the
+    runtime's queue assignment; whichever it is, the call returns, twice the
+    same, and leaves both streams idle.  A pool's two workers do overlap."""
+    import time
+    from pegaflow_amd.runtime import Stream
+    a, b = Stream(), Stream()
+    t0 = time.perf_counter()
+    assert a.runs_concurrently_with(a) is False
+    assert time.perf_counter() - t0 < 1.0
+    first = a.runs_concurrently_with(b)
+    assert a.runs_concurrently_with(b) is first
+    a.synchronize()
+    b.synchronize()
+    a.close()
+    b.close()
