@@ -433,17 +433,21 @@ def main():
         import subprocess
         del src_cache, dst_cache, save_layers, load_layers, scratch, scratch2
         torch.cuda.empty_cache()
-        cmd = [sys.executable, os.path.abspath(__file__), "--engine-child", "--workload",
-               args.workload, "--seed", str(args.seed), "--engine-mode", args.engine_mode]
-        if args.layers:
-            cmd += ["--layers", str(args.layers)]
-        proc = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
-        lines = [ln for ln in proc.stdout.splitlines() if ln.startswith("{")]
-        if proc.returncode == 0 and lines:
-            engine = json.loads(lines[-1])
-        else:
-            print("bench.py: engine section failed:\n" + proc.stderr[-2000:], file=sys.stderr)
-            sys.exit(1)
+        def engine_run(mode):
+            cmd = [sys.executable, os.path.abspath(__file__), "--engine-child", "--workload",
+                   args.workload, "--seed", str(args.seed), "--engine-mode", mode]
+            if args.layers:
+                cmd += ["--layers", str(args.layers)]
+            proc = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+            lines = [ln for ln in proc.stdout.splitlines() if ln.startswith("{")]
+            if proc.returncode != 0 or not lines:
+                print("bench.py: engine section failed:\n" + proc.stderr[-2000:], file=sys.stderr)
+                sys.exit(1)
+            return json.loads(lines[-1])
+        engine = engine_run(args.engine_mode)
+        # the other transfer mode, for comparison (instances choose one at registration)
+        other = "kernel" if args.engine_mode == "direct" else "direct"
+        engine["other_mode"] = engine_run(other)
 
     # ---- CPU baseline: the oracle's memcpy executor on the host cores -----
     cpu = None
