@@ -75,6 +75,34 @@ int Xfer::ensure_slot(Slot& sl, uint64_t bytes) {
   return PF_OK;
 }
 
+// The side stream carries the link copies next to the gather / scatter kernels
+// on the caller's stream `s`; on one hardware queue the two would simply take
+// turns.  Created on first use and, when the caller's stream is idle at that
+// moment (the check synchronises both streams), swapped for a fresh one while
+// kernels of the two do not overlap.
+int Xfer::ensure_side_stream(hipStream_t s) {
+  if (side_ != nullptr) return PF_OK;
+  PF_HIP(hipStreamCreateWithFlags(&side_, hipStreamNonBlocking));
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone ||
+      hipStreamQuery(s) != hipSuccess) {
+    (void)hipGetLastError();
+    return PF_OK;
+  }
+  std::vector<hipStream_t> rejected;
+  for (int attempt = 0; attempt < 4; ++attempt) {
+    bool concurrent = false;
+    if (streams_run_concurrently(side_, s, &concurrent) != PF_OK || concurrent) break;
+    hipStream_t fresh = nullptr;
+    if (hipStreamCreateWithFlags(&fresh, hipStreamNonBlocking) != hipSuccess) break;
+    rejected.push_back(side_);
+    side_ = fresh;
+  }
+  for (hipStream_t r : rejected) (void)hipStreamDestroy(r);
+  (void)hipGetLastError();
+  return PF_OK;
+}
+
 int Xfer::timing_begin(hipStream_t s) {
   if (!timing_) return PF_OK;
   if (timing_used_ == timing_pool_.size()) {
@@ -442,11 +470,13 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
     }
   }
 
+  // Before anything of this call is on `s`: the check wants the stream idle.
+  if (use_side_stream(chunks.size())) {
+    const int side_status = ensure_side_stream(s);
+    if (side_status != PF_OK) return side_status;
+  }
   began_ = true;
   PF_HIP(hipMemcpyAsync(slab->dev, slab->host, slab_bytes, hipMemcpyHostToDevice, s));
-  if (use_side_stream(chunks.size()) && side_ == nullptr) {
-    PF_HIP(hipStreamCreateWithFlags(&side_, hipStreamNonBlocking));
-  }
   hipStream_t side = use_side_stream(chunks.size()) ? side_ : s;
   if (side != s) {
     PF_HIP(hipEventRecord(fork_, s));
@@ -720,6 +750,13 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
   next_slot_ = slot_cursor;
 
   // ---- 4. enqueue ---------------------------------------------------------
+  size_t staged_units = 0;
+  for (const UnitRef& r : unit_refs) staged_units += plans[r.plan].staged ? 1 : 0;
+  // Before anything of this call is on `s`: the check wants the stream idle.
+  if (use_side_stream(staged_units)) {
+    const int side_status = ensure_side_stream(s);
+    if (side_status != PF_OK) return side_status;
+  }
   began_ = true;
   PF_HIP(hipMemcpyAsync(slab->dev, slab->host, head_bytes, hipMemcpyHostToDevice, s));
   // Sorting the ids of a long list takes the submitting thread about a
@@ -740,11 +777,6 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
   };
   // With kernel timing on, the DMA copies run on the caller's stream too, so
   // that every timed kernel executes alone (a measurement mode: no overlap).
-  size_t staged_units = 0;
-  for (const UnitRef& r : unit_refs) staged_units += plans[r.plan].staged ? 1 : 0;
-  if (use_side_stream(staged_units) && side_ == nullptr) {
-    PF_HIP(hipStreamCreateWithFlags(&side_, hipStreamNonBlocking));
-  }
   hipStream_t side = use_side_stream(staged_units) ? side_ : s;
   bool side_used = false;
   auto fork_side = [&]() -> int {

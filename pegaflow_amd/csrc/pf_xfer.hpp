@@ -105,6 +105,7 @@ class Xfer {
     if (x->init() != PF_OK) return nullptr;
     return x;
   }
+  int ensure_side_stream(hipStream_t s);
   int run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save, hipStream_t s);
   int run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save,
                hipStream_t s);
