@@ -320,6 +320,25 @@ std::unique_ptr<GpuWorkerPool> GpuWorkerPool::spawn(int device_id, NumaNode numa
 // the end (destroying one at once could hand its queue to the very next
 // stream).  No task has been accepted yet.
 namespace {
+// Work on the pool's device from a thread that may have another one current
+// (spawn runs on the registering thread): the previous device comes back.
+class DeviceScope {
+ public:
+  explicit DeviceScope(int device) {
+    if (hipGetDevice(&previous_) != hipSuccess) previous_ = -1;
+    ok_ = hipSetDevice(device) == hipSuccess;
+  }
+  ~DeviceScope() {
+    if (previous_ >= 0) (void)hipSetDevice(previous_);
+    (void)hipGetLastError();
+  }
+  bool ok() const { return ok_; }
+
+ private:
+  int previous_ = -1;
+  bool ok_ = false;
+};
+
 std::mutex g_worker_streams_mu;
 std::vector<std::pair<int, hipStream_t>> g_worker_streams;  // (device, stream) of live pools
 
@@ -336,7 +355,8 @@ size_t clashes(hipStream_t candidate, const std::vector<hipStream_t>& others) {
 }  // namespace
 
 void GpuWorkerPool::separate_worker_queues() {
-  if (hipSetDevice(device_id_) != hipSuccess) return;
+  DeviceScope device(device_id_);
+  if (!device.ok()) return;
   std::lock_guard<std::mutex> registry(g_worker_streams_mu);
   std::vector<hipStream_t> others;
   for (auto it = g_worker_streams.rbegin(); it != g_worker_streams.rend() && others.size() < 6;
@@ -385,7 +405,8 @@ void GpuWorkerPool::separate_worker_queues() {
 // once, a few 32 MiB copies on the save stream and, while they run, the same
 // on the load stream.  Failure here only loses the overlap.
 void GpuWorkerPool::prime_copy_overlap() {
-  if (hipSetDevice(device_id_) != hipSuccess) return;
+  DeviceScope device(device_id_);
+  if (!device.ok()) return;
   const size_t chunk = 32u << 20;
   void* host = nullptr;
   void* dev = nullptr;
