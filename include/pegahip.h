@@ -606,6 +606,14 @@ int pf_engine_create_group_lease(pf_engine_t e, const char* instance_id, uint32_
                                  uint64_t n, uint64_t* out_lease);
 int pf_engine_pool_usage(pf_engine_t e, uint64_t* out_used, uint64_t* out_total);
 uint64_t pf_engine_cached_blocks(pf_engine_t e);
+/* Blocks that hold some but not all of their slots (saves of the remaining
+ * layers or ranks are still expected). */
+uint64_t pf_engine_inflight_blocks(pf_engine_t e);
+/* gc_stale_inflight, storage/write_path.rs:52-61,302-330: drop the incomplete
+ * blocks whose first slot arrived more than max_age_ms ago, returning their
+ * pinned memory; returns how many.  The reference's server calls this
+ * periodically. */
+uint64_t pf_engine_gc_stale_inflight(pf_engine_t e, uint64_t max_age_ms);
 /* Drop every cached block that is not leased; returns how many. */
 uint64_t pf_engine_evict_all(pf_engine_t e);
 

@@ -277,6 +277,8 @@ PROTOTYPES = {
                                                u64, C.POINTER(u64)]),
     "pf_engine_pool_usage": (C.c_int, [vp, C.POINTER(u64), C.POINTER(u64)]),
     "pf_engine_cached_blocks": (u64, [vp]),
+    "pf_engine_inflight_blocks": (u64, [vp]),
+    "pf_engine_gc_stale_inflight": (u64, [vp, u64]),
     "pf_engine_evict_all": (u64, [vp]),
 }
 

@@ -2,6 +2,7 @@
 // and pegaflow-common/src/block.rs:1-43 of the reference.
 #pragma once
 
+#include <chrono>
 #include <cstdint>
 #include <memory>
 #include <string>
@@ -124,7 +125,8 @@ class SealedBlock {
 class InflightBlock {
  public:
   explicit InflightBlock(size_t total_slots)
-      : slots_(total_slots), filled_(total_slots, false), remaining_(total_slots) {}
+      : slots_(total_slots), filled_(total_slots, false), remaining_(total_slots),
+        created_(std::chrono::steady_clock::now()) {}
   enum class Insert { Inserted, Completed, Duplicate };
   Insert insert_slot(size_t slot_id, RawBlock block) {
     if (slot_id >= slots_.size() || filled_[slot_id]) return Insert::Duplicate;
@@ -136,6 +138,11 @@ class InflightBlock {
   size_t total_slots() const { return slots_.size(); }
   size_t filled_count() const { return slots_.size() - remaining_; }
   bool complete() const { return remaining_ == 0; }
+  // Time since the first slot arrived (write_path.rs:302-330 collects blocks
+  // that stay incomplete for too long).
+  std::chrono::steady_clock::duration age() const {
+    return std::chrono::steady_clock::now() - created_;
+  }
   std::shared_ptr<SealedBlock> seal() { return std::make_shared<SealedBlock>(std::move(slots_)); }
   // Move every filled slot of `other` into this block (slots already filled
   // here are kept: a repeated slot is a duplicate, as in insert_slot).
@@ -155,6 +162,7 @@ class InflightBlock {
   std::vector<RawBlock> slots_;
   std::vector<bool> filled_;
   size_t remaining_;
+  std::chrono::steady_clock::time_point created_;
 };
 
 }  // namespace pf

@@ -343,6 +343,27 @@ size_t Engine::cached_blocks() {
   return sealed_.size();
 }
 
+size_t Engine::inflight_blocks() {
+  std::lock_guard<std::mutex> lock(mu_);
+  return inflight_.size();
+}
+
+// write_path.rs:302-330: blocks whose remaining slots never arrived give their
+// pinned memory back.
+size_t Engine::gc_stale_inflight(std::chrono::milliseconds max_age) {
+  std::lock_guard<std::mutex> lock(mu_);
+  size_t cleaned = 0;
+  for (auto it = inflight_.begin(); it != inflight_.end();) {
+    if (it->second.age() > max_age) {
+      it = inflight_.erase(it);
+      ++cleaned;
+    } else {
+      ++it;
+    }
+  }
+  return cleaned;
+}
+
 size_t Engine::evict_all() {
   std::lock_guard<std::mutex> lock(mu_);
   size_t n = 0;
@@ -702,6 +723,8 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
         auto it = inflight_.find(key);
         if (it == inflight_.end()) {
           it = inflight_.emplace(key, InflightBlock(topo->total_slots())).first;
+        } else if (it->second.total_slots() != topo->total_slots()) {
+          continue;  // another layout is filling this key: skip it (write_path.rs:147-165)
         }
         if (it->second.insert_slot(slot_id, RawBlock::single_segment(std::move(seg))) ==
             InflightBlock::Insert::Completed) {
@@ -720,6 +743,12 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
           } else {
             inflight_.emplace(key, std::move(a.block));
           }
+        } else if (it->second.total_slots() != a.block.total_slots()) {
+          // The block in flight was begun by an instance with another slot
+          // count (a namespace shared by incompatible layouts): this save's
+          // part is dropped, the other one can still complete
+          // (write_path.rs:147-165).
+          continue;
         } else if (it->second.absorb(std::move(a.block)) == InflightBlock::Insert::Completed) {
           seal(key, &it->second);
           inflight_.erase(it);

@@ -7,6 +7,7 @@
 // reproduced: blocks are kept until evicted oldest-first under pool pressure.
 #pragma once
 
+#include <chrono>
 #include <cstdint>
 #include <future>
 #include <list>
@@ -140,6 +141,10 @@ class Engine {
                                        std::future<TaskResult>* out, std::string* err);
   void pool_usage(uint64_t* used, uint64_t* total) { pool_->usage(used, total); }
   size_t cached_blocks();
+  // Blocks that have some but not all of their slots.
+  size_t inflight_blocks();
+  // Drop the incomplete blocks older than `max_age`; returns how many.
+  size_t gc_stale_inflight(std::chrono::milliseconds max_age);
   // Test hook / pressure valve: drop every sealed block that is not leased.
   size_t evict_all();
 

@@ -511,6 +511,16 @@ uint64_t pf_engine_cached_blocks(pf_engine_t e) {
   return e ? reinterpret_cast<pf::Engine*>(e)->cached_blocks() : 0;
 }
 
+uint64_t pf_engine_inflight_blocks(pf_engine_t e) {
+  return e ? reinterpret_cast<pf::Engine*>(e)->inflight_blocks() : 0;
+}
+
+uint64_t pf_engine_gc_stale_inflight(pf_engine_t e, uint64_t max_age_ms) {
+  return e ? reinterpret_cast<pf::Engine*>(e)->gc_stale_inflight(
+                 std::chrono::milliseconds(max_age_ms))
+           : 0;
+}
+
 uint64_t pf_engine_evict_all(pf_engine_t e) {
   return e ? reinterpret_cast<pf::Engine*>(e)->evict_all() : 0;
 }

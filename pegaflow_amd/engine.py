@@ -382,6 +382,15 @@ class PegaEngine:
     def cached_blocks(self) -> int:
         return self._lib.pf_engine_cached_blocks(self.handle)
 
+    @property
+    def inflight_blocks(self) -> int:
+        """Blocks that have some but not all of their slots."""
+        return self._lib.pf_engine_inflight_blocks(self.handle)
+
+    def gc_stale_inflight(self, max_age_seconds: float) -> int:
+        """Drop incomplete blocks older than ``max_age_seconds``; returns how many."""
+        return self._lib.pf_engine_gc_stale_inflight(self.handle, int(max_age_seconds * 1000))
+
     def evict_all(self) -> int:
         return self._lib.pf_engine_evict_all(self.handle)
 

@@ -663,6 +663,53 @@ def test_save_query_load_roundtrip_with_numa(gpu):
     e.close()
 
 
+def test_incomplete_blocks_wait_are_collected_and_late_saves_are_dropped(engine):
+    """The write path's rules for blocks that do not have all their slots yet
+    (storage/write_path.rs:445-603): a repeated slot changes nothing, a save
+    from an instance with another slot count skips the key, a late save for a
+    block that is already complete leaves nothing behind, and incomplete blocks
+    that grow old are collected with their pinned memory."""
+    two = [Layer("layer_0", 4, 1024), Layer("layer_1", 4, 1024)]
+    four = [Layer(f"layer_{i}", 4, 1024, overwrite=7) for i in range(4)]
+    register(engine, "two-slots", two, ns="shared")
+    register(engine, "four-slots", four, ns="shared")
+    h = make_block_hashes(2, 77)
+    engine.batch_save_kv_blocks("two-slots", 0, 0, 0, [LayerSave("layer_0", [0, 1], h)])
+    assert engine.inflight_blocks == 2 and engine.cached_blocks == 0
+    used_one_slot = engine.pool_usage()[0]
+    # the same slot again: idempotent
+    engine.batch_save_kv_blocks("two-slots", 0, 0, 0, [LayerSave("layer_0", [2, 3], h)])
+    assert engine.inflight_blocks == 2 and engine.query_prefix("two-slots", h) == (0, 0)
+    # another layout tries to fill the same keys: skipped, nothing completes, nothing leaks
+    engine.batch_save_kv_blocks("four-slots", 0, 0, 0, [LayerSave("layer_1", [0, 1], h)])
+    assert engine.inflight_blocks == 2 and engine.cached_blocks == 0
+    assert engine.pool_usage()[0] == used_one_slot
+    # the rightful second slot completes both blocks, with the first slot's original bytes
+    engine.batch_save_kv_blocks("two-slots", 0, 0, 0, [LayerSave("layer_1", [0, 1], h)])
+    assert engine.inflight_blocks == 0 and engine.cached_blocks == 2
+    used_sealed = engine.pool_usage()[0]
+    # a late save for complete blocks is dropped without a trace
+    engine.batch_save_kv_blocks("two-slots", 0, 0, 0, [LayerSave("layer_0", [0, 1], h)])
+    assert engine.inflight_blocks == 0 and engine.pool_usage()[0] == used_sealed
+    for l in two:
+        l.zero_gpu()
+    hits, lease = engine.query_prefix("two-slots", h)
+    assert hits == 2
+    engine.batch_load_kv_blocks_multi_layer("two-slots", 0, 0, [["layer_0", "layer_1"]], lease,
+                                            [[0, 1]]).wait()
+    for l in two:
+        want = np.zeros_like(l.expected)
+        want[:2048] = l.expected[:2048]
+        l.assert_gpu_matches(want)
+    # stale incomplete blocks: kept while young, collected when older than the limit
+    g = make_block_hashes(3, 78)
+    engine.batch_save_kv_blocks("two-slots", 0, 0, 0, [LayerSave("layer_0", [0, 1, 2], g)])
+    assert engine.inflight_blocks == 3
+    assert engine.gc_stale_inflight(60.0) == 0 and engine.inflight_blocks == 3
+    assert engine.gc_stale_inflight(0.0) == 3 and engine.inflight_blocks == 0
+    assert engine.pool_usage()[0] == used_sealed
+
+
 def test_namespace_isolation(engine):
     """engine_basic.rs:254-271: blocks of one namespace are invisible to another."""
     a, b = Layer("layer_0", 4, 1024), Layer("layer_0", 4, 1024)
