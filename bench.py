@@ -83,6 +83,9 @@ def parse_args():
     ap.add_argument("--no-engine", action="store_true", help="skip the save/query/load engine section")
     ap.add_argument("--engine-mode", choices=["direct", "kernel"], default="direct",
                     help="transfer mode the engine section registers its instances with")
+    ap.add_argument("--engine-descriptors", action="store_true",
+                    help="engine section: the workers build one descriptor per fragment and call "
+                         "the descriptor backends, as the reference's workers do")
     ap.add_argument("--engine-child", action="store_true",
                     help="(internal) run only the engine section and print its JSON")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
@@ -179,7 +182,7 @@ def main():
     if args.engine_child:
         torch.cuda.synchronize()
         print(json.dumps(run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids,
-                                    payload, args.engine_mode)))
+                                    payload, args.engine_mode, args.engine_descriptors)))
         return
     t0 = time.time()
     pool = PinnedMemory(payload)
@@ -436,6 +439,8 @@ def main():
         def engine_run(mode):
             cmd = [sys.executable, os.path.abspath(__file__), "--engine-child", "--workload",
                    args.workload, "--seed", str(args.seed), "--engine-mode", mode]
+            if args.engine_descriptors:
+                cmd.append("--engine-descriptors")
             if args.layers:
                 cmd += ["--layers", str(args.layers)]
             proc = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
@@ -649,7 +654,7 @@ def run_ref_transfer_bench(torch, np, args):
 
 
 def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, payload,
-               mode_name="direct"):
+               mode_name="direct", descriptors=False):
     """End to end through pf_engine_*: registration, batch_save (host image
     allocation in the pinned pool, one worker task, block bookkeeping), prefix
     query, batch_load into a second instance of the same namespace.  Times are
@@ -659,7 +664,8 @@ def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, pa
     nb, seg, n = w["num_blocks"], w["seg"], w["n"]
     nseg = 2 if w["split"] else 1
     n_layers = len(names)
-    eng = PegaEngine(pool_size=int(payload * 2.3) + (256 << 20))
+    eng = PegaEngine(pool_size=int(payload * 2.3) + (256 << 20),
+                     use_descriptor_backends=descriptors)
     kv = nb * seg if nseg == 2 else 0
     for inst, caches in (("bench-src", src_cache), ("bench-dst", dst_cache)):
         eng.register_context_layer_batch(
@@ -670,7 +676,7 @@ def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, pa
     for t in dst_cache:
         t.zero_()
     torch.cuda.synchronize()
-    out = {"transfer_mode": mode_name}
+    out = {"transfer_mode": mode_name, "worker_form": "descriptors" if descriptors else "block ids"}
     reps = 3
     save_s, load_s, query_s = [], [], []
     for rep in range(reps):
