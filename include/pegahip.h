@@ -212,6 +212,22 @@ const char* pf_backend_name(pf_backend_t b);
 /* TransferBackend::h2d / d2h.  Enqueue only. */
 int pf_backend_h2d(pf_backend_t b, const pf_copy_desc* copies, uint64_t n, pf_stream_t s);
 int pf_backend_d2h(pf_backend_t b, const pf_copy_desc* copies, uint64_t n, pf_stream_t s);
+/* The copy of PF_MODE_KERNEL for callers that cannot allocate: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  No
+ * counterpart in the reference (its KernelBackend reallocates its device table
+ * whenever a batch outgrows it, transfer/kernel.rs:102-111).  Same bytes as
+ * pf_backend_h2d (host_is_src != 0) / pf_backend_d2h (host_is_src == 0) of a
+ * kernel backend, enqueue only, but the device-side descriptor table lives in
+ * a fixed 1.5 MiB array inside the library's device image and the call makes
+ * no hipMalloc / hipFree / hipHostMalloc, on any call including the first.
+ * Limits: n <= pf_desc_copy_noalloc_max() (32768), more is refused with
+ * PF_ERR_INVALID_ARGUMENT; `copies` is read by the upload that the call
+ * enqueues, so it stays alive and unchanged until the stream has been
+ * synchronised (the usual descriptor rule); every call on one GPU shares the
+ * one table, so calls on different streams of that GPU need an order between
+ * them (calls on one stream are ordered by the stream). */
+int pf_desc_copy_noalloc(const pf_copy_desc* copies, uint64_t n, int host_is_src, pf_stream_t s);
+uint64_t pf_desc_copy_noalloc_max(void);
 /* TransferMode from the connector's string ("direct" | "kernel"),
  * python/pegaflow/connector/common.py:577-594. */
 int pf_transfer_mode_from_name(const char* name, int* out_mode);

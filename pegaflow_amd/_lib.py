@@ -187,6 +187,8 @@ PROTOTYPES = {
     "pf_backend_name": (C.c_char_p, [vp]),
     "pf_backend_h2d": (C.c_int, [vp, C.POINTER(PfCopyDesc), u64, vp]),
     "pf_backend_d2h": (C.c_int, [vp, C.POINTER(PfCopyDesc), u64, vp]),
+    "pf_desc_copy_noalloc": (C.c_int, [C.POINTER(PfCopyDesc), u64, C.c_int, vp]),
+    "pf_desc_copy_noalloc_max": (u64, []),
     "pf_transfer_mode_from_name": (C.c_int, [C.c_char_p, C.POINTER(C.c_int)]),
     "pf_build_copy_descs": (C.c_int, [C.POINTER(PfLayerTransfer), u64, C.POINTER(PfCopyDesc), u64,
                                       C.POINTER(u64), C.POINTER(u64)]),

@@ -11,6 +11,8 @@
 //   * all per-tile address arithmetic is wave-uniform (scalar registers).
 #include "pf_kernels.hpp"
 
+#include <mutex>
+
 #include "pf_common.hpp"
 
 namespace pf {
@@ -131,6 +133,34 @@ __global__ __launch_bounds__(kLanes) void desc_copy_kernel(const uint64_t* __res
     const uint64_t dst = table[3ull * i + 0];
     const uint64_t src = table[3ull * i + 1];
     const uint64_t size = table[3ull * i + 2];
+    const uint64_t n_tiles = (size + kTile - 1) / kTile;
+    const bool vec = ((dst | src) & 15ull) == 0;
+    for (uint64_t t = blockIdx.y; t < n_tiles; t += gridDim.y) {
+      const uint64_t off = t * kTile;
+      const uint64_t left = size - off;
+      const uint32_t bytes = left < kTile ? static_cast<uint32_t>(left) : static_cast<uint32_t>(kTile);
+      if (vec) {
+        copy_tile_vec<U>(dst + off, src + off, bytes);
+      } else {
+        copy_tile_any(dst + off, src + off, bytes);
+      }
+    }
+  }
+}
+
+// The same copy over caller-format descriptors (pf_copy_desc, 48 bytes each):
+// the table is the caller's array as it is, so the host side repacks nothing.
+// HOST_IS_SRC picks which of the two device-visible addresses is the source.
+template <int U, bool HOST_IS_SRC>
+__global__ __launch_bounds__(kLanes) void desc48_copy_kernel(
+    const pf_copy_desc* __restrict__ table, uint32_t n) {
+  constexpr uint64_t kTile = static_cast<uint64_t>(U) * kLanes * 16;
+  for (uint32_t i = blockIdx.x; i < n; i += gridDim.x) {
+    const uint64_t near_addr = table[i].device;
+    const uint64_t far_addr = table[i].host_device;
+    const uint64_t size = table[i].size;
+    const uint64_t dst = HOST_IS_SRC ? near_addr : far_addr;
+    const uint64_t src = HOST_IS_SRC ? far_addr : near_addr;
     const uint64_t n_tiles = (size + kTile - 1) / kTile;
     const bool vec = ((dst | src) & 15ull) == 0;
     for (uint64_t t = blockIdx.y; t < n_tiles; t += gridDim.y) {
@@ -492,23 +522,31 @@ int launch_plain_copy(void* dst, const void* src, uint64_t bytes, int unroll, hi
   return PF_OK;
 }
 
-int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipStream_t s,
-                     uint32_t max_workgroups) {
-  if (n == 0) return PF_OK;
+namespace {
+// Grid of a descriptor-copy launch: x over descriptors, y over the tiles of the
+// largest one.  The kernels stride in both dimensions, so any grid covers the
+// batch; `max_workgroups` (0 = no cap) bounds the whole launch.
+dim3 desc_copy_grid(uint64_t n, uint64_t max_size, uint32_t max_workgroups) {
   constexpr uint64_t kTile = tile_bytes(kDescUnroll);
   uint64_t gx = n < kMaxGridX ? n : kMaxGridX;
   uint64_t gy = (max_size + kTile - 1) / kTile;
   if (gy < 1) gy = 1;
   if (gy > 64) gy = 64;
   if (max_workgroups != 0) {
-    // The kernel strides over descriptors and tiles, so any grid covers the batch.
     while (gx * gy > max_workgroups && gy > 1) gy >>= 1;
     if (gx * gy > max_workgroups) gx = max_workgroups / gy ? max_workgroups / gy : 1;
   }
-  // Keep the launch to a few million workgroups; the kernel strides in both
-  // dimensions, so a smaller grid only means more iterations per workgroup.
+  // Keep the launch to a few million workgroups; a smaller grid only means
+  // more iterations per workgroup.
   while (gx * gy > (1ull << 22) && gy > 1) gy >>= 1;
-  dim3 grid(static_cast<uint32_t>(gx), static_cast<uint32_t>(gy), 1), block(kLanes, 1, 1);
+  return dim3(static_cast<uint32_t>(gx), static_cast<uint32_t>(gy), 1);
+}
+}  // namespace
+
+int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipStream_t s,
+                     uint32_t max_workgroups) {
+  if (n == 0) return PF_OK;
+  const dim3 grid = desc_copy_grid(n, max_size, max_workgroups), block(kLanes, 1, 1);
   hipLaunchKernelGGL(desc_copy_kernel<kDescUnroll>, grid, block, 0, s, table,
                      static_cast<uint32_t>(n));
   hipError_t e = hipGetLastError();
@@ -517,3 +555,101 @@ int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipSt
 }
 
 }  // namespace pf
+
+// ---------------------------------------------------------------------------
+// Descriptor copy that allocates nothing
+// ---------------------------------------------------------------------------
+//
+// The kernel backend keeps its descriptor table in device memory it allocates
+// (and grows) on demand.  Callers that must not allocate get the same copy with
+// the table in a fixed array that is part of the library's device image.  Every
+// GPU the library runs on holds its own copy of the array, at its own address,
+// until the process ends; every call on a GPU shares it, so calls that overlap
+// on one GPU (different streams, no ordering between them) race on the table.
+// Nothing in it has to start at zero: a call overwrites rows [0, n) before its
+// kernel reads exactly those rows.
+
+// Most descriptors one call takes: 32768 x 48 bytes = 1.5 MiB per GPU.
+#define PF_NOALLOC_MAX_DESCS 32768u
+
+static __device__ __align__(256) unsigned char scratch[PF_NOALLOC_MAX_DESCS * sizeof(pf_copy_desc)];
+
+namespace {
+
+constexpr int kNoAllocMaxDevices = 64;
+// Same cap as the kernel backend: the host link wants few requesters.
+constexpr uint32_t kNoAllocWorkgroups = 64;
+
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kNoAllocMaxDevices] = {};
+
+// Device address of `scratch` on the current device.  The array's name is only
+// a host-side handle for the symbol; the address comes from the runtime, once
+// per device, and is what every later use takes.
+int scratch_on_current_device(void** out) {
+  int device = -1;
+  PF_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kNoAllocMaxDevices) {
+    return pf::fail(PF_ERR_INVALID_ARGUMENT, "device %d is beyond the %d this call supports",
+                    device, kNoAllocMaxDevices);
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (g_scratch_ptr[device] == nullptr) {
+    void* ptr = nullptr;
+    PF_HIP(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) {
+      return pf::fail(PF_ERR_DEVICE_INIT, "hipGetSymbolAddress(scratch) returned a null address");
+    }
+    g_scratch_ptr[device] = ptr;
+  }
+  *out = g_scratch_ptr[device];
+  return PF_OK;
+}
+
+}  // namespace
+
+extern "C" int pf_desc_copy_noalloc(const pf_copy_desc* copies, uint64_t n, int host_is_src,
+                                    pf_stream_t s) {
+  if (n == 0) return PF_OK;
+  PF_REQUIRE_PTR(copies);
+  if (n > PF_NOALLOC_MAX_DESCS) {
+    return pf::fail(PF_ERR_INVALID_ARGUMENT,
+                    "pf_desc_copy_noalloc takes at most %u descriptors per call, got %llu "
+                    "(split the batch, or use pf_backend_h2d / pf_backend_d2h)",
+                    PF_NOALLOC_MAX_DESCS, static_cast<unsigned long long>(n));
+  }
+  uint64_t max_size = 0;
+  for (uint64_t i = 0; i < n; ++i) {
+    const pf_copy_desc& c = copies[i];
+    if (c.size != 0 && (c.device == 0 || c.host_device == 0)) {
+      // The kernel dereferences both addresses; a null one would fault the GPU.
+      return pf::fail(PF_ERR_INVALID_ARGUMENT,
+                      "descriptor %llu: the copy kernel needs a device address and a "
+                      "device-visible host address",
+                      static_cast<unsigned long long>(i));
+    }
+    if (c.size > max_size) max_size = c.size;
+  }
+  if (max_size == 0) return PF_OK;
+  void* table = nullptr;
+  int st = scratch_on_current_device(&table);
+  if (st != PF_OK) return st;
+  hipStream_t stream = pf::native(s);
+  // The caller's array is the table: one copy, in stream order behind the
+  // previous call's kernel on this stream.
+  PF_HIP(hipMemcpyAsync(table, copies, n * sizeof(pf_copy_desc), hipMemcpyHostToDevice, stream));
+  const dim3 grid = pf::desc_copy_grid(n, max_size, kNoAllocWorkgroups), block(pf::kLanes, 1, 1);
+  const pf_copy_desc* rows = static_cast<const pf_copy_desc*>(table);
+  if (host_is_src) {
+    hipLaunchKernelGGL((pf::desc48_copy_kernel<pf::kDescUnroll, true>), grid, block, 0, stream, rows,
+                       static_cast<uint32_t>(n));
+  } else {
+    hipLaunchKernelGGL((pf::desc48_copy_kernel<pf::kDescUnroll, false>), grid, block, 0, stream,
+                       rows, static_cast<uint32_t>(n));
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return pf::fail_hip(e, "desc48_copy_kernel launch");
+  return PF_OK;
+}
+
+extern "C" uint64_t pf_desc_copy_noalloc_max(void) { return PF_NOALLOC_MAX_DESCS; }

@@ -112,6 +112,20 @@ class TransferBackend:
             pass
 
 
+def desc_copy_noalloc(copies, stream: Stream, host_is_src: bool):
+    """The kernel backend's copy through ``pf_desc_copy_noalloc``: nothing is
+    allocated, the batch is limited to ``desc_copy_noalloc_max()`` descriptors.
+    Returns the packed descriptor array, which the caller keeps alive until
+    the stream has been synchronised."""
+    arr, n = _pack(copies)
+    check(_lib.load().pf_desc_copy_noalloc(arr, n, 1 if host_is_src else 0, stream.handle))
+    return arr
+
+
+def desc_copy_noalloc_max() -> int:
+    return int(_lib.load().pf_desc_copy_noalloc_max())
+
+
 class MemcpyBackend(TransferBackend):
     """One DMA copy per merged range ("direct")."""
 
