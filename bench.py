@@ -34,15 +34,40 @@ if ROOT not in sys.path:
 
 PCIE_GEN5_X16_GBPS = 63.0   # 32 GT/s x 16 lanes x 128/130 / 8
 HBM_PEAK_GBPS = 8000.0      # MI355X published HBM3E bandwidth
-# HBM bytes one staged gather/scatter launch moves (mean over the launches of a
-# step) at each workload's default shape, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of this script: KiB per dispatch, scaled by what a plain copy
-# of exactly 1 GiB reads on the same counters (x2.000 and x1.000).
-MEASURED_TRAFFIC_STAGED = {
-    "llama8b": int((160399.4 * 2.000 + 320000.0 * 1.000) * 1024),
-    "llama70b_fp8": int((131709.5 * 2.000 + 262144.0 * 1.000) * 1024),
-    "dsv3_mla": int((249954.4 * 2.000 + 499712.0 * 1.000) * 1024),
+# rocprofv3 summaries of the staged gather/scatter kernel, one per workload.  Each
+# carries one line `traffic-record: key=value ...` with the HBM bytes a launch
+# moved (FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same counters
+# read for a plain copy of exactly 1 GiB) and the algorithmic bytes of the
+# launches it was measured on; `roofline.traffic` is read from there and only
+# reported when this run's launches have that same algorithmic size.
+TRAFFIC_PROFILES = {
+    "llama8b": "block_tiles_kernel_llama8b_save_load.md",
+    "llama70b_fp8": "block_tiles_kernel_llama70b_fp8_save_load.md",
+    "dsv3_mla": "block_tiles_kernel_dsv3_mla_page_first_save_load.md",
 }
+
+
+def measured_traffic(workload, alg_bytes_per_launch):
+    """(bytes per launch, source file) from the committed profile summary of this
+    workload, or (None, reason) when there is none for launches of this size."""
+    name = TRAFFIC_PROFILES.get(workload)
+    path = os.path.join(ROOT, "profiles", name) if name else None
+    if not path or not os.path.exists(path):
+        return None, "no profile summary for this workload"
+    rec = None
+    with open(path) as f:
+        for line in f:
+            if line.startswith("traffic-record:"):
+                rec = dict(kv.split("=", 1) for kv in line.split()[1:])
+    if rec is None:
+        return None, f"profiles/{name} has no traffic-record line"
+    if abs(float(rec["alg_bytes"]) - alg_bytes_per_launch) > 0.005 * alg_bytes_per_launch:
+        return None, (f"profiles/{name} was measured on launches of {rec['alg_bytes']} algorithmic "
+                      f"bytes, this run's move {int(alg_bytes_per_launch)}")
+    total = (float(rec["fetch_kib"]) * float(rec["fetch_scale"]) +
+             float(rec["write_kib"]) * float(rec["write_scale"])) * 1024
+    return int(round(total)), f"profiles/{name}"
+
 
 WORKLOADS = {
     # BASELINE configs[1] (save) + configs[2] (load)
@@ -201,25 +226,26 @@ def main():
         page = topo.shard_page_size(0)
         assert page * n == payload
         offsets = [topo.page_placement(topo.layer_id(nm))[0] for nm in names]
-        page_host = (pool.host_ptr + np.arange(n, dtype=np.uint64) * page).astype(np.uint64)
-        page_dev = (pool.device_ptr + np.arange(n, dtype=np.uint64) * page).astype(np.uint64)
+        pages = np.arange(n, dtype=np.uint64) * page
 
-        def layers_for(caches, ids):
-            return [LayerBlocks(layout=L, block_ids=ids, page_host=page_host,
-                                page_host_device=page_dev, page_offset=offsets[li], page_len=page,
-                                layer_name=names[li])
+        def layers_for(caches, ids, mem=pool):
+            return [LayerBlocks(layout=L, block_ids=ids,
+                                page_host=(mem.host_ptr + pages).astype(np.uint64),
+                                page_host_device=(mem.device_ptr + pages).astype(np.uint64),
+                                page_offset=offsets[li], page_len=page, layer_name=names[li])
                     for li, L in enumerate(layouts_for(caches))]
     else:
+        page, offsets = 0, None
         buf = n * seg  # one host segment buffer (K or V) of one layer
 
-        def layers_for(caches, ids):
+        def layers_for(caches, ids, mem=pool):
             out = []
             for li, L in enumerate(layouts_for(caches)):
                 off = li * payload_per_layer
                 out.append(LayerBlocks(
                     layout=L, block_ids=ids,
-                    host=tuple(pool.host_ptr + off + s * buf for s in range(nseg)),
-                    host_device=tuple(pool.device_ptr + off + s * buf for s in range(nseg)),
+                    host=tuple(mem.host_ptr + off + s * buf for s in range(nseg)),
+                    host_device=tuple(mem.device_ptr + off + s * buf for s in range(nseg)),
                     host_len=tuple(buf for _ in range(nseg)), host_stride=seg,
                     layer_name=names[li]))
             return out
@@ -288,21 +314,10 @@ def main():
     load_gbps = payload * args.steps / (load_ms / 1e3) / 1e9
 
     # ---- byte-exactness of what was just timed (untimed) -------------------
-    pool_t = torch.from_numpy(pool.as_numpy())
-    sid = torch.from_numpy(save_ids.astype(np.int64))
-    lid = torch.from_numpy(load_ids.astype(np.int64))
-    for li in sorted({0, n_layers - 1}):
-        src = src_cache[li].view(torch.uint8).reshape(nseg, nb, seg)
-        want = src[:, sid.to(dev)].cpu()                       # [nseg, n, seg]
-        if w["page_first"]:
-            img = pool_t.reshape(n, page)[:, offsets[li]:offsets[li] + seg].reshape(1, n, seg)
-        else:
-            img = pool_t[li * payload_per_layer:(li + 1) * payload_per_layer].reshape(nseg, n, seg)
-        assert torch.equal(img, want), f"layer {li}: saved image differs from the device cache"
-        dst = dst_cache[li].view(torch.uint8).reshape(nseg, nb, seg).cpu()
-        expect = torch.zeros_like(dst)
-        expect[:, lid] = want
-        assert torch.equal(dst, expect), f"layer {li}: loaded cache differs"
+    checker = ByteChecker(torch, np, runtime, stream, w, src_cache, dst_cache, save_ids, load_ids,
+                          payload_per_layer, page, offsets)
+    checker.image(pool, "timed steps")
+    checker.destination("timed steps")
 
     # ---- link peak: one large contiguous pinned <-> device copy -----------
     link_bytes = min(1 << 30, payload)
@@ -377,17 +392,17 @@ def main():
     launches = live_launches_per_step
     assert launches == alone_launches, (launches, alone_launches)
     bytes_per_launch = 2 * payload / max(launches, 1)          # payload bytes one launch moves
-    default_shape = not args.layers and not args.slot_mb
     # staged: every payload byte is read once and written once in HBM -> 2 x
     # payload algorithmic bytes per launch; zero-copy: the kernel touches HBM
     # once per payload byte and is bounded by the host link, not by HBM
     staged_path = used_path == "staged"
     alg_bytes = (2 if staged_path else 1) * bytes_per_launch
     achieved = alg_bytes / (live_launch_ms / 1e3) / 1e9
+    traffic, traffic_source = (measured_traffic(args.workload, alg_bytes) if staged_path
+                               else (None, "zero-copy launches are not profiled for HBM traffic"))
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                "traffic": (MEASURED_TRAFFIC_STAGED[args.workload]
-                            if staged_path and default_shape else None),
+                "traffic": traffic, "traffic_source": traffic_source,
                 "kernel": ("block_tiles_kernel (staged gather/scatter)" if staged_path
                            else "block_units_kernel (zero-copy, host-link bound)"),
                 "measured": f"HIP events around each of the {live['launches']} launches of the "
@@ -412,22 +427,44 @@ def main():
             "save_frac_of_theoretical": round(save_gbps / PCIE_GEN5_X16_GBPS, 4),
             "load_frac_of_theoretical": round(load_gbps / PCIE_GEN5_X16_GBPS, 4)}
 
+    # The resource that bounds the step is the host link: payload bytes cross it
+    # once, so achieved = payload / time against PCIe Gen5 x16, with the box's
+    # measured one-large-copy rate beside the theoretical peak.
+    link_t = (save_ms + load_ms) / 1e3
+    link_achieved = 2 * payload * args.steps / link_t / 1e9
+    link_measured = 2.0 / (1.0 / d2h_peak + 1.0 / h2d_peak)   # same bytes each way
+    roofline["link"] = {"bound": "pcie_gen5_x16", "achieved": round(link_achieved, 2),
+                        "peak": PCIE_GEN5_X16_GBPS, "unit": "GB/s",
+                        "frac": round(link_achieved / PCIE_GEN5_X16_GBPS, 4),
+                        "measured_peak": round(link_measured, 2),
+                        "frac_of_measured": round(link_achieved / link_measured, 4),
+                        "alg_bytes_per_step": 2 * payload,
+                        "measured": "stream events around the save pass and the load pass of "
+                                    "every timed step; measured_peak = one 1 GiB hipMemcpyAsync "
+                                    "each way in this run (harmonic mean of d2h and h2d)"}
+
     # ---- compute overlap (configs[2]): transfers next to a GEMM stream ----
     overlap = None
     if not args.no_overlap:
-        overlap = run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_layers)
+        overlap = run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_layers,
+                              checker, pool)
 
     # ---- both directions at once (the worker pool runs a load thread and a
     # save thread per GPU: gpu_worker.rs:116-345 of the reference) ----------
     duplex = None
     if not args.no_overlap:
-        duplex = run_duplex(xfer, save_layers, load_layers, stream, path, payload, args)
+        pool2 = PinnedMemory(payload)
+        duplex = run_duplex(layers_for(src_cache, save_ids, pool2), load_layers, path, payload, args,
+                            checker, pool, pool2, runtime)
+        pool2.close()
 
     # ---- the same workload through the save / query / load engine -----------
     # In a process of its own, as the engine is deployed (a server that runs
     # nothing else on the GPU): which link copies the runtime overlaps depends
     # on the history of a process's streams, and this process has used many by
     # now.  The child allocates its own caches, so this one releases its first.
+    byte_checks = list(checker.checked)
+    del checker
     xfer.close()
     stream.close()
     pool.close()
@@ -489,15 +526,104 @@ def main():
         "overlap": overlap,
         "duplex": duplex,
         "engine": engine,
+        "byte_checks": byte_checks,
         "pool_alloc_s": round(pool_alloc_s, 2),
         "device": runtime.device_name(0),
     }
     print(json.dumps(result))
 
 
-def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_layers):
-    """Transfer alone, GEMM stream alone, then both at once (load and save)."""
-    from pegaflow_amd.runtime import Event
+class ByteChecker:
+    """Byte checks of what the bench moves, on every layer: the host image holds
+    block save_ids[i] of the source cache at list position i (K buffer then V
+    buffer per layer, or one page per block with the layers at their offsets),
+    and the destination cache holds it at block load_ids[i] with every other
+    block still zero.  The comparisons run on the device (the image is uploaded
+    a piece at a time); a difference ends the bench with exit status 1."""
+
+    PAGES_PER_PIECE = 128
+
+    def __init__(self, torch, np, runtime, stream, w, src, dst, save_ids, load_ids,
+                 payload_per_layer, page, offsets):
+        self.torch, self.runtime, self.stream = torch, runtime, stream
+        self.src, self.dst = src, dst
+        self.nb, self.seg, self.n = w["num_blocks"], w["seg"], w["n"]
+        self.nseg = 2 if w["split"] else 1
+        self.page_first, self.page, self.offsets = w["page_first"], page, offsets
+        self.payload_per_layer = payload_per_layer
+        dev = src[0].device
+        self.sid = torch.from_numpy(save_ids.astype(np.int64)).to(dev)
+        self.lid = torch.from_numpy(load_ids.astype(np.int64)).to(dev)
+        untouched = torch.ones(self.nb, dtype=torch.bool, device=dev)
+        untouched[self.lid] = False
+        self.rest = torch.nonzero(untouched).reshape(-1)
+        piece = self.PAGES_PER_PIECE * page if self.page_first else payload_per_layer
+        self.piece = torch.empty(piece, device=dev, dtype=torch.uint8)
+        self.zeros = torch.zeros(piece, device=dev, dtype=torch.uint8)
+        self.checked = []
+
+    def _fail(self, message):
+        print("bench.py: byte check failed: " + message, file=sys.stderr)
+        sys.exit(1)
+
+    def _pieces(self, total):
+        step = self.piece.numel()
+        return [(o, min(step, total - o)) for o in range(0, total, step)]
+
+    def clear_image(self, pool):
+        total = self.n * self.page if self.page_first else self.payload_per_layer * len(self.src)
+        for off, size in self._pieces(total):
+            self.runtime.memcpy_d2h_async(pool.host_ptr + off, self.zeros.data_ptr(), size, self.stream)
+        self.stream.synchronize()
+
+    def clear_destination(self):
+        for t in self.dst:
+            t.zero_()
+        self.torch.cuda.synchronize()
+
+    def _upload(self, pool, off, size):
+        self.runtime.memcpy_h2d_async(self.piece.data_ptr(), pool.host_ptr + off, size, self.stream)
+        self.stream.synchronize()
+
+    def image(self, pool, what):
+        torch = self.torch
+        if self.page_first:
+            for off, size in self._pieces(self.n * self.page):
+                self._upload(pool, off, size)
+                first, k = off // self.page, size // self.page
+                got = self.piece[:size].view(k, self.page)
+                for li, cache in enumerate(self.src):
+                    want = cache.view(torch.uint8).view(self.nb, self.seg)[self.sid[first:first + k]]
+                    lo = self.offsets[li]
+                    if not torch.equal(got[:, lo:lo + self.seg], want):
+                        self._fail(f"{what}: host pages {first}..{first + k - 1}, layer {li}")
+        else:
+            for li, cache in enumerate(self.src):
+                self._upload(pool, li * self.payload_per_layer, self.payload_per_layer)
+                want = cache.view(torch.uint8).view(self.nseg, self.nb, self.seg)[:, self.sid]
+                if not torch.equal(self.piece.view(self.nseg, self.n, self.seg), want):
+                    self._fail(f"{what}: host image of layer {li} differs from the device cache")
+        self.checked.append(f"{what}: host image, {len(self.src)} layers")
+
+    def destination(self, what):
+        torch = self.torch
+        for li, (s_, d_) in enumerate(zip(self.src, self.dst)):
+            s_ = s_.view(torch.uint8).view(self.nseg, self.nb, self.seg)
+            d_ = d_.view(torch.uint8).view(self.nseg, self.nb, self.seg)
+            if not torch.equal(d_[:, self.lid], s_[:, self.sid]):
+                self._fail(f"{what}: layer {li}: loaded blocks differ")
+            if bool(d_[:, self.rest].any()):
+                self._fail(f"{what}: layer {li}: a block outside the list changed")
+        self.checked.append(f"{what}: destination cache, {len(self.dst)} layers")
+
+
+def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_layers, checker,
+                pool):
+    """Transfer alone, GEMM stream alone, then both at once (load and save).
+    The pass that runs next to the GEMM stream starts from a cleared target and
+    is byte-checked on every layer; the GEMM's result is compared with the one
+    it gives alone."""
+    from pegaflow_amd.runtime import Event, Stream
     dev = torch.device("cuda:0")
     m = 4096
     a = torch.randn(m, m, device=dev, dtype=torch.bfloat16)
@@ -509,46 +635,96 @@ def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_
     e0, e1 = Event(timing=True), Event(timing=True)
     layer_ev = [Event(timing=True) for _ in range(n_layers)]
 
-    def gemms(count):
+    ticks = []   # (GEMMs launched so far, event on the GEMM stream), one per 64 GEMMs
+
+    def gemms(count, tick_pool=None):
+        del ticks[:]
         with torch.cuda.stream(gemm_stream):
             g0.record()
-            for _ in range(count):
+            for i in range(count):
                 torch.matmul(a, b, out=c)
+                if tick_pool is not None and i % 64 == 63 and i // 64 < len(tick_pool):
+                    tick_pool[i // 64].record(gemm_native)
+                    ticks.append((i + 1, tick_pool[i // 64]))
             g1.record()
 
     gemms(50)
     torch.cuda.synchronize()
+    host0 = time.perf_counter()
     gemms(200)
+    enqueue_ms = (time.perf_counter() - host0) * 1e3 / 200     # host time per launch
     torch.cuda.synchronize()
     gemm_alone_ms = g0.elapsed_time(g1) / 200
+    # The device works through the GEMMs while the host still launches them: the
+    # backlog left when the launches end grows by (GEMM time - launch time) per
+    # GEMM, and it has to outlast the transfer that is enqueued after them.
+    backlog_per_gemm_ms = max(gemm_alone_ms - enqueue_ms, 0.1 * gemm_alone_ms)
+    gemm_native = Stream.wrap(gemm_stream.cuda_stream)
+    m0, m1 = Event(timing=True), Event(timing=True)
+    tick_pool = [Event(timing=True) for _ in range(512)]
+    c_alone = c.clone()
     out = {"gemm": "4096x4096x4096 bf16, back to back on its own stream",
            "gemm_alone_tflops": round(flop / (gemm_alone_ms / 1e3) / 1e12, 1)}
+    gemm_ok = True
     for name, fn, layers in (("load", xfer.load, load_layers), ("save", xfer.save, save_layers)):
         e0.record(stream)
         fn(layers, stream, path)
         e1.record(stream)
         e1.synchronize()
         alone_ms = e0.elapsed_ms(e1)
-        count = max(50, int(alone_ms / gemm_alone_ms * 1.2))
+        count = max(50, int(1.6 * alone_ms / backlog_per_gemm_ms))
         if name == "load":
             xfer.set_layer_events(layer_ev)
-        gemms(count)
+            checker.clear_destination()
+        else:
+            checker.clear_image(pool)
+        c.zero_()
+        torch.cuda.synchronize()
+        m0.record(gemm_native)
+        gemms(count, tick_pool)
+        m1.record(gemm_native)
         e0.record(stream)
         fn(layers, stream, path)
         e1.record(stream)
         e1.synchronize()
         torch.cuda.synchronize()
+        # share of the transfer during which the GEMM stream was running
+        begin, end = m0.elapsed_ms(e0), m0.elapsed_ms(e1)
+        together = (min(m0.elapsed_ms(m1), end) - max(0.0, begin)) / (end - begin)
         xfer.set_layer_events(None)
         both_ms = e0.elapsed_ms(e1)
-        out[f"gemm_with_{name}_tflops"] = round(flop / (g0.elapsed_time(g1) / count / 1e3) / 1e12, 1)
+        if name == "load":
+            checker.destination("load next to the GEMM stream")
+        else:
+            checker.image(pool, "save next to the GEMM stream")
+        gemm_ok = gemm_ok and bool(torch.equal(c, c_alone))
+        # GEMM rate while the transfer was in flight: between the first and the last
+        # of the marks (one per 64 GEMMs) that fell inside the transfer's span
+        inside = [(k, m0.elapsed_ms(ev)) for k, ev in ticks]
+        inside = [(k, t) for k, t in inside if begin <= t <= end]
+        if len(inside) >= 2:
+            during_ms = (inside[-1][1] - inside[0][1]) / (inside[-1][0] - inside[0][0])
+            out[f"gemm_with_{name}_tflops"] = round(flop / (during_ms / 1e3) / 1e12, 1)
+        else:
+            out[f"gemm_with_{name}_tflops"] = None
+        out[f"gemm_stream_with_{name}_tflops_whole_run"] = round(
+            flop / (g0.elapsed_time(g1) / count / 1e3) / 1e12, 1)
         out[f"{name}_alone_gbps"] = round(payload / (alone_ms / 1e3) / 1e9, 2)
         out[f"{name}_with_gemm_gbps"] = round(payload / (both_ms / 1e3) / 1e9, 2)
+        out[f"{name}_share_next_to_gemm"] = round(together, 3)
         if name == "load":
             done = [e0.elapsed_ms(le) for le in layer_ev]
             per_layer = [done[0]] + [done[i] - done[i - 1] for i in range(1, len(done))]
             out["per_layer_ms_mean"] = round(sum(per_layer) / len(per_layer), 3)
             out["per_layer_ms_max"] = round(max(per_layer), 3)
             out["first_layer_ready_ms"] = round(done[0], 3)
+    if not gemm_ok:
+        print("bench.py: the GEMM next to a transfer differs from the GEMM alone", file=sys.stderr)
+        sys.exit(1)
+    out["verified"] = True
+    out["verified_what"] = ("every layer of the destination caches (load) and of the host image (save) "
+                            "after the passes that ran next to the GEMM stream; GEMM result equal to "
+                            "the GEMM alone")
     return out
 
 
@@ -758,30 +934,62 @@ def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, pa
     return out
 
 
-def run_duplex(xfer, save_layers, load_layers, stream, path, payload, args):
+def run_duplex(save_layers2, load_layers, path, payload, args, checker, pool, pool2, runtime):
     """A save and a load in flight together, each with its own stream and
-    engine, as the two worker threads of one GPU issue them.  (The load reads
-    the host image while the save rewrites it with the same bytes; only the
-    rates are used.)  Two forms: link copies on each engine's side stream (the
+    engine, as the two worker threads of one GPU issue them: the load scatters
+    the host image of `pool` while the save gathers the same source blocks into
+    a second pool.  Two forms: link copies on each engine's side stream (the
     stand-alone default) and on the callers' streams (what the worker pool
-    configures, so that the two directions never share a hardware queue)."""
+    configures).  `plain_pair_gbps` is the yardstick: two plain hipMemcpyAsync
+    streams, 1 GiB copies, one stream per direction, in this same run.  The last
+    pass of each form starts from cleared targets and is byte-checked."""
     from pegaflow_amd.runtime import Event, Stream
     from pegaflow_amd.transfer import BlockTransfer
     out = {}
     ev = [Event(timing=True) for _ in range(4)]
+
+    # -- yardstick: plain copies, both directions at once --------------------
+    piece = min(1 << 30, payload // 2)
+    dbuf = checker.torch.empty(2 * piece, device=checker.src[0].device, dtype=checker.torch.uint8)
+    sa, sb = Stream(), Stream()
+
+    def pair(reps):
+        ev[0].record(sa)
+        ev[2].record(sb)
+        for _ in range(reps):
+            runtime.memcpy_d2h_async(pool2.host_ptr, dbuf.data_ptr(), piece, sa)
+            runtime.memcpy_h2d_async(dbuf.data_ptr() + piece, pool2.host_ptr + piece, piece, sb)
+        ev[1].record(sa)
+        ev[3].record(sb)
+        ev[1].synchronize()
+        ev[3].synchronize()
+        span = max(ev[0].elapsed_ms(ev[1]), ev[0].elapsed_ms(ev[3])) - min(0.0, ev[0].elapsed_ms(ev[2]))
+        return {"d2h_gbps": round(piece * reps / ev[0].elapsed_ms(ev[1]) / 1e6, 2),
+                "h2d_gbps": round(piece * reps / ev[2].elapsed_ms(ev[3]) / 1e6, 2),
+                "aggregate_gbps": round(2 * piece * reps / span / 1e6, 2)}
+    pair(1)
+    out["plain_pair"] = pair(5)
+    out["plain_pair_gbps"] = out["plain_pair"]["aggregate_gbps"]
+    sa.close()
+    sb.close()
+    del dbuf
+
     for label, mode in (("side_stream_copies", 1), ("in_order_copies", 2)):
         xa, xb = (BlockTransfer(staging_slot_bytes=args.slot_mb << 20, staging_slots=args.slots,
                                 tile_unroll=args.unroll, zerocopy_max_workgroups=args.zc_max_wg,
                                 copy_stream=mode) for _ in range(2))
         sa, sb = Stream(), Stream()
-        xa.save(save_layers, sa, path)   # allocate staging
+        xa.save(save_layers2, sa, path)   # allocate staging
         xb.load(load_layers, sb, path)
         sa.synchronize()
         sb.synchronize()
-        for _ in range(2):
+        for rep in range(2):
+            if rep == 1:
+                checker.clear_image(pool2)
+                checker.clear_destination()
             ev[0].record(sa)
             ev[2].record(sb)
-            xa.save(save_layers, sa, path)
+            xa.save(save_layers2, sa, path)
             xb.load(load_layers, sb, path)
             ev[1].record(sa)
             ev[3].record(sb)
@@ -791,9 +999,15 @@ def run_duplex(xfer, save_layers, load_layers, stream, path, payload, args):
             span_ms = max(ev[0].elapsed_ms(ev[1]), ev[0].elapsed_ms(ev[3]))
             out[label] = {"save_gbps": round(payload / save_ms / 1e6, 2),
                           "load_gbps": round(payload / load_ms / 1e6, 2),
-                          "aggregate_gbps": round(2 * payload / span_ms / 1e6, 2)}
+                          "aggregate_gbps": round(2 * payload / span_ms / 1e6, 2),
+                          "frac_of_plain_pair": round(2 * payload / span_ms / 1e6 /
+                                                      out["plain_pair_gbps"], 4)}
+        checker.image(pool2, f"save next to a load ({label})")
+        checker.image(pool, f"image read by the load ({label})")
+        checker.destination(f"load next to a save ({label})")
         for o in (xa, xb, sa, sb):
             o.close()
+    out["verified"] = True
     return out
 
 

@@ -297,7 +297,8 @@ typedef struct pf_layer_blocks {
 typedef struct pf_xfer_config {
   uint64_t staging_slot_bytes; /* 0 = default */
   uint32_t staging_slots;      /* 0 = default (2) */
-  uint32_t zerocopy_max_workgroups; /* 0 = default (64); workgroups of a zero-copy launch */
+  uint32_t zerocopy_max_workgroups; /* workgroups of a zero-copy launch; 0 = default (16 for
+                                       fragments of 16 KiB and more, up to 64 for smaller ones) */
   uint64_t auto_staged_min_bytes;   /* 0 = default threshold for PF_PATH_AUTO */
   uint32_t tile_unroll;             /* zero-copy kernel: 16-byte loads in flight per lane:
                                        1,2,4,8; 0 = default (4) */

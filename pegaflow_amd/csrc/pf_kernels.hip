@@ -176,54 +176,61 @@ __global__ __launch_bounds__(kLanes) void desc48_copy_kernel(
   }
 }
 
-// Block-ID gather / scatter.  blockIdx.y selects the unit, blockIdx.x strides
-// over its tiles.  Tile order is (segment, list position, tile in fragment),
-// so consecutive workgroups touch consecutive far-side addresses.
+// Block-ID gather / scatter over mapped host memory (the zero-copy form).  The
+// grid is one row of workgroups, as many as the launch may keep on the device;
+// all of them walk the units one after the other and stride over the tiles of
+// each, so the units complete in order and the workgroup count does not grow
+// with the number of units.  Tile order inside a unit is (segment, list
+// position, tile in fragment), so at any moment the workgroups touch
+// neighbouring far-side addresses.
 template <int U, bool TO_FAR>
-__global__ __launch_bounds__(kLanes) void block_units_kernel(const BlockUnit* __restrict__ units) {
+__global__ __launch_bounds__(kLanes) void block_units_kernel(const BlockUnit* __restrict__ units,
+                                                             uint32_t n_units) {
   constexpr uint64_t kTile = static_cast<uint64_t>(U) * kLanes * 16;
-  // Every field below is wave-uniform: read once into scalar registers.
-  const BlockUnit* __restrict__ up = units + blockIdx.y;
-  const uint64_t near_base = up->near_base;
-  const uint64_t block_stride = up->block_stride;
-  const uint64_t kv_stride = up->kv_stride;
-  const uint64_t frag_bytes = up->frag_bytes;
-  const uint64_t far_base0 = up->far_base[0];
-  const uint64_t far_base1 = up->far_base[1];
-  const uint64_t far_stride = up->far_stride;
-  c_u32* ids = reinterpret_cast<c_u32*>(reinterpret_cast<uint64_t>(up->ids));
-  c_u64* far_table = reinterpret_cast<c_u64*>(reinterpret_cast<uint64_t>(up->far_table));
-  const bool paged = up->far_table != nullptr;
-  const uint64_t far_table_off = up->far_table_off;
-  const uint32_t tiles_per_frag = up->tiles_per_frag;
-  const bool vec_ok = up->vec_ok != 0;
-  // The host keeps a unit's tile count below 2^32, so 32-bit scalar division.
-  const uint32_t tiles_per_seg = up->n_blocks * tiles_per_frag;
-  const uint32_t n_tiles = tiles_per_seg * up->n_seg;
-  for (uint32_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
-    const uint32_t seg = t >= tiles_per_seg ? 1u : 0u;
-    const uint32_t r = seg ? t - tiles_per_seg : t;
-    // The quotient is wave-uniform; pin it to a scalar register so the id and
-    // page-table reads below are scalar loads.
-    const uint32_t pos = __builtin_amdgcn_readfirstlane(r / tiles_per_frag);
-    const uint32_t c = r - pos * tiles_per_frag;
-    const uint64_t off = static_cast<uint64_t>(c) * kTile;
-    const uint64_t left = frag_bytes - off;
-    const uint32_t bytes = left < kTile ? static_cast<uint32_t>(left) : static_cast<uint32_t>(kTile);
-    const uint64_t id = ids[pos];
-    const uint64_t near_addr = near_base + id * block_stride + (seg ? kv_stride : 0) + off;
-    uint64_t far_addr;
-    if (paged) {
-      far_addr = far_table[pos] + far_table_off + (seg ? frag_bytes : 0) + off;
-    } else {
-      far_addr = (seg ? far_base1 : far_base0) + static_cast<uint64_t>(pos) * far_stride + off;
-    }
-    const uint64_t dst = TO_FAR ? far_addr : near_addr;
-    const uint64_t src = TO_FAR ? near_addr : far_addr;
-    if (vec_ok) {
-      copy_tile_vec<U>(dst, src, bytes);
-    } else {
-      copy_tile_any(dst, src, bytes);
+  for (uint32_t unit = 0; unit < n_units; ++unit) {
+    // Every field below is wave-uniform: read once into scalar registers.
+    const BlockUnit* __restrict__ up = units + unit;
+    const uint64_t near_base = up->near_base;
+    const uint64_t block_stride = up->block_stride;
+    const uint64_t kv_stride = up->kv_stride;
+    const uint64_t frag_bytes = up->frag_bytes;
+    const uint64_t far_base0 = up->far_base[0];
+    const uint64_t far_base1 = up->far_base[1];
+    const uint64_t far_stride = up->far_stride;
+    c_u32* ids = reinterpret_cast<c_u32*>(reinterpret_cast<uint64_t>(up->ids));
+    c_u64* far_table = reinterpret_cast<c_u64*>(reinterpret_cast<uint64_t>(up->far_table));
+    const bool paged = up->far_table != nullptr;
+    const uint64_t far_table_off = up->far_table_off;
+    const uint32_t tiles_per_frag = up->tiles_per_frag;
+    const bool vec_ok = up->vec_ok != 0;
+    // The host keeps a unit's tile count below 2^32, so 32-bit scalar division.
+    const uint32_t tiles_per_seg = up->n_blocks * tiles_per_frag;
+    const uint32_t n_tiles = tiles_per_seg * up->n_seg;
+    for (uint32_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
+      const uint32_t seg = t >= tiles_per_seg ? 1u : 0u;
+      const uint32_t r = seg ? t - tiles_per_seg : t;
+      // The quotient is wave-uniform; pin it to a scalar register so the id and
+      // page-table reads below are scalar loads.
+      const uint32_t pos = __builtin_amdgcn_readfirstlane(r / tiles_per_frag);
+      const uint32_t c = r - pos * tiles_per_frag;
+      const uint64_t off = static_cast<uint64_t>(c) * kTile;
+      const uint64_t left = frag_bytes - off;
+      const uint32_t bytes = left < kTile ? static_cast<uint32_t>(left) : static_cast<uint32_t>(kTile);
+      const uint64_t id = ids[pos];
+      const uint64_t near_addr = near_base + id * block_stride + (seg ? kv_stride : 0) + off;
+      uint64_t far_addr;
+      if (paged) {
+        far_addr = far_table[pos] + far_table_off + (seg ? frag_bytes : 0) + off;
+      } else {
+        far_addr = (seg ? far_base1 : far_base0) + static_cast<uint64_t>(pos) * far_stride + off;
+      }
+      const uint64_t dst = TO_FAR ? far_addr : near_addr;
+      const uint64_t src = TO_FAR ? near_addr : far_addr;
+      if (vec_ok) {
+        copy_tile_vec<U>(dst, src, bytes);
+      } else {
+        copy_tile_any(dst, src, bytes);
+      }
     }
   }
 }
@@ -362,29 +369,22 @@ int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipSt
 int launch_block_units(const BlockUnit* units, uint32_t n_units, uint64_t max_tiles, bool to_far,
                        int unroll, uint32_t max_workgroups_x, hipStream_t s) {
   if (n_units == 0 || max_tiles == 0) return PF_OK;
-  if (n_units > 65535u) {
-    return fail(PF_ERR_INVALID_ARGUMENT, "too many units in one launch: %u", n_units);
-  }
   if (max_tiles > 0x7FFFFFFFull) {
     return fail(PF_ERR_INVALID_ARGUMENT, "unit of %llu tiles exceeds the kernel limit",
                 static_cast<unsigned long long>(max_tiles));
   }
+  // One row of workgroups for the whole launch, whatever the number of units.
   uint64_t gx = max_tiles < kMaxGridX ? max_tiles : kMaxGridX;
-  if (max_workgroups_x != 0) {
-    // The cap bounds the whole launch (all units together).
-    uint64_t per_unit = max_workgroups_x / n_units;
-    if (per_unit < 1) per_unit = 1;
-    if (gx > per_unit) gx = per_unit;
-  }
-  dim3 grid(static_cast<uint32_t>(gx), n_units, 1);
+  if (max_workgroups_x != 0 && gx > max_workgroups_x) gx = max_workgroups_x;
+  dim3 grid(static_cast<uint32_t>(gx), 1, 1);
   dim3 block(kLanes, 1, 1);
-#define PF_LAUNCH_UNITS(U_)                                                          \
-  case U_:                                                                           \
-    if (to_far) {                                                                    \
-      hipLaunchKernelGGL((block_units_kernel<U_, true>), grid, block, 0, s, units);  \
-    } else {                                                                         \
-      hipLaunchKernelGGL((block_units_kernel<U_, false>), grid, block, 0, s, units); \
-    }                                                                                \
+#define PF_LAUNCH_UNITS(U_)                                                                   \
+  case U_:                                                                                    \
+    if (to_far) {                                                                             \
+      hipLaunchKernelGGL((block_units_kernel<U_, true>), grid, block, 0, s, units, n_units);  \
+    } else {                                                                                  \
+      hipLaunchKernelGGL((block_units_kernel<U_, false>), grid, block, 0, s, units, n_units); \
+    }                                                                                         \
     break;
   switch (unroll) {
     PF_LAUNCH_UNITS(1)
@@ -459,11 +459,44 @@ int launch_block_tiles(const BlockUnit* units, uint32_t n_units, uint32_t max_bl
   return PF_OK;
 }
 
+}  // namespace pf
+
+// The two words of the stream-concurrency probe ([0] the posted word, [1] what
+// the waiter saw) live in the library's device image: a probe allocates and
+// frees nothing, so it never waits for unrelated work on the device (hipFree
+// synchronises the whole device).
+static __device__ __align__(256) uint32_t probe_words[2];
+
+namespace pf {
+
+namespace {
+constexpr int kProbeMaxDevices = 64;
+std::mutex g_probe_mu;  // one probe at a time: they share the two words
+uint32_t* g_probe_ptr[kProbeMaxDevices] = {};
+
+int probe_words_on_current_device(uint32_t** out) {
+  int device = -1;
+  PF_HIP(hipGetDevice(&device));
+  if (device < 0 || device >= kProbeMaxDevices) {
+    return fail(PF_ERR_INVALID_ARGUMENT, "device %d is beyond the %d the probe supports", device,
+                kProbeMaxDevices);
+  }
+  if (g_probe_ptr[device] == nullptr) {
+    void* ptr = nullptr;
+    PF_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(probe_words)));
+    g_probe_ptr[device] = static_cast<uint32_t*>(ptr);
+  }
+  *out = g_probe_ptr[device];
+  return PF_OK;
+}
+}  // namespace
+
 int streams_run_concurrently(hipStream_t a, hipStream_t b, bool* out) {
   *out = false;
-  uint32_t* words = nullptr;  // [0] the posted word, [1] what the waiter saw
-  PF_HIP(hipMalloc(reinterpret_cast<void**>(&words), 2 * sizeof(uint32_t)));
-  int st = PF_OK;
+  std::lock_guard<std::mutex> lock(g_probe_mu);
+  uint32_t* words = nullptr;
+  int st = probe_words_on_current_device(&words);
+  if (st != PF_OK) return st;
   uint32_t seen = 0;
   // Cleared on `a` and waited for there: no other stream of the device is touched.
   hipError_t e = hipMemsetAsync(words, 0, 2 * sizeof(uint32_t), a);
@@ -474,13 +507,13 @@ int streams_run_concurrently(hipStream_t a, hipStream_t b, bool* out) {
     hipLaunchKernelGGL(probe_post_kernel, dim3(1), dim3(64), 0, b, words);
     e = hipGetLastError();
   }
-  // Wait for both whatever was launched, so that the words can be freed.
+  // Wait for both whatever was launched: the next probe reuses the words.
   const hipError_t ea = hipStreamSynchronize(a);
   const hipError_t eb = hipStreamSynchronize(b);
   if (e == hipSuccess) e = ea != hipSuccess ? ea : eb;
-  if (e == hipSuccess) e = hipMemcpy(&seen, words + 1, sizeof(seen), hipMemcpyDeviceToHost);
+  if (e == hipSuccess) e = hipMemcpyAsync(&seen, words + 1, sizeof(seen), hipMemcpyDeviceToHost, a);
+  if (e == hipSuccess) e = hipStreamSynchronize(a);
   if (e != hipSuccess) st = fail_hip(e, "stream concurrency probe");
-  (void)hipFree(words);
   *out = seen != 0;
   return st;
 }
@@ -577,8 +610,15 @@ static __device__ __align__(256) unsigned char scratch[PF_NOALLOC_MAX_DESCS * si
 namespace {
 
 constexpr int kNoAllocMaxDevices = 64;
-// Same cap as the kernel backend: the host link wants few requesters.
-constexpr uint32_t kNoAllocWorkgroups = 64;
+// Same rule as the kernel backend: the host link wants few requesters, 16
+// workgroups when the average fragment fills a 16 KiB tile, up to 64 below.
+uint32_t noalloc_workgroups(uint64_t total_bytes, uint64_t n) {
+  constexpr uint64_t kTile = 16384;
+  const uint64_t avg = total_bytes / n ? total_bytes / n : 1;
+  if (avg >= kTile) return 16;
+  const uint64_t scaled = 16 * ((kTile + avg - 1) / avg);
+  return static_cast<uint32_t>(scaled < 64 ? scaled : 64);
+}
 
 std::mutex g_scratch_mu;
 void* g_scratch_ptr[kNoAllocMaxDevices] = {};
@@ -618,9 +658,10 @@ extern "C" int pf_desc_copy_noalloc(const pf_copy_desc* copies, uint64_t n, int 
                     "(split the batch, or use pf_backend_h2d / pf_backend_d2h)",
                     PF_NOALLOC_MAX_DESCS, static_cast<unsigned long long>(n));
   }
-  uint64_t max_size = 0;
+  uint64_t max_size = 0, total_size = 0;
   for (uint64_t i = 0; i < n; ++i) {
     const pf_copy_desc& c = copies[i];
+    total_size += c.size;
     if (c.size != 0 && (c.device == 0 || c.host_device == 0)) {
       // The kernel dereferences both addresses; a null one would fault the GPU.
       return pf::fail(PF_ERR_INVALID_ARGUMENT,
@@ -638,7 +679,7 @@ extern "C" int pf_desc_copy_noalloc(const pf_copy_desc* copies, uint64_t n, int 
   // The caller's array is the table: one copy, in stream order behind the
   // previous call's kernel on this stream.
   PF_HIP(hipMemcpyAsync(table, copies, n * sizeof(pf_copy_desc), hipMemcpyHostToDevice, stream));
-  const dim3 grid = pf::desc_copy_grid(n, max_size, kNoAllocWorkgroups), block(pf::kLanes, 1, 1);
+  const dim3 grid = pf::desc_copy_grid(n, max_size, noalloc_workgroups(total_size, n)), block(pf::kLanes, 1, 1);
   const pf_copy_desc* rows = static_cast<const pf_copy_desc*>(table);
   if (host_is_src) {
     hipLaunchKernelGGL((pf::desc48_copy_kernel<pf::kDescUnroll, true>), grid, block, 0, stream, rows,

@@ -38,10 +38,10 @@ constexpr uint32_t tile_bytes(int unroll) { return static_cast<uint32_t>(unroll)
 // Unroll factors the kernels are instantiated for.
 bool unroll_supported(int unroll);
 
-// Launch the block-ID kernel over `n_units` units (grid.y) starting at
+// Launch the zero-copy block-ID kernel over the `n_units` units starting at
 // `units` (device).  `max_tiles` is the largest tile count of any of them;
-// `max_workgroups_x` (0 = no cap) bounds the workgroups of the whole launch
-// (all units together); the kernel grid-strides.
+// `max_workgroups_x` (0 = no cap) is the number of workgroups of the launch:
+// all of them walk the units in order and stride over each unit's tiles.
 // to_far: true = gather near -> far (save), false = scatter far -> near (load).
 int launch_block_units(const BlockUnit* units, uint32_t n_units, uint64_t max_tiles, bool to_far,
                        int unroll, uint32_t max_workgroups_x, hipStream_t s);

@@ -9,11 +9,21 @@ namespace pf {
 
 // Grid cap for descriptor-copy launches whose far side is mapped host memory.
 // The host link is saturated by a few dozen workgroups; more of them only add
-// outstanding small requests on the link.  Measured on MI355X with shuffled
-// fragments (4 KiB x 65536, 16 KiB x 32768, 32 KiB x 20000), GB/s d2h / h2d:
-// uncapped 53.0/53.8, 53.8/55.4, 54.1/55.6; 64 workgroups 53.8/56.1,
-// 54.6/57.2, 54.8/57.2; 16 workgroups fall to 48/32 on the 4 KiB shape.
-constexpr uint32_t kHostLinkWorkgroups = 64;
+// outstanding small requests on the link and take compute units away from
+// whatever else runs on the device for as long as the copy lasts.  Measured on
+// MI355X with shuffled fragments (4 KiB x 65536, 16 KiB x 32768, 32 KiB x
+// 20000), GB/s d2h / h2d: uncapped 53.0/53.8, 53.8/55.4, 54.1/55.6; 64
+// workgroups 53.8/56.1, 54.6/57.2, 54.8/57.2; 16 workgroups fall to 48/32 on
+// the 4 KiB shape but hold the full rate from 16 KiB fragments on.  So: 16
+// workgroups for batches whose average fragment fills a 16 KiB tile, more for
+// smaller fragments, at most 64.
+static uint32_t host_link_workgroups(uint64_t total_bytes, uint64_t n) {
+  constexpr uint64_t kTile = 16384;
+  const uint64_t avg = n ? total_bytes / n : 0;
+  if (avg >= kTile) return 16;
+  const uint64_t scaled = 16 * ((kTile + (avg ? avg : 1) - 1) / (avg ? avg : 1));
+  return static_cast<uint32_t>(scaled < 64 ? scaled : 64);
+}
 
 // ---------------------------------------------------------------------------
 // merge
@@ -318,7 +328,7 @@ int MemcpyBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_
   const uint64_t* table_dev = static_cast<const uint64_t*>(slab->dev);
   uint64_t row = 0;
   // Rows of the isolated ranges first, then run by run.
-  uint64_t max_isolated = 0;
+  uint64_t max_isolated = 0, isolated_bytes = 0;
   if (isolated_by_kernel) {
     for (uint32_t i : isolated) {
       const Range& r = ranges[i];
@@ -326,6 +336,7 @@ int MemcpyBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_
       table[3 * row + 1] = host_is_src ? r.host_device : r.device;
       table[3 * row + 2] = r.size;
       max_isolated = std::max(max_isolated, r.size);
+      isolated_bytes += r.size;
       ++row;
     }
   }
@@ -348,7 +359,8 @@ int MemcpyBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_
                         hipMemcpyHostToDevice, s));
   row = 0;
   if (isolated_by_kernel) {
-    st = launch_desc_copy(table_dev, isolated.size(), max_isolated, s, kHostLinkWorkgroups);
+    st = launch_desc_copy(table_dev, isolated.size(), max_isolated, s,
+                          host_link_workgroups(isolated_bytes, isolated.size()));
     if (st != PF_OK) return st;
     row = isolated.size();
   }
@@ -393,9 +405,10 @@ int KernelBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_
   int st = slabs_.acquire(bytes, &slab);
   if (st != PF_OK) return st;
   uint64_t* table = static_cast<uint64_t*>(slab->host);
-  uint64_t max_size = 0;
+  uint64_t max_size = 0, total_size = 0;
   for (uint64_t i = 0; i < n; ++i) {
     const CopyDesc& c = copies[i];
+    total_size += c.size;
     if (c.size != 0 && (c.device == 0 || c.host_device == 0)) {
       // The kernel dereferences both addresses; a null one would fault the GPU.
       return fail(PF_ERR_INVALID_ARGUMENT,
@@ -409,7 +422,8 @@ int KernelBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_
     max_size = std::max<uint64_t>(max_size, c.size);
   }
   PF_HIP(hipMemcpyAsync(slab->dev, slab->host, bytes, hipMemcpyHostToDevice, s));
-  st = launch_desc_copy(static_cast<const uint64_t*>(slab->dev), n, max_size, s, kHostLinkWorkgroups);
+  st = launch_desc_copy(static_cast<const uint64_t*>(slab->dev), n, max_size, s,
+                        host_link_workgroups(total_size, n));
   if (st != PF_OK) return st;
   return slabs_.release_after(slab, s);
 }

@@ -123,10 +123,11 @@ int Xfer::timing_end(hipStream_t s) {
 }
 
 int Xfer::launch_strided(const BlockUnit* dev_units, uint32_t n_units, uint64_t max_tiles,
-                         bool to_far, hipStream_t s) {
+                         uint64_t min_frag_bytes, bool to_far, hipStream_t s) {
   int st = timing_begin(s);
   if (st != PF_OK) return st;
-  st = launch_block_units(dev_units, n_units, max_tiles, to_far, unroll_, zc_max_wg_, s);
+  st = launch_block_units(dev_units, n_units, max_tiles, to_far, unroll_,
+                          zero_copy_workgroups(min_frag_bytes), s);
   if (st != PF_OK) return st;
   return timing_end(s);
 }
@@ -808,13 +809,16 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
       // wants a completion event per layer.
       size_t uj = ui + 1;
       uint64_t max_tiles = tiles_of(units_host[ui]);
+      uint64_t min_frag = units_host[ui].frag_bytes;
       if (!want_events) {
-        while (uj < unit_refs.size() && !plans[unit_refs[uj].plan].staged && uj - ui < 65535) {
+        while (uj < unit_refs.size() && !plans[unit_refs[uj].plan].staged) {
           max_tiles = std::max(max_tiles, tiles_of(units_host[uj]));
+          min_frag = std::min(min_frag, units_host[uj].frag_bytes);
           ++uj;
         }
       }
-      st = launch_strided(units_dev + ui, static_cast<uint32_t>(uj - ui), max_tiles, save, s);
+      st = launch_strided(units_dev + ui, static_cast<uint32_t>(uj - ui), max_tiles, min_frag, save,
+                          s);
       if (st != PF_OK) return st;
       st = fire_events_through(plans[unit_refs[uj - 1].plan].src_index, s);
       if (st != PF_OK) return st;

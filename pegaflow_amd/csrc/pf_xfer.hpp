@@ -37,10 +37,24 @@ constexpr uint32_t kDefaultSlots = 2;
 constexpr uint64_t kDefaultAutoStagedMin = 64ull << 20;
 constexpr int kDefaultUnroll = 4;
 // Zero-copy launches are capped to a few workgroups: the host link, not the
-// GPU, is the bound, and fewer in-flight requests use it better.  Measured on
-// MI355X (Llama shape, 16 layers per launch): 64 workgroups load at 57.4 GB/s
-// and save at 55.0-55.8 GB/s; 2048 and more give 56.0 and 54.5 GB/s.
-constexpr uint32_t kDefaultZeroCopyWorkgroups = 64;
+// GPU, is the bound, and every workgroup that stays resident for the length of
+// the transfer takes its compute unit away from kernels that need a whole one.
+// Measured on MI355X, Llama shape (32 KiB fragments, 32 layers per launch),
+// GB/s save / load alone, then a back-to-back 4096^3 bf16 GEMM stream next to
+// the load / the save (1210 TFLOP/s alone):
+//     4 workgroups  56.6 / 45.0    772 / 776
+//     8             56.3 / 57.1    779 / 779
+//    16             56.8 / 57.3    765 / 752
+//    32             57.1 / 56.6    720 / 576
+//    64             57.1 / 57.3    557 / 405
+//   128             56.9 / 57.4    309 / 488
+// (~775 is what that GEMM runs at next to ONE resident workgroup of any kind:
+// its 256 workgroups of 512 registers per lane need every compute unit.)
+// Sixteen workgroups of full 16 KiB tiles keep 256 KiB in flight, twice the
+// link's bandwidth-delay product; fragments smaller than a tile get
+// proportionally more workgroups, up to 64.
+constexpr uint32_t kZeroCopyWorkgroupsFullTiles = 16;
+constexpr uint32_t kZeroCopyWorkgroupsMax = 64;
 
 class Xfer {
  public:
@@ -155,8 +169,16 @@ class Xfer {
   int plan_layer(const pf_layer_blocks& in, size_t index, int path, LayerPlan* out, bool* skip);
   int ensure_slot(Slot& sl, uint64_t bytes);
   // Zero-copy form: grid-stride kernel over `n_units` units, capped grid.
-  int launch_strided(const BlockUnit* dev_units, uint32_t n_units, uint64_t max_tiles, bool to_far,
-                     hipStream_t s);
+  int launch_strided(const BlockUnit* dev_units, uint32_t n_units, uint64_t max_tiles,
+                     uint64_t min_frag_bytes, bool to_far, hipStream_t s);
+  // Workgroups of a zero-copy launch whose smallest fragment is `min_frag_bytes`.
+  uint32_t zero_copy_workgroups(uint64_t min_frag_bytes) const {
+    if (zc_max_wg_ != 0) return zc_max_wg_;
+    const uint64_t tile = tile_bytes(unroll_);
+    if (min_frag_bytes == 0 || min_frag_bytes >= tile) return kZeroCopyWorkgroupsFullTiles;
+    const uint64_t scaled = kZeroCopyWorkgroupsFullTiles * ((tile + min_frag_bytes - 1) / min_frag_bytes);
+    return static_cast<uint32_t>(scaled < kZeroCopyWorkgroupsMax ? scaled : kZeroCopyWorkgroupsMax);
+  }
   // Staged form: one tile per workgroup over one unit.
   int launch_tiles(const BlockUnit* dev_unit, const BlockUnit& host_unit, bool to_far,
                    hipStream_t s);
@@ -166,7 +188,7 @@ class Xfer {
   int device_ = 0;
   uint64_t slot_bytes_ = kDefaultSlotBytes;
   uint32_t n_slots_ = kDefaultSlots;
-  uint32_t zc_max_wg_ = kDefaultZeroCopyWorkgroups;
+  uint32_t zc_max_wg_ = 0;  // 0 = by fragment size (zero_copy_workgroups)
   uint64_t auto_min_ = kDefaultAutoStagedMin;
   int unroll_ = kDefaultUnroll;
 
