@@ -548,6 +548,7 @@ typedef struct pf_engine_config {
   uint32_t ssd_enabled;              /* 512-byte host padding + CPU-readable backing */
   uint32_t use_descriptor_backends;  /* see pf_worker_pool_spawn */
   uint64_t unit_size_hint;
+  uint64_t lease_ttl_ms;             /* lease.rs:11: 0 = default (600 000 ms) */
 } pf_engine_config;
 
 typedef struct pf_layer_save {       /* LayerSave, block.rs:20-25 */
@@ -633,6 +634,76 @@ uint64_t pf_engine_inflight_blocks(pf_engine_t e);
 uint64_t pf_engine_gc_stale_inflight(pf_engine_t e, uint64_t max_age_ms);
 /* Drop every cached block that is not leased; returns how many. */
 uint64_t pf_engine_evict_all(pf_engine_t e);
+/* Query leases expire (lease.rs:11-12,47,91-118,174-181): a lease that is not
+ * consumed within lease_ttl_ms stops protecting its blocks from eviction, and
+ * a load that names it afterwards fails with "query lease is unknown or
+ * expired".  Expired leases are dropped whenever a lease is created, consumed
+ * or released, before a save gives up for lack of pinned memory, by
+ * pf_engine_gc_stale_inflight, and by this call, which stands in for the
+ * reference's 30-second sweeper task; returns how many were dropped. */
+uint64_t pf_engine_sweep_expired_leases(pf_engine_t e);
+/* Leases that have not been consumed, released or swept. */
+uint64_t pf_engine_live_leases(pf_engine_t e);
+
+/* ------------------------------------------------------------------------ */
+/* Device memory handed over by another process                              */
+/* Replaces CudaIPCWrapper (python/pegaflow/ipc_wrapper.py:102-160) and      */
+/* CudaTensorRegistry (pegaflow-server/src/registry.rs:45-203): the worker   */
+/* process exports the allocation behind each KV cache tensor, the server    */
+/* process opens it and registers the mapped address with the engine         */
+/* (pegaflow-server/src/service.rs:205-336, RegisterContextBatch).           */
+/* ------------------------------------------------------------------------ */
+
+/* What a worker sends per layer in place of the reference's pickled wrapper:
+ * IPC handle of the allocation, where the tensor's storage sits in it, and the
+ * UUID of the GPU (device ordinals differ between processes). */
+typedef struct pf_ipc_tensor {
+  uint8_t handle[64];      /* hipIpcMemHandle_t */
+  uint64_t alloc_size;     /* bytes of the exported allocation */
+  uint64_t offset;         /* storage start inside the allocation */
+  uint64_t size_bytes;     /* storage bytes (the engine's size_bytes) */
+  uint8_t device_uuid[16];
+} pf_ipc_tensor;
+
+int pf_device_uuid(int device, uint8_t out_uuid[16]);
+/* ipc_wrapper.py:75-98: ordinal of the device with this UUID in this process. */
+int pf_device_from_uuid(const uint8_t uuid[16], int* out_device);
+/* Worker side (CudaIPCWrapper.__init__): describe [dev_ptr, +size_bytes), which
+ * lies inside one device allocation of this process.  Keep an allocation that
+ * is shared this way below 2 GiB. */
+int pf_ipc_export(uint64_t dev_ptr, uint64_t size_bytes, pf_ipc_tensor* out);
+
+typedef struct pf_tensor_registry_s* pf_tensor_registry_t;
+
+int pf_registry_create(pf_tensor_registry_t* out);
+/* Closes every mapping it still holds. */
+int pf_registry_destroy(pf_tensor_registry_t r);
+/* register_layers, registry.rs:67-107: open each layer's allocation (once per
+ * allocation) on device_id and return the mapped data_ptr / size_bytes per
+ * layer.  Errors with the reference's wording: "context {key} is already
+ * registered", "layer {name} appears more than once in context {key}",
+ * "context {key} is pinned to device {a} but got {b}".  On error nothing stays
+ * mapped. */
+int pf_registry_register_layers(pf_tensor_registry_t r, const char* context_key, int device_id,
+                                uint64_t n_layers, const char* const* layer_names,
+                                const pf_ipc_tensor* tensors, uint64_t* out_data_ptrs,
+                                uint64_t* out_size_bytes);
+/* registry.rs:108-171; each returns the number of tensors released.  An
+ * instance's contexts are the keys that start with "{instance_id}:". */
+uint64_t pf_registry_drop_context(pf_tensor_registry_t r, const char* context_key);
+uint64_t pf_registry_drop_instance(pf_tensor_registry_t r, const char* instance_id);
+uint64_t pf_registry_clear(pf_tensor_registry_t r);
+uint64_t pf_registry_context_count(pf_tensor_registry_t r);
+/* The RegisterContextBatch handler (service.rs:205-336): validate, open the
+ * tensors under the context key "{instance}:tp{r}:pp{p}:dev{d}", register the
+ * mapped addresses with the engine, and roll the mappings back when the engine
+ * refuses.  layer_group_ids may be NULL. */
+int pf_server_register_context_batch(
+    pf_engine_t e, pf_tensor_registry_t r, const char* instance_id, const char* namespace_,
+    int device_id, uint64_t tp_rank, uint64_t pp_rank, uint64_t tp_size, uint64_t world_size,
+    uint64_t n_layers, const char* const* layer_names, const pf_ipc_tensor* tensors,
+    const uint64_t* num_blocks, const uint64_t* bytes_per_block, const uint64_t* kv_stride_bytes,
+    const uint64_t* segments, const uint32_t* layer_group_ids, int transfer_mode, int page_first);
 
 #ifdef __cplusplus
 } /* extern "C" */

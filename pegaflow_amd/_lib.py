@@ -119,7 +119,13 @@ class PfTaskResult(C.Structure):
 class PfEngineConfig(C.Structure):
     _fields_ = [("pool_size", u64), ("use_hugepages", u32), ("numa_aware", u32),
                 ("pool_shards", u32), ("blockwise_alloc", u32), ("ssd_enabled", u32),
-                ("use_descriptor_backends", u32), ("unit_size_hint", u64)]
+                ("use_descriptor_backends", u32), ("unit_size_hint", u64),
+                ("lease_ttl_ms", u64)]
+
+
+class PfIpcTensor(C.Structure):
+    _fields_ = [("handle", C.c_uint8 * 64), ("alloc_size", u64), ("offset", u64),
+                ("size_bytes", u64), ("device_uuid", C.c_uint8 * 16)]
 
 
 class PfLayerSave(C.Structure):
@@ -282,6 +288,24 @@ PROTOTYPES = {
     "pf_engine_inflight_blocks": (u64, [vp]),
     "pf_engine_gc_stale_inflight": (u64, [vp, u64]),
     "pf_engine_evict_all": (u64, [vp]),
+    "pf_device_uuid": (C.c_int, [C.c_int, C.POINTER(C.c_uint8)]),
+    "pf_device_from_uuid": (C.c_int, [C.POINTER(C.c_uint8), C.POINTER(C.c_int)]),
+    "pf_ipc_export": (C.c_int, [u64, u64, C.POINTER(PfIpcTensor)]),
+    "pf_registry_create": (C.c_int, [C.POINTER(vp)]),
+    "pf_registry_destroy": (C.c_int, [vp]),
+    "pf_registry_register_layers": (C.c_int, [vp, C.c_char_p, C.c_int, u64, C.POINTER(C.c_char_p),
+                                              C.POINTER(PfIpcTensor), C.POINTER(u64),
+                                              C.POINTER(u64)]),
+    "pf_registry_drop_context": (u64, [vp, C.c_char_p]),
+    "pf_registry_drop_instance": (u64, [vp, C.c_char_p]),
+    "pf_registry_clear": (u64, [vp]),
+    "pf_registry_context_count": (u64, [vp]),
+    "pf_server_register_context_batch": (C.c_int, [
+        vp, vp, C.c_char_p, C.c_char_p, C.c_int, u64, u64, u64, u64, u64, C.POINTER(C.c_char_p),
+        C.POINTER(PfIpcTensor), C.POINTER(u64), C.POINTER(u64), C.POINTER(u64), C.POINTER(u64),
+        C.POINTER(u32), C.c_int, C.c_int]),
+    "pf_engine_sweep_expired_leases": (u64, [vp]),
+    "pf_engine_live_leases": (u64, [vp]),
 }
 
 

@@ -330,11 +330,40 @@ bool Engine::evict_one() {
   return false;
 }
 
+size_t Engine::sweep_expired_locked() {
+  const auto now = std::chrono::steady_clock::now();
+  size_t gone = 0;
+  for (auto it = leases_.begin(); it != leases_.end();) {
+    if (it->second.expires_at > now) {
+      ++it;
+    } else {
+      it = leases_.erase(it);
+      ++gone;
+    }
+  }
+  return gone;
+}
+
+size_t Engine::sweep_expired_leases() {
+  std::lock_guard<std::mutex> lock(mu_);
+  return sweep_expired_locked();
+}
+
+size_t Engine::live_leases() {
+  std::lock_guard<std::mutex> lock(mu_);
+  return leases_.size();
+}
+
 std::shared_ptr<PinnedAllocation> Engine::allocate(uint64_t size, NumaNode numa) {
+  bool swept = false;
   for (;;) {
     if (auto a = pool_->allocate(size, numa)) return a;
     std::lock_guard<std::mutex> lock(mu_);
-    if (!evict_one()) return nullptr;
+    if (evict_one()) continue;
+    // Nothing evictable is left: blocks pinned by leases whose time is up
+    // (a worker that died between query and load) are given back first.
+    if (swept || sweep_expired_locked() == 0) return nullptr;
+    swept = true;
   }
 }
 
@@ -352,6 +381,7 @@ size_t Engine::inflight_blocks() {
 // pinned memory back.
 size_t Engine::gc_stale_inflight(std::chrono::milliseconds max_age) {
   std::lock_guard<std::mutex> lock(mu_);
+  sweep_expired_locked();  // the same periodic caller keeps the lease table clean
   size_t cleaned = 0;
   for (auto it = inflight_.begin(); it != inflight_.end();) {
     if (it->second.age() > max_age) {
@@ -798,9 +828,11 @@ int Engine::create_group_lease(const std::string& instance_id, uint32_t group,
     return bad(err, PF_ERR_INVALID_ARGUMENT, "query lease requires at least one block");
   }
   std::lock_guard<std::mutex> lock(mu_);
+  sweep_expired_locked();
   Lease lease;
   lease.instance_id = instance_id;
   lease.remaining_consumers = std::max<size_t>(instance->world_size(), 1);
+  lease.expires_at = lease_deadline();
   for (size_t i = 0; i < hashes.size(); ++i) {
     auto it = sealed_.find(BlockKey{instance->ns(), group_hash(hashes[i], group)});
     if (it == sealed_.end()) {
@@ -826,9 +858,11 @@ int Engine::query_prefix(const std::string& instance_id, const std::vector<std::
   auto instance = get_instance(instance_id, err);
   if (!instance) return PF_ERR_INSTANCE_MISSING;
   std::lock_guard<std::mutex> lock(mu_);
+  sweep_expired_locked();
   Lease lease;
   lease.instance_id = instance_id;
   lease.remaining_consumers = std::max<size_t>(instance->world_size(), 1);
+  lease.expires_at = lease_deadline();
   for (const std::string& h : hashes) {
     auto it = sealed_.find(BlockKey{instance->ns(), h});
     if (it == sealed_.end()) break;
@@ -846,6 +880,7 @@ int Engine::query_prefix(const std::string& instance_id, const std::vector<std::
 
 bool Engine::release_query_lease(uint64_t lease) {
   std::lock_guard<std::mutex> lock(mu_);
+  sweep_expired_locked();
   return leases_.erase(lease) > 0;
 }
 
@@ -899,6 +934,7 @@ int Engine::batch_load_kv_blocks_multi_layer(
     {
       std::lock_guard<std::mutex> lock(mu_);
       // lease.rs:105-134.
+      sweep_expired_locked();
       auto it = leases_.find(lr.lease);
       if (it == leases_.end()) {
         return bad(err, PF_ERR_STORAGE, "query lease is unknown or expired");

@@ -33,6 +33,8 @@ struct EngineConfig {
   bool ssd_enabled = false;       // pad host strides to 512 B; regular (CPU-readable) backing
   bool use_descriptor_backends = false;  // workers use per-fragment descriptors + backends
   uint64_t unit_size_hint = 0;
+  // lease.rs:11: a lease that nobody consumes stops pinning its blocks after this long.
+  uint64_t lease_ttl_ms = 600000;
 };
 
 // block.rs:20-25, as a view of the caller's arrays (valid for the call).
@@ -131,6 +133,10 @@ class Engine {
                          const std::vector<std::string>& hashes, uint64_t* out_lease,
                          std::string* err);
   bool release_query_lease(uint64_t lease);
+  // The periodic sweep of the reference's lease manager (lease.rs:66-80), for
+  // the embedder's timer: drops expired leases, returns how many.
+  size_t sweep_expired_leases();
+  size_t live_leases();
   // lib.rs:654-898.  On success *out is fulfilled when the load settles (at
   // once when nothing is to be loaded).
   int batch_load_kv_blocks_multi_layer(const std::string& instance_id, size_t tp_rank,
@@ -180,9 +186,17 @@ class Engine {
     std::string instance_id;
     std::vector<std::shared_ptr<SealedBlock>> blocks;
     size_t remaining_consumers = 1;
+    std::chrono::steady_clock::time_point expires_at;  // lease.rs:47
   };
   std::map<uint64_t, Lease> leases_;
   uint64_t next_lease_ = 1;
+  // lease.rs:91-118,174-181: drop the leases whose time is up; runs (mu_ held)
+  // whenever a lease is created, consumed or released, before an allocation
+  // gives up, and from sweep_expired_leases().  Returns how many went.
+  size_t sweep_expired_locked();
+  std::chrono::steady_clock::time_point lease_deadline() const {
+    return std::chrono::steady_clock::now() + std::chrono::milliseconds(cfg_.lease_ttl_ms);
+  }
   SaveProfile last_save_profile_;
 };
 

@@ -256,6 +256,7 @@ int pf_engine_create(const pf_engine_config* cfg, pf_engine_t* out) {
   c.ssd_enabled = cfg->ssd_enabled != 0;
   c.use_descriptor_backends = cfg->use_descriptor_backends != 0;
   c.unit_size_hint = cfg->unit_size_hint;
+  if (cfg->lease_ttl_ms != 0) c.lease_ttl_ms = cfg->lease_ttl_ms;
   std::string err;
   int status = PF_ERR_STORAGE;
   auto e = pf::Engine::create(c, &err, &status);
@@ -523,6 +524,14 @@ uint64_t pf_engine_gc_stale_inflight(pf_engine_t e, uint64_t max_age_ms) {
 
 uint64_t pf_engine_evict_all(pf_engine_t e) {
   return e ? reinterpret_cast<pf::Engine*>(e)->evict_all() : 0;
+}
+
+uint64_t pf_engine_sweep_expired_leases(pf_engine_t e) {
+  return e ? reinterpret_cast<pf::Engine*>(e)->sweep_expired_leases() : 0;
+}
+
+uint64_t pf_engine_live_leases(pf_engine_t e) {
+  return e ? reinterpret_cast<pf::Engine*>(e)->live_leases() : 0;
 }
 
 }  // extern "C"

@@ -218,11 +218,14 @@ class PegaEngine:
 
     def __init__(self, pool_size: int, use_hugepages: bool = False, numa_aware: bool = False,
                  pool_shards: int = 1, blockwise_alloc: bool = False, ssd_enabled: bool = False,
-                 use_descriptor_backends: bool = False, unit_size_hint: int = 0):
+                 use_descriptor_backends: bool = False, unit_size_hint: int = 0,
+                 lease_ttl_ms: int = 0):
+        """``lease_ttl_ms``: how long an unconsumed query lease pins its blocks
+        (0 = the reference's 600 s, lease.rs:11)."""
         self._lib = _lib.load()
         cfg = _lib.PfEngineConfig(pool_size, int(use_hugepages), int(numa_aware), pool_shards,
                                   int(blockwise_alloc), int(ssd_enabled),
-                                  int(use_descriptor_backends), unit_size_hint)
+                                  int(use_descriptor_backends), unit_size_hint, lease_ttl_ms)
         h = C.c_void_p()
         check(self._lib.pf_engine_create(C.byref(cfg), C.byref(h)))
         self.handle = h
@@ -393,6 +396,14 @@ class PegaEngine:
 
     def evict_all(self) -> int:
         return self._lib.pf_engine_evict_all(self.handle)
+
+    def sweep_expired_leases(self) -> int:
+        """Drop the query leases whose time is up (the reference's periodic
+        sweeper, lease.rs:66-80); returns how many."""
+        return self._lib.pf_engine_sweep_expired_leases(self.handle)
+
+    def live_leases(self) -> int:
+        return self._lib.pf_engine_live_leases(self.handle)
 
     def close(self) -> None:
         if self.handle is not None:

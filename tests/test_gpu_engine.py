@@ -562,6 +562,58 @@ def test_leased_blocks_survive_eviction_pressure(gpu):
     e.close()
 
 
+def test_unconsumed_lease_expires_and_frees_its_blocks(gpu):
+    """lease.rs:11,47,91-118,174-181: a lease that no worker consumes (a crashed
+    worker, a request aborted after the query) pins its blocks only until its
+    time is up.  Afterwards a save under pool pressure may evict them instead of
+    failing, and a load that still names the lease is told so."""
+    import time
+    e, layer = _one_layer_engine("inst-ttl", 4, 4096, pool_size=4 * 4096 * 2, lease_ttl_ms=800)
+    first = make_block_hashes(4, 30)
+    _save(e, "inst-ttl", first)
+    hits, lease = e.query_prefix("inst-ttl", first)
+    assert hits == 4 and e.live_leases() == 1
+    _save(e, "inst-ttl", make_block_hashes(4, 31))           # fills the pool
+    # while the lease lives, its blocks cannot go: the pool has no room for a third batch
+    # once the unleased batch is gone, and the save fails rather than touch them
+    _save(e, "inst-ttl", make_block_hashes(4, 32))           # evicts batch 31
+    assert _hits_then_release(e, "inst-ttl", first) == 4
+    hits2, lease2 = e.query_prefix("inst-ttl", make_block_hashes(4, 32))
+    assert hits2 == 4                                         # now both resident batches are leased
+    with pytest.raises(_lib.StorageError, match="exhausted|allocate"):
+        _save(e, "inst-ttl", make_block_hashes(4, 33))
+    time.sleep(1.0)                                           # both leases are past their time
+    _save(e, "inst-ttl", make_block_hashes(4, 34))           # succeeds: expired leases no longer pin
+    assert e.live_leases() == 0
+    assert _hits_then_release(e, "inst-ttl", make_block_hashes(4, 34)) == 4
+    with pytest.raises(_lib.StorageError, match="query lease is unknown or expired"):
+        e.batch_load_kv_blocks_multi_layer("inst-ttl", 0, 0, [["layer_0"]], lease, [[0, 1, 2, 3]])
+    with pytest.raises(_lib.StorageError, match="not found"):
+        e.release_query_lease(lease2)                         # swept, like an unknown one
+    e.close()
+
+
+def test_lease_consumed_in_time_loads_and_sweep_counts(gpu):
+    """A lease consumed before its time serves the load; the periodic sweep
+    (lease.rs:66-80) drops only the ones that are past it."""
+    import time
+    e, layer = _one_layer_engine("inst-ttl2", 4, 1024, pool_size=1 << 20, lease_ttl_ms=1000)
+    hashes = make_block_hashes(4, 40)
+    _save(e, "inst-ttl2", hashes)
+    _h, stale = e.query_prefix("inst-ttl2", hashes)
+    time.sleep(0.6)
+    _h, fresh = e.query_prefix("inst-ttl2", hashes)
+    assert e.sweep_expired_leases() == 0 and e.live_leases() == 2
+    time.sleep(0.6)                                           # `stale` is past its time, `fresh` is not
+    assert e.sweep_expired_leases() == 1 and e.live_leases() == 1
+    layer.zero_gpu()
+    e.batch_load_kv_blocks_multi_layer("inst-ttl2", 0, 0, [["layer_0"]], fresh, [[0, 1, 2, 3]]).wait()
+    layer.assert_gpu_matches(layer.expected)
+    with pytest.raises(_lib.StorageError, match="query lease is unknown or expired"):
+        e.batch_load_kv_blocks_multi_layer("inst-ttl2", 0, 0, [["layer_0"]], stale, [[0, 1, 2, 3]])
+    e.close()
+
+
 def test_recurrent_group_seals_final_block_save(engine):
     """hybrid_groups.rs:14-176: the recurrent group seals a tail-only checkpoint
     save, membership is per group, and one load with two leases restores the
