@@ -516,6 +516,22 @@ typedef struct pf_task_result {
 int pf_worker_pool_spawn(int device_id, int numa_node, int transfer_mode,
                          int use_descriptor_backends, pf_worker_pool_t* out);
 int pf_worker_pool_destroy(pf_worker_pool_t p);
+/* A process's streams share a few hardware queues (GPU_MAX_HW_QUEUES, 4 by
+ * default), and kernels of two streams on one queue run one after the other.
+ * A pool that is spawned probes its two streams against each other and against
+ * the idle worker streams of the pools already on the device, and swaps a
+ * stream that clashes for a fresh one, a few times at most.  This is how many
+ * clashing pairs were left for this pool (0 = its streams and every stream
+ * probed have queues of their own; with more worker streams than hardware
+ * queues some pairs must share, and the transfers of those two workers take
+ * turns).  No counterpart in the reference, which never checks. */
+uint64_t pf_worker_pool_queue_clashes(pf_worker_pool_t p);
+/* The same question for all live pools of `device`, asked now: number of worker
+ * streams, pairs among the idle ones that share a hardware queue, and streams
+ * left out because they were busy.  Probes run on the worker streams
+ * themselves: call it while the workers are idle. */
+int pf_worker_stream_report(int device, uint64_t* out_streams, uint64_t* out_clashing_pairs,
+                            uint64_t* out_skipped);
 /* submit_load, gpu_worker.rs:204-212.  The layers are copied; host memory they
  * point to must stay valid until the task settles.  load_state_shm (may be NULL)
  * names a LoadState to signal. */

@@ -254,6 +254,9 @@ PROTOTYPES = {
     "pf_worker_submit_load": (C.c_int, [vp, C.POINTER(PfLayerTransfer), u64, C.c_char_p,
                                         C.POINTER(vp)]),
     "pf_worker_submit_save": (C.c_int, [vp, C.POINTER(PfLayerTransfer), u64, C.POINTER(vp)]),
+    "pf_worker_pool_queue_clashes": (u64, [vp]),
+    "pf_worker_stream_report": (C.c_int, [C.c_int, C.POINTER(u64), C.POINTER(u64),
+                                          C.POINTER(u64)]),
     "pf_task_wait": (C.c_int, [vp, C.c_int, C.POINTER(PfTaskResult)]),
     "pf_task_destroy": (C.c_int, [vp]),
     "pf_engine_create": (C.c_int, [C.POINTER(PfEngineConfig), C.POINTER(vp)]),

@@ -173,6 +173,23 @@ int pf_worker_pool_spawn(int device_id, int numa_node, int transfer_mode,
   return PF_OK;
 }
 
+uint64_t pf_worker_pool_queue_clashes(pf_worker_pool_t p) {
+  return p ? reinterpret_cast<pf::GpuWorkerPool*>(p)->queue_clashes() : 0;
+}
+
+int pf_worker_stream_report(int device, uint64_t* out_streams, uint64_t* out_clashing_pairs,
+                            uint64_t* out_skipped) {
+  PF_REQUIRE_PTR(out_streams);
+  PF_REQUIRE_PTR(out_clashing_pairs);
+  PF_REQUIRE_PTR(out_skipped);
+  size_t streams = 0, pairs = 0, skipped = 0;
+  int st = pf::worker_stream_report(device, &streams, &pairs, &skipped);
+  *out_streams = streams;
+  *out_clashing_pairs = pairs;
+  *out_skipped = skipped;
+  return st;
+}
+
 int pf_worker_pool_destroy(pf_worker_pool_t p) {
   delete reinterpret_cast<pf::GpuWorkerPool*>(p);
   return PF_OK;

@@ -342,17 +342,56 @@ class DeviceScope {
 std::mutex g_worker_streams_mu;
 std::vector<std::pair<int, hipStream_t>> g_worker_streams;  // (device, stream) of live pools
 
+// Do kernels of `candidate` (idle by construction) and `other` run side by side?
+// `other` belongs to a live pool and may receive a task at any moment: a probe
+// that finds it busy, or that reports a clash once but not twice, says nothing.
+bool clash_with(hipStream_t candidate, hipStream_t other) {
+  for (int attempt = 0; attempt < 2; ++attempt) {
+    if (hipStreamQuery(other) != hipSuccess) {
+      (void)hipGetLastError();
+      return false;  // busy: the posting kernel would queue behind its work
+    }
+    bool concurrent = true;
+    // The waiting kernel goes on the candidate.
+    if (streams_run_concurrently(candidate, other, &concurrent) != PF_OK) return false;
+    if (concurrent) return false;
+  }
+  return true;
+}
+
 size_t clashes(hipStream_t candidate, const std::vector<hipStream_t>& others) {
   size_t n = 0;
-  for (hipStream_t other : others) {
-    bool concurrent = true;
-    // The waiting kernel goes on the candidate, which is idle by construction.
-    if (streams_run_concurrently(candidate, other, &concurrent) != PF_OK) return 0;
-    n += concurrent ? 0 : 1;
-  }
+  for (hipStream_t other : others) n += clash_with(candidate, other) ? 1 : 0;
   return n;
 }
 }  // namespace
+
+int worker_stream_report(int device, size_t* out_streams, size_t* out_clashing_pairs,
+                         size_t* out_skipped) {
+  DeviceScope scope(device);
+  if (!scope.ok()) return fail(PF_ERR_DEVICE_INIT, "cannot select device %d", device);
+  std::lock_guard<std::mutex> registry(g_worker_streams_mu);
+  std::vector<hipStream_t> idle;
+  size_t skipped = 0, total = 0;
+  for (const auto& entry : g_worker_streams) {
+    if (entry.first != device) continue;
+    ++total;
+    if (hipStreamQuery(entry.second) == hipSuccess) {
+      idle.push_back(entry.second);
+    } else {
+      ++skipped;
+    }
+  }
+  (void)hipGetLastError();
+  size_t pairs = 0;
+  for (size_t i = 0; i < idle.size(); ++i) {
+    for (size_t j = i + 1; j < idle.size(); ++j) pairs += clash_with(idle[i], idle[j]) ? 1 : 0;
+  }
+  *out_streams = total;
+  *out_clashing_pairs = pairs;
+  *out_skipped = skipped;
+  return PF_OK;
+}
 
 void GpuWorkerPool::separate_worker_queues() {
   DeviceScope device(device_id_);
@@ -387,6 +426,7 @@ void GpuWorkerPool::separate_worker_queues() {
       std::lock_guard<std::mutex> lock(w->mu);
       w->stream = best;
     }
+    queue_clashes_ += best_clashes;
     others.push_back(best);
   }
   for (hipStream_t s : rejected) (void)hipStreamDestroy(s);
@@ -408,13 +448,11 @@ void GpuWorkerPool::prime_copy_overlap() {
   DeviceScope device(device_id_);
   if (!device.ok()) return;
   const size_t chunk = 32u << 20;
-  void* host = nullptr;
-  void* dev = nullptr;
-  if (hipHostMalloc(&host, 2 * chunk, hipHostMallocMapped) == hipSuccess &&
-      hipMalloc(&dev, 2 * chunk) == hipSuccess) {
-    std::memset(host, 0, 2 * chunk);
-    uint8_t* h = static_cast<uint8_t*>(host);
-    uint8_t* d = static_cast<uint8_t*>(dev);
+  if (hipHostMalloc(&prime_host_, 2 * chunk, hipHostMallocMapped) == hipSuccess &&
+      hipMalloc(&prime_dev_, 2 * chunk) == hipSuccess) {
+    std::memset(prime_host_, 0, 2 * chunk);
+    uint8_t* h = static_cast<uint8_t*>(prime_host_);
+    uint8_t* d = static_cast<uint8_t*>(prime_dev_);
     for (int i = 0; i < 6; ++i) {
       (void)hipMemcpyAsync(h, d, chunk, hipMemcpyDeviceToHost, save_.stream);
     }
@@ -424,8 +462,6 @@ void GpuWorkerPool::prime_copy_overlap() {
     (void)hipStreamSynchronize(save_.stream);
     (void)hipStreamSynchronize(load_.stream);
   }
-  if (dev) (void)hipFree(dev);
-  if (host) (void)hipHostFree(host);
   (void)hipGetLastError();
 }
 
@@ -445,6 +481,12 @@ GpuWorkerPool::~GpuWorkerPool() {
     }
     w->cv.notify_all();
     if (w->thread.joinable()) w->thread.join();
+  }
+  if (prime_dev_ || prime_host_) {
+    DeviceScope device(device_id_);
+    if (prime_dev_) (void)hipFree(prime_dev_);
+    if (prime_host_) (void)hipHostFree(prime_host_);
+    (void)hipGetLastError();
   }
 }
 

@@ -104,6 +104,11 @@ class GpuWorkerPool {
   // gpu_worker.rs:216-243.
   std::future<TaskResult> batch_save(std::vector<LayerTransferData> layers);
   int device_id() const { return device_id_; }
+  // Pairs among {this pool's two streams, the idle worker streams of the other
+  // pools on the device that were probed} whose kernels did NOT run side by
+  // side when the pool was spawned: 0 = every worker stream probed has a
+  // hardware queue of its own.
+  size_t queue_clashes() const { return queue_clashes_; }
 
  private:
   struct Task {
@@ -132,7 +137,19 @@ class GpuWorkerPool {
   bool use_descriptors_ = false;
   Worker load_;
   Worker save_;
+  size_t queue_clashes_ = 0;
+  // Buffers of prime_copy_overlap, kept until the pool goes: freeing device or
+  // pinned memory synchronises the whole device, and a pool is spawned while
+  // other instances transfer.
+  void* prime_host_ = nullptr;
+  void* prime_dev_ = nullptr;
 };
+
+// Worker streams of the live pools on `device` and how many pairs of them share
+// a hardware queue right now (kernels of the two do not overlap).  Streams that
+// are busy are left out of the probe and counted in *out_skipped.
+int worker_stream_report(int device, size_t* out_streams, size_t* out_clashing_pairs,
+                         size_t* out_skipped);
 
 // gpu_worker.rs:353-423 over the C++ types (the C-ABI form is pf_build_copy_descs).
 // Layers [begin, end) only when end > begin; the whole task otherwise.

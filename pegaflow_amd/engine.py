@@ -129,6 +129,12 @@ class GpuWorkerPool:
                                              1 if use_descriptor_backends else 0, C.byref(h)))
         self.handle = h
 
+    @property
+    def queue_clashes(self) -> int:
+        """Pairs of worker streams (this pool's two and the idle ones of the
+        other pools probed at spawn) that were left sharing a hardware queue."""
+        return self._lib.pf_worker_pool_queue_clashes(self.handle)
+
     def submit_load(self, layers: Sequence[LayerTransferData],
                     load_state: LoadState | None = None) -> Task:
         arr, n, keep = _pack_layer_transfers(layers)
@@ -153,6 +159,14 @@ class GpuWorkerPool:
             self.close()
         except Exception:
             pass
+
+
+def worker_stream_report(device: int = 0) -> tuple[int, int, int]:
+    """(worker streams of the live pools on ``device``, pairs among the idle
+    ones that share a hardware queue right now, streams skipped because busy)."""
+    a, b, c = C.c_uint64(), C.c_uint64(), C.c_uint64()
+    check(_lib.load().pf_worker_stream_report(device, C.byref(a), C.byref(b), C.byref(c)))
+    return a.value, b.value, c.value
 
 
 @dataclass
