@@ -209,7 +209,16 @@ int pf_backend_create(int mode, pf_backend_t* out);
 int pf_backend_destroy(pf_backend_t b);
 /* TransferBackend::name: "direct" or "kernel". */
 const char* pf_backend_name(pf_backend_t b);
-/* TransferBackend::h2d / d2h.  Enqueue only. */
+/* TransferBackend::h2d / d2h.  Enqueue only.
+ * Two things differ from the reference's MemcpyBackend, which issues one
+ * stream-ordered copy per merged range in list order (memcpy.rs:57-102):
+ *  - the "direct" backend reorders a batch (large ranges first, then isolated
+ *    small ones, then packed runs), so a batch must not contain ranges whose
+ *    DESTINATIONS overlap: which writer wins is not the list order;
+ *  - a backend keeps internal staging shared by its batches.  Batches on one
+ *    stream are ordered by the stream; a batch submitted on another stream
+ *    waits (on the device) for the previous batch's use of the staging
+ *    buffer.  A handle still belongs to one thread at a time. */
 int pf_backend_h2d(pf_backend_t b, const pf_copy_desc* copies, uint64_t n, pf_stream_t s);
 int pf_backend_d2h(pf_backend_t b, const pf_copy_desc* copies, uint64_t n, pf_stream_t s);
 /* The copy of PF_MODE_KERNEL for callers that cannot allocate: code under HIP

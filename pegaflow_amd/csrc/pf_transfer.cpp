@@ -165,6 +165,10 @@ int SlabPool::release_after(Slab* slab, hipStream_t s) {
 // ---------------------------------------------------------------------------
 
 MemcpyBackend::~MemcpyBackend() {
+  if (staging_done_) {
+    if (staging_used_) (void)hipEventSynchronize(staging_done_);
+    (void)hipEventDestroy(staging_done_);
+  }
   if (staging_) (void)hipFree(staging_);
   (void)hipGetLastError();
 }
@@ -307,18 +311,30 @@ int MemcpyBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_
                 static_cast<unsigned long long>(table_rows));
   }
 
-  if (staged_pieces != 0 && staging_cap_ < max_run_bytes) {
-    // Grow-only; the stream order of the previous batch protects the old buffer.
-    if (staging_) {
-      PF_HIP(hipStreamSynchronize(s));
-      PF_HIP(hipFree(staging_));
-      staging_ = nullptr;
-      staging_cap_ = 0;
+  if (staged_pieces != 0) {
+    if (staging_done_ == nullptr) {
+      PF_HIP(hipEventCreateWithFlags(&staging_done_, hipEventDisableTiming));
     }
-    uint64_t cap = 1ull << 20;
-    while (cap < max_run_bytes) cap <<= 1;
-    PF_HIP(hipMalloc(&staging_, cap));
-    staging_cap_ = cap;
+    if (staging_cap_ < max_run_bytes) {
+      // Grow-only; the last batch that used the old buffer must be through with it,
+      // whichever stream it ran on.
+      if (staging_) {
+        if (staging_used_) PF_HIP(hipEventSynchronize(staging_done_));
+        PF_HIP(hipFree(staging_));
+        staging_ = nullptr;
+        staging_cap_ = 0;
+        staging_used_ = false;
+      }
+      uint64_t cap = 1ull << 20;
+      while (cap < max_run_bytes) cap <<= 1;
+      PF_HIP(hipMalloc(&staging_, cap));
+      staging_cap_ = cap;
+    }
+    // A batch on another stream than the previous one is not ordered behind it
+    // by the stream: make it wait until the buffer is free.
+    if (staging_used_ && staging_stream_ != s) {
+      PF_HIP(hipStreamWaitEvent(s, staging_done_, 0));
+    }
   }
 
   SlabPool::Slab* slab = nullptr;
@@ -381,6 +397,11 @@ int MemcpyBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_
                                 run.bytes, s));
     }
     row += run.members.size();
+  }
+  if (staged_pieces != 0) {
+    PF_HIP(hipEventRecord(staging_done_, s));
+    staging_stream_ = s;
+    staging_used_ = true;
   }
   return slabs_.release_after(slab, s);
 }

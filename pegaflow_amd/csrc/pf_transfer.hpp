@@ -88,8 +88,14 @@ class MemcpyBackend : public TransferBackend {
   int submit(const CopyDesc* copies, uint64_t n, bool host_is_src, hipStream_t s);
   int submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_src, hipStream_t s);
   SlabPool slabs_;
+  // One staging buffer serves every batch.  Batches on one stream are ordered
+  // by the stream; a batch on another stream first waits for `staging_done_`,
+  // recorded behind the last batch that used the buffer.
   void* staging_ = nullptr;
   uint64_t staging_cap_ = 0;
+  hipEvent_t staging_done_ = nullptr;
+  hipStream_t staging_stream_ = nullptr;  // stream of the last batch that used staging_
+  bool staging_used_ = false;
 };
 
 // transfer/kernel.rs:51-151: one kernel launch for the whole batch, host side

@@ -193,6 +193,52 @@ def test_two_batches_without_sync_between(backends, stream):
     host.close()
 
 
+def test_direct_backend_batches_on_two_streams_share_its_staging(gpu):
+    """Two host-dense batches through ONE direct backend on two different
+    streams with no synchronise between them: both are packed through the
+    backend's one staging buffer, so the second has to wait (on the device) for
+    the first one's use of it."""
+    from pegaflow_amd.transfer import desc_array
+    rng = np.random.default_rng(21)
+    seg, n = 4096, 6000
+    data = random_bytes(rng, 2 * n * seg)
+    host = PinnedMemory(2 * n * seg)
+    dev = DeviceBuffer(2 * n * seg)
+    s1, s2 = Stream(), Stream()
+    b = MemcpyBackend()
+    perm1 = rng.permutation(n).astype(np.uint64)
+    perm2 = rng.permutation(n).astype(np.uint64) + n
+    pos = np.arange(n, dtype=np.uint64)
+    first = desc_array(dev.ptr + perm1 * seg, host.host_ptr + pos * seg, host.device_ptr + pos * seg,
+                       seg, 0, 1)
+    second = desc_array(dev.ptr + perm2 * seg, host.host_ptr + (n + pos) * seg,
+                        host.device_ptr + (n + pos) * seg, seg, 0, 1)
+    try:
+        for _ in range(3):
+            host.as_numpy()[:] = data
+            dev.fill(0)
+            b.h2d(first, s1)
+            b.h2d(second, s2)
+            s1.synchronize()
+            s2.synchronize()
+            got = dev.copy_to_host().reshape(2 * n, seg)
+            want = data.reshape(2 * n, seg)
+            assert np.array_equal(got[perm1.astype(np.int64)], want[:n])
+            assert np.array_equal(got[perm2.astype(np.int64)], want[n:])
+            host.as_numpy()[:] = 0
+            b.d2h(first, s2)
+            b.d2h(second, s1)
+            s1.synchronize()
+            s2.synchronize()
+            assert np.array_equal(host.as_numpy(), data)
+    finally:
+        b.close()
+        s1.close()
+        s2.close()
+        dev.close()
+        host.close()
+
+
 def _run_both_directions(backend, stream, descs_fn, dev_bytes, host_bytes, rows, seed):
     """rows: (device offset, host offset, size).  Checks h2d and d2h of one
     backend against the oracle, including the bytes outside the fragments."""
