@@ -30,6 +30,8 @@ struct BlockUnit {
   uint32_t n_seg;             // fragments per block: 1 or 2
   uint32_t tiles_per_frag;    // ceil(frag_bytes / tile_bytes)
   uint32_t vec_ok;            // every address and stride is 16-byte aligned
+  uint32_t ids16;             // the id list holds 16-bit ids (zero-copy form only)
+  uint32_t reserved;
 };
 
 // Bytes one workgroup moves per tile for the given unroll (256 lanes x 16 B x U).
@@ -45,6 +47,18 @@ bool unroll_supported(int unroll);
 // to_far: true = gather near -> far (save), false = scatter far -> near (load).
 int launch_block_units(const BlockUnit* units, uint32_t n_units, uint64_t max_tiles, bool to_far,
                        int unroll, uint32_t max_workgroups_x, hipStream_t s);
+
+// A slab small enough to travel in the arguments of a launch (the limit for all
+// arguments of a kernel is 4 KiB): units first, then id lists and page tables,
+// with the units' `ids` / `far_table` holding byte offsets into the slab.
+constexpr uint32_t kArgSlabBytes = 3840;
+struct ArgSlab {
+  uint64_t words[kArgSlabBytes / 8];
+};
+// Units [first_unit, first_unit + n_units) of the slab.
+int launch_block_units_args(const ArgSlab& slab, uint32_t first_unit, uint32_t n_units,
+                            uint64_t max_tiles, bool to_far, int unroll, uint32_t max_workgroups_x,
+                            hipStream_t s);
 
 // Limits of one block_tiles launch (grid.y and grid.z are 16-bit).
 constexpr uint32_t kMaxTileBlocks = 65535;

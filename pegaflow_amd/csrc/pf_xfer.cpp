@@ -132,6 +132,17 @@ int Xfer::launch_strided(const BlockUnit* dev_units, uint32_t n_units, uint64_t 
   return timing_end(s);
 }
 
+int Xfer::launch_strided_args(const ArgSlab& slab, uint32_t first_unit, uint32_t n_units,
+                              uint64_t max_tiles, uint64_t min_frag_bytes, bool to_far,
+                              hipStream_t s) {
+  int st = timing_begin(s);
+  if (st != PF_OK) return st;
+  st = launch_block_units_args(slab, first_unit, n_units, max_tiles, to_far, unroll_,
+                               zero_copy_workgroups(min_frag_bytes), s);
+  if (st != PF_OK) return st;
+  return timing_end(s);
+}
+
 int Xfer::launch_tiles(const BlockUnit* dev_unit, const BlockUnit& host_unit, bool to_far,
                        hipStream_t s) {
   int st = timing_begin(s);
@@ -623,60 +634,84 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
       max_unit_bytes = std::max(max_unit_bytes, count * block_bytes);
     }
   }
-  uint64_t slab_bytes = unit_refs.size() * sizeof(BlockUnit);
-  slab_bytes = (slab_bytes + 255) & ~255ull;
   // The visiting orders of staged loads sit behind everything else in the slab
   // and are uploaded on their own, after the first link copy is under way:
   // `order_slab_off` is relative to that tail until the head's size is known.
-  uint64_t order_bytes = 0;
-  for (size_t pi = 0; pi < plans.size(); ++pi) {
-    LayerPlan& p = plans[pi];
-    // Layers that pass the very same id array share one upload.
-    bool shared = false;
-    for (size_t pj = 0; pj < pi; ++pj) {
-      if (plans[pj].n_blocks == p.n_blocks &&
-          (plans[pj].ids == p.ids ||
-           std::memcmp(plans[pj].ids, p.ids, p.n_blocks * sizeof(uint32_t)) == 0)) {
-        p.ids_slab_off = plans[pj].ids_slab_off;
-        shared = true;
-        break;
-      }
+  uint64_t slab_bytes = 0, order_bytes = 0;
+  bool all_zero_copy = true;
+  uint32_t max_id = 0;
+  for (const LayerPlan& p : plans) {
+    all_zero_copy = all_zero_copy && !p.staged;
+    if (all_zero_copy) {
+      for (uint64_t i = 0; i < p.n_blocks; ++i) max_id = std::max(max_id, p.ids[i]);
     }
-    if (!shared) {
-      p.ids_slab_off = slab_bytes;
-      slab_bytes += (p.n_blocks * sizeof(uint32_t) + 255) & ~255ull;
-    }
-    // Staged loads visit each unit's positions in ascending destination id
-    // (launch_block_tiles); layers with the same ids and unit size share it.
-    if (!save && p.staged && p.n_blocks > 1) {
-      p.ordered = true;
+  }
+  auto lay_out = [&](uint64_t id_bytes) {
+    slab_bytes = unit_refs.size() * sizeof(BlockUnit);
+    slab_bytes = (slab_bytes + 255) & ~255ull;
+    order_bytes = 0;
+    for (size_t pi = 0; pi < plans.size(); ++pi) {
+      LayerPlan& p = plans[pi];
+      p.ordered = p.order_owner = p.order_shared = false;
+      // Layers that pass the very same id array share one upload.
+      bool shared = false;
       for (size_t pj = 0; pj < pi; ++pj) {
-        if (plans[pj].ordered && plans[pj].ids_slab_off == p.ids_slab_off &&
-            plans[pj].per_unit == p.per_unit) {
-          p.order_slab_off = plans[pj].order_slab_off;
-          p.order_shared = true;
+        if (plans[pj].n_blocks == p.n_blocks &&
+            (plans[pj].ids == p.ids ||
+             std::memcmp(plans[pj].ids, p.ids, p.n_blocks * sizeof(uint32_t)) == 0)) {
+          p.ids_slab_off = plans[pj].ids_slab_off;
+          shared = true;
           break;
         }
       }
-      if (!p.order_shared) {
-        p.order_owner = true;
-        p.order_slab_off = order_bytes;
-        order_bytes += (p.n_blocks * sizeof(uint32_t) + 255) & ~255ull;
+      if (!shared) {
+        p.ids_slab_off = slab_bytes;
+        slab_bytes += (p.n_blocks * id_bytes + 255) & ~255ull;
       }
-    }
-    if (p.page_dev) {
-      bool tshared = false;
-      for (size_t pj = 0; pj < pi; ++pj) {
-        if (plans[pj].page_dev == p.page_dev && plans[pj].n_blocks == p.n_blocks) {
-          p.table_slab_off = plans[pj].table_slab_off;
-          tshared = true;
-          break;
+      // Staged loads visit each unit's positions in ascending destination id
+      // (launch_block_tiles); layers with the same ids and unit size share it.
+      if (!save && p.staged && p.n_blocks > 1) {
+        p.ordered = true;
+        for (size_t pj = 0; pj < pi; ++pj) {
+          if (plans[pj].ordered && plans[pj].ids_slab_off == p.ids_slab_off &&
+              plans[pj].per_unit == p.per_unit) {
+            p.order_slab_off = plans[pj].order_slab_off;
+            p.order_shared = true;
+            break;
+          }
+        }
+        if (!p.order_shared) {
+          p.order_owner = true;
+          p.order_slab_off = order_bytes;
+          order_bytes += (p.n_blocks * sizeof(uint32_t) + 255) & ~255ull;
         }
       }
-      if (!tshared) {
-        p.table_slab_off = slab_bytes;
-        slab_bytes += (p.n_blocks * sizeof(uint64_t) + 255) & ~255ull;
+      if (p.page_dev) {
+        bool tshared = false;
+        for (size_t pj = 0; pj < pi; ++pj) {
+          if (plans[pj].page_dev == p.page_dev && plans[pj].n_blocks == p.n_blocks) {
+            p.table_slab_off = plans[pj].table_slab_off;
+            tshared = true;
+            break;
+          }
+        }
+        if (!tshared) {
+          p.table_slab_off = slab_bytes;
+          slab_bytes += (p.n_blocks * sizeof(uint64_t) + 255) & ~255ull;
+        }
       }
+    }
+  };
+  lay_out(sizeof(uint32_t));
+  // Short lists of zero-copy layers travel in the launch's arguments (below);
+  // ids below 65536 are halved in size when that is what makes them fit.
+  bool ids16 = false;
+  if (all_zero_copy && slab_bytes > kArgSlabBytes && max_id < 65536u) {
+    lay_out(sizeof(uint16_t));
+    if (slab_bytes <= kArgSlabBytes) {
+      ids16 = true;
+    } else {
+      lay_out(sizeof(uint32_t));
     }
   }
   const uint64_t head_bytes = slab_bytes;
@@ -684,14 +719,30 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
   for (LayerPlan& p : plans) {
     if (p.ordered) p.order_slab_off += head_bytes;
   }
+  // A call of zero-copy layers whose units, id lists and page tables fit the
+  // argument segment of a launch carries them there: nothing to upload first.
+  bool in_args = slab_bytes <= kArgSlabBytes;
+  for (const LayerPlan& p : plans) in_args = in_args && !p.staged;
+  ArgSlab arg_slab;
   SlabPool::Slab* slab = nullptr;
-  int st = slabs_.acquire(slab_bytes, &slab);
-  if (st != PF_OK) return st;
-  uint8_t* slab_host = static_cast<uint8_t*>(slab->host);
-  const uint64_t slab_dev = reinterpret_cast<uint64_t>(slab->dev);
+  int st = PF_OK;
+  if (!in_args) {
+    st = slabs_.acquire(slab_bytes, &slab);
+    if (st != PF_OK) return st;
+  }
+  uint8_t* slab_host = in_args ? reinterpret_cast<uint8_t*>(&arg_slab) : static_cast<uint8_t*>(slab->host);
+  // In the argument form the units carry offsets into the slab, not addresses.
+  const uint64_t slab_dev = in_args ? 0 : reinterpret_cast<uint64_t>(slab->dev);
   for (size_t pi = 0; pi < plans.size(); ++pi) {
     LayerPlan& p = plans[pi];
-    std::memcpy(slab_host + p.ids_slab_off, p.ids, p.n_blocks * sizeof(uint32_t));
+    if (ids16) {
+      uint16_t* narrow = reinterpret_cast<uint16_t*>(slab_host + p.ids_slab_off);
+      for (uint64_t i = 0; i < p.n_blocks; ++i) narrow[i] = static_cast<uint16_t>(p.ids[i]);
+      // the kernel reads whole words: the odd half of the last one must be readable
+      if (p.n_blocks & 1) narrow[p.n_blocks] = 0;
+    } else {
+      std::memcpy(slab_host + p.ids_slab_off, p.ids, p.n_blocks * sizeof(uint32_t));
+    }
     if (p.page_dev) {
       std::memcpy(slab_host + p.table_slab_off, p.page_dev, p.n_blocks * sizeof(uint64_t));
     }
@@ -717,7 +768,9 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     u.block_stride = p.layout.block_stride_bytes();
     u.kv_stride = p.layout.kv_stride_bytes();
     u.frag_bytes = p.frag_bytes;
-    u.ids = reinterpret_cast<const uint32_t*>(slab_dev + p.ids_slab_off) + r.first;
+    // Zero-copy units start at list position 0, so a 16-bit list starts on a word.
+    u.ids = reinterpret_cast<const uint32_t*>(slab_dev + p.ids_slab_off) + (ids16 ? 0 : r.first);
+    u.ids16 = ids16 ? 1 : 0;
     if (p.ordered) {
       u.order = reinterpret_cast<const uint32_t*>(slab_dev + p.order_slab_off) + r.first;
     }
@@ -759,7 +812,9 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     if (side_status != PF_OK) return side_status;
   }
   began_ = true;
-  PF_HIP(hipMemcpyAsync(slab->dev, slab->host, head_bytes, hipMemcpyHostToDevice, s));
+  if (!in_args) {
+    PF_HIP(hipMemcpyAsync(slab->dev, slab->host, head_bytes, hipMemcpyHostToDevice, s));
+  }
   // Sorting the ids of a long list takes the submitting thread about a
   // millisecond per 64 Ki ids: do it while the first unit's link copy runs.
   bool orders_pending = order_bytes != 0;
@@ -817,8 +872,13 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
           ++uj;
         }
       }
-      st = launch_strided(units_dev + ui, static_cast<uint32_t>(uj - ui), max_tiles, min_frag, save,
-                          s);
+      if (in_args) {
+        st = launch_strided_args(arg_slab, static_cast<uint32_t>(ui), static_cast<uint32_t>(uj - ui),
+                                 max_tiles, min_frag, save, s);
+      } else {
+        st = launch_strided(units_dev + ui, static_cast<uint32_t>(uj - ui), max_tiles, min_frag,
+                            save, s);
+      }
       if (st != PF_OK) return st;
       st = fire_events_through(plans[unit_refs[uj - 1].plan].src_index, s);
       if (st != PF_OK) return st;
@@ -884,7 +944,7 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     st = fire_events_through(n_layers - 1, s);
     if (st != PF_OK) return st;
   }
-  return slabs_.release_after(slab, s);
+  return in_args ? PF_OK : slabs_.release_after(slab, s);
 }
 
 }  // namespace pf

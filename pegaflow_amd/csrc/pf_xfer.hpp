@@ -179,6 +179,9 @@ class Xfer {
     const uint64_t scaled = kZeroCopyWorkgroupsFullTiles * ((tile + min_frag_bytes - 1) / min_frag_bytes);
     return static_cast<uint32_t>(scaled < kZeroCopyWorkgroupsMax ? scaled : kZeroCopyWorkgroupsMax);
   }
+  // The same with the slab in the launch's arguments (short lists).
+  int launch_strided_args(const ArgSlab& slab, uint32_t first_unit, uint32_t n_units,
+                          uint64_t max_tiles, uint64_t min_frag_bytes, bool to_far, hipStream_t s);
   // Staged form: one tile per workgroup over one unit.
   int launch_tiles(const BlockUnit* dev_unit, const BlockUnit& host_unit, bool to_far,
                    hipStream_t s);

@@ -147,6 +147,14 @@ LAYOUTS = {
     "misaligned_base": dict(num_blocks=50, seg=4096, segments=2, base_off=4),
     # more list positions than one tile launch can index (65535): the staged path splits units
     "many_tiny_64": dict(num_blocks=70000, seg=64, segments=1, n_ids=70000),
+    # zero-copy lists short enough to travel in the launch's arguments: as 32-bit ids
+    # (850 fill the argument slab to the last byte), as 16-bit ids (an odd count, so
+    # the last word is half used), and too long or too large for either form
+    "args_ids32_850": dict(num_blocks=4096, seg=2048, segments=2, n_ids=850),
+    "args_ids16_1001": dict(num_blocks=4096, seg=2048, segments=2, n_ids=1001),
+    "args_ids16_1791": dict(num_blocks=4096, seg=1024, segments=1, n_ids=1791),
+    "slab_ids16_too_many_1800": dict(num_blocks=4096, seg=1024, segments=1, n_ids=1800),
+    "slab_ids_over_65535": dict(num_blocks=70000, seg=256, segments=1, n_ids=1001),
 }
 
 

@@ -1,7 +1,8 @@
 """The C ABI from native programs, built with the library (make -C
 pegaflow_amd/csrc): tests/native/engine_roundtrip.cpp runs the save -> query ->
 load cycle in C++ against libpegahip.so; tests/native/engine_threads.cpp drives
-one engine from several threads under pool pressure.  Both check every byte
+one engine from several threads under pool pressure; tests/native/
+small_transfers.cpp times and checks small transfers.  All check every byte
 themselves."""
 
 import os
@@ -11,7 +12,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 BINARIES = {name: os.path.join(ROOT, "tests", "native", name)
-            for name in ("engine_roundtrip", "engine_threads")}
+            for name in ("engine_roundtrip", "engine_threads", "small_transfers")}
 
 
 @pytest.mark.parametrize("name", sorted(BINARIES))
@@ -40,3 +41,16 @@ def test_engine_shared_by_threads_under_pool_pressure():
     fields = dict(item.split("=") for item in summary.split())
     # loads really happened (how many queries miss depends on thread timing)
     assert int(fields["loaded"]) > 1000, summary
+
+
+@pytest.mark.gpu
+def test_small_transfers_from_cpp():
+    """tests/native/small_transfers.cpp: every small case moves the right bytes;
+    the timings it prints are reported by bench.py --workload ref_transfer_bench."""
+    import json
+    out = _run("small_transfers")
+    rows = json.loads([ln for ln in out.splitlines() if ln.startswith("{")][-1])["rows"]
+    cases = {r["case"] for r in rows}
+    assert {"block_ids_save_4MiB", "block_ids_load_4MiB", "kernel_backend_d2h_1024x4KiB",
+            "noalloc_h2d_1024x4KiB"} <= cases
+    assert all(r["us"] > 0 for r in rows)
