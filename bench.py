@@ -106,8 +106,10 @@ def parse_args():
     ap.add_argument("--no-overlap", action="store_true", help="skip the GEMM-overlap section")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-engine", action="store_true", help="skip the save/query/load engine section")
-    ap.add_argument("--engine-mode", choices=["direct", "kernel"], default="direct",
-                    help="transfer mode the engine section registers its instances with")
+    ap.add_argument("--engine-mode", choices=["direct", "kernel", "zerocopy"], default="direct",
+                    help="transfer mode the engine section registers its instances with "
+                         "(zerocopy = PF_MODE_ZEROCOPY: the block-ID engine pinned to the "
+                         "zero-copy kernel)")
     ap.add_argument("--engine-descriptors", action="store_true",
                     help="engine section: the workers build one descriptor per fragment and call "
                          "the descriptor backends, as the reference's workers do")
@@ -488,7 +490,9 @@ def main():
             return json.loads(lines[-1])
         engine = engine_run(args.engine_mode)
         # the other transfer mode, for comparison (instances choose one at registration)
-        other = "kernel" if args.engine_mode == "direct" else "direct"
+        # the zero-copy worker mode, for comparison (instances choose a mode at registration;
+        # "direct" and "kernel" both let the engine pick the path per call)
+        other = "zerocopy" if args.engine_mode != "zerocopy" else "direct"
         engine["other_mode"] = engine_run(other)
 
     # ---- CPU baseline: the oracle's memcpy executor on the host cores -----
@@ -637,31 +641,35 @@ def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_
 
     ticks = []   # (GEMMs launched so far, event on the GEMM stream), one per 64 GEMMs
 
-    def gemms(count, tick_pool=None):
+    def gemms(count, tick_pool=None, until=None):
+        """Launch `count` GEMMs; with `until` (an event on another stream), keep
+        launching in groups of 64 after that until the event has completed, so
+        that the GEMM stream stays busy for as long as that work takes.
+        Returns the number launched."""
         del ticks[:]
+        launched = 0
         with torch.cuda.stream(gemm_stream):
             g0.record()
-            for i in range(count):
-                torch.matmul(a, b, out=c)
-                if tick_pool is not None and i % 64 == 63 and i // 64 < len(tick_pool):
-                    tick_pool[i // 64].record(gemm_native)
-                    ticks.append((i + 1, tick_pool[i // 64]))
+            while True:
+                for _ in range(count if launched == 0 else 64):
+                    torch.matmul(a, b, out=c)
+                    launched += 1
+                    if tick_pool is not None and launched % 64 == 0 and launched // 64 <= len(tick_pool):
+                        tick_pool[launched // 64 - 1].record(gemm_native)
+                        ticks.append((launched, tick_pool[launched // 64 - 1]))
+                if until is None or until.query() or launched > 60000:
+                    break
             g1.record()
+        return launched
 
     gemms(50)
     torch.cuda.synchronize()
-    host0 = time.perf_counter()
     gemms(200)
-    enqueue_ms = (time.perf_counter() - host0) * 1e3 / 200     # host time per launch
     torch.cuda.synchronize()
     gemm_alone_ms = g0.elapsed_time(g1) / 200
-    # The device works through the GEMMs while the host still launches them: the
-    # backlog left when the launches end grows by (GEMM time - launch time) per
-    # GEMM, and it has to outlast the transfer that is enqueued after them.
-    backlog_per_gemm_ms = max(gemm_alone_ms - enqueue_ms, 0.1 * gemm_alone_ms)
     gemm_native = Stream.wrap(gemm_stream.cuda_stream)
     m0, m1 = Event(timing=True), Event(timing=True)
-    tick_pool = [Event(timing=True) for _ in range(512)]
+    tick_pool = [Event(timing=True) for _ in range(1024)]
     c_alone = c.clone()
     out = {"gemm": "4096x4096x4096 bf16, back to back on its own stream",
            "gemm_alone_tflops": round(flop / (gemm_alone_ms / 1e3) / 1e12, 1)}
@@ -672,7 +680,6 @@ def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_
         e1.record(stream)
         e1.synchronize()
         alone_ms = e0.elapsed_ms(e1)
-        count = max(50, int(1.6 * alone_ms / backlog_per_gemm_ms))
         if name == "load":
             xfer.set_layer_events(layer_ev)
             checker.clear_destination()
@@ -680,12 +687,16 @@ def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_
             checker.clear_image(pool)
         c.zero_()
         torch.cuda.synchronize()
+        # A backlog of GEMMs, the transfer (the call only enqueues), then more GEMMs
+        # until the transfer's end event has completed: the GEMM stream is busy
+        # from before the transfer starts until after it ends.
         m0.record(gemm_native)
-        gemms(count, tick_pool)
-        m1.record(gemm_native)
+        gemms(1000)
         e0.record(stream)
         fn(layers, stream, path)
         e1.record(stream)
+        count = gemms(64, tick_pool, until=e1)    # the GEMMs launched after the transfer call
+        m1.record(gemm_native)
         e1.synchronize()
         torch.cuda.synchronize()
         # share of the transfer during which the GEMM stream was running
@@ -847,7 +858,9 @@ def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, pa
         eng.register_context_layer_batch(
             inst, "bench", 0, 0, 0, 1, 1, names, [t.data_ptr() for t in caches],
             [nseg * nb * seg] * n_layers, [nb] * n_layers, [seg] * n_layers, [kv] * n_layers,
-            [nseg] * n_layers, transfer_mode=TransferMode.from_name(mode_name),
+            [nseg] * n_layers,
+            transfer_mode=(TransferMode.ZEROCOPY if mode_name == "zerocopy"
+                           else TransferMode.from_name(mode_name)),
             page_first=w["page_first"])
     for t in dst_cache:
         t.zero_()

@@ -198,6 +198,11 @@ typedef struct pf_merged_range {
 
 #define PF_MODE_DIRECT 0 /* one DMA copy per merged range ("direct") */
 #define PF_MODE_KERNEL 1 /* one copy kernel over mapped host memory ("kernel") */
+/* Worker pools and engine registrations only (not a descriptor backend, not a
+ * name the connector sends): always the zero-copy kernel, whatever the size.
+ * For instances that offload while the GPU is otherwise idle; see
+ * pf_worker_pool_spawn. */
+#define PF_MODE_ZEROCOPY 2
 
 typedef struct pf_backend_s* pf_backend_t;
 
@@ -519,8 +524,13 @@ typedef struct pf_task_result {
 /* GpuWorkerPool::spawn, gpu_worker.rs:131-201: a load thread and a save thread
  * pinned to `numa_node` (< 0 = no pinning), each with its own stream.
  * use_descriptor_backends != 0: per-fragment descriptors through the backend of
- * `transfer_mode`, exactly as the reference; 0: the block-ID engine, with
- * PF_MODE_DIRECT = PF_PATH_AUTO and PF_MODE_KERNEL = PF_PATH_ZEROCOPY.
+ * `transfer_mode`, exactly as the reference (PF_MODE_ZEROCOPY = the kernel
+ * backend); 0: the block-ID engine, which picks the way across the link per
+ * call (PF_PATH_AUTO) for PF_MODE_DIRECT and PF_MODE_KERNEL alike -- the
+ * reference's two modes differ in how they issue the copies, not in the bytes
+ * moved, and what they were invented to choose between (one driver call per
+ * fragment against one kernel) does not arise here -- and always takes the
+ * zero-copy kernel for PF_MODE_ZEROCOPY.
  * Initialisation errors are returned here, synchronously. */
 int pf_worker_pool_spawn(int device_id, int numa_node, int transfer_mode,
                          int use_descriptor_backends, pf_worker_pool_t* out);

@@ -28,6 +28,7 @@ PF_HOST_HUGEPAGES = 2
 
 PF_MODE_DIRECT = 0
 PF_MODE_KERNEL = 1
+PF_MODE_ZEROCOPY = 2
 
 PF_PATH_AUTO = 0
 PF_PATH_ZEROCOPY = 1

@@ -157,7 +157,8 @@ int pf_worker_pool_spawn(int device_id, int numa_node, int transfer_mode,
                          int use_descriptor_backends, pf_worker_pool_t* out) {
   PF_REQUIRE_PTR(out);
   if (device_id < 0) return pf::fail(PF_ERR_INVALID_ARGUMENT, "device_id %d must be >= 0", device_id);
-  if (transfer_mode != PF_MODE_DIRECT && transfer_mode != PF_MODE_KERNEL) {
+  if (transfer_mode != PF_MODE_DIRECT && transfer_mode != PF_MODE_KERNEL &&
+      transfer_mode != PF_MODE_ZEROCOPY) {
     return pf::fail(PF_ERR_INVALID_ARGUMENT, "unknown transfer mode %d", transfer_mode);
   }
   std::string err;
@@ -300,7 +301,8 @@ int pf_engine_register_context_layer_batch(
   PF_REQUIRE_PTR(e);
   PF_REQUIRE_PTR(instance_id);
   PF_REQUIRE_PTR(namespace_);
-  if (transfer_mode != PF_MODE_DIRECT && transfer_mode != PF_MODE_KERNEL) {
+  if (transfer_mode != PF_MODE_DIRECT && transfer_mode != PF_MODE_KERNEL &&
+      transfer_mode != PF_MODE_ZEROCOPY) {
     return pf::fail(PF_ERR_INVALID_ARGUMENT, "unknown transfer mode %d", transfer_mode);
   }
   std::vector<std::string> names;

@@ -450,7 +450,7 @@ int KernelBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_
 }
 
 std::unique_ptr<TransferBackend> build_backend(TransferMode mode) {
-  if (mode == TransferMode::Kernel) return std::unique_ptr<TransferBackend>(new KernelBackend());
+  if (mode != TransferMode::Direct) return std::unique_ptr<TransferBackend>(new KernelBackend());
   return std::unique_ptr<TransferBackend>(new MemcpyBackend());
 }
 

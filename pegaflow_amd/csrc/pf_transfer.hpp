@@ -20,7 +20,11 @@ using CopyDesc = pf_copy_desc;       // transfer/mod.rs:36-44
 using MergedRange = pf_merged_range; // transfer/memcpy.rs:16-20
 
 // transfer/mod.rs:62-76.
-enum class TransferMode : int { Direct = PF_MODE_DIRECT, Kernel = PF_MODE_KERNEL };
+enum class TransferMode : int {
+  Direct = PF_MODE_DIRECT,
+  Kernel = PF_MODE_KERNEL,
+  ZeroCopy = PF_MODE_ZEROCOPY,  // worker pools only: block-ID engine pinned to the zero-copy kernel
+};
 
 // transfer/memcpy.rs:25-55: greedy left-to-right join of list-adjacent copies
 // that share both allocations and are contiguous on both sides.

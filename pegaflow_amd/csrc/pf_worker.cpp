@@ -567,7 +567,10 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
     if (stream) (void)hipStreamDestroy(stream);
     return;
   }
-  const int path = mode_ == TransferMode::Kernel ? PF_PATH_ZEROCOPY : PF_PATH_AUTO;
+  // Direct and kernel mode alike let the engine choose per call: large dense
+  // transfers are staged (their link crossing needs no compute unit, so model
+  // kernels beside them keep their rate), small and scattered ones go zero-copy.
+  const int path = mode_ == TransferMode::ZeroCopy ? PF_PATH_ZEROCOPY : PF_PATH_AUTO;
 
   for (;;) {
     std::unique_ptr<Task> task;

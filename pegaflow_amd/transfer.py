@@ -70,6 +70,7 @@ def merge(copies: Sequence[CopyDesc]) -> list[tuple[int, int, int]]:
 class TransferMode:
     DIRECT = _lib.PF_MODE_DIRECT
     KERNEL = _lib.PF_MODE_KERNEL
+    ZEROCOPY = _lib.PF_MODE_ZEROCOPY   # worker pools / engine registrations only
 
     @staticmethod
     def from_name(name: str) -> int:

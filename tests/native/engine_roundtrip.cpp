@@ -75,7 +75,10 @@ int main(){
   rc|=run(true,1,false,false,1,5,128,8192,60,64);
   rc|=run(true,0,false,false,1,5,2048,65536,1500,1200);   // page-first, whole-page staging (>64 MiB)
   rc|=run(false,0,false,false,2,20,4096,32768,2500,4000); // staged, two-part conversion on load
-  rc|=run(false,1,false,false,2,8,4096,32768,2500,2000);  // kernel mode at the same size: zero-copy both ways
+  rc|=run(false,1,false,false,2,8,4096,32768,2500,2000);  // kernel mode at the same size: the engine picks the path, as in direct mode
+  rc|=run(false,2,false,false,2,8,4096,32768,2500,2000);  // PF_MODE_ZEROCOPY at the same size: zero-copy both ways
+  rc|=run(true,2,false,false,1,5,128,8192,60,64);         // PF_MODE_ZEROCOPY over page-first pages
+  rc|=run(false,2,true,false,2,4,256,4096,100,64);        // PF_MODE_ZEROCOPY with per-fragment descriptors: the kernel backend
   rc|=run(false,0,true,false,2,8,4096,32768,2500,2000);   // per-fragment descriptors, direct backend, 40 000 per task
   rc|=run(false,1,true,false,2,8,4096,32768,2500,2000);   // per-fragment descriptors, kernel backend
   printf(rc?"FAILED\n":"all ok\n"); return rc;

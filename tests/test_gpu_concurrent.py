@@ -178,20 +178,23 @@ def test_save_then_load_next_to_gemm_stream(world, path, copy_stream):
         xfer.save(world.layers(world.src, save_ids, world.pool_a)[:1], stream, path)
         stream.synchronize()
         world.clear_pool(world.pool_a)
-        # The device works through the GEMMs while the host is still launching them, so
-        # the backlog left when the launches end grows by (gemm_ms - enqueue_ms) per
-        # GEMM; it has to outlast ~0.4 s of transfer at link rate, with a margin.
-        assert world.enqueue_ms < 0.8 * world.gemm_ms, "the host cannot launch GEMMs fast enough"
-        count = int(2.0 * 400.0 / (world.gemm_ms - world.enqueue_ms))
+        # A backlog of GEMMs first, so that the stream is busy when the transfer starts;
+        # then the transfer is enqueued (the calls only enqueue), and the host keeps feeding
+        # the GEMM stream until the transfer's last event has completed.
         gemm_native = Stream.wrap(world.gemm_stream.cuda_stream)
         marks = [runtime.Event(timing=True) for _ in range(4)]
         marks[0].record(gemm_native)
+        count = 1500
         world.run_gemms(count)
-        marks[1].record(gemm_native)
         marks[2].record(stream)
         xfer.save(world.layers(world.src, save_ids, world.pool_a), stream, path)
         xfer.load(world.layers(world.dst, load_ids, world.pool_a), stream, path)
         marks[3].record(stream)
+        while not marks[3].query():
+            world.run_gemms(32)
+            count += 32
+            assert count < 40000, "the transfer does not finish"
+        marks[1].record(gemm_native)
         stream.synchronize()
         torch.cuda.synchronize()
         gemm_ms = marks[0].elapsed_ms(marks[1])

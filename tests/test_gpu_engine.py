@@ -77,7 +77,8 @@ def test_save_query_load_roundtrip(engine):
     assert engine.pool_usage()[0] == used and engine.cached_blocks == 4
 
 
-@pytest.mark.parametrize("mode", [TransferMode.DIRECT, TransferMode.KERNEL], ids=["direct", "kernel"])
+@pytest.mark.parametrize("mode", [TransferMode.DIRECT, TransferMode.KERNEL, TransferMode.ZEROCOPY],
+                         ids=["direct", "kernel", "zerocopy"])
 def test_split_layout_roundtrip_both_backends(engine, mode):
     """K/V split registration (tests/common/harness.rs:53-80), both transfer modes."""
     layer = Layer("kv", 16, 4096, split_kv_stride=16 * 4096)
@@ -278,7 +279,8 @@ def test_blockwise_alloc_and_odd_segment_size(gpu):
 
 
 @pytest.mark.parametrize("use_desc", [False, True], ids=["block_ids", "descriptors"])
-@pytest.mark.parametrize("mode", [TransferMode.DIRECT, TransferMode.KERNEL], ids=["direct", "kernel"])
+@pytest.mark.parametrize("mode", [TransferMode.DIRECT, TransferMode.KERNEL, TransferMode.ZEROCOPY],
+                         ids=["direct", "kernel", "zerocopy"])
 def test_worker_pool_matches_oracle(gpu, mode, use_desc):
     """Raw worker ABI: a save task then a load task with a LoadState, checked
     against the oracle's descriptor executor on the same inputs."""

@@ -80,7 +80,8 @@ def test_export_describes_the_allocation(gpu):
     buf.close()
 
 
-@pytest.mark.parametrize("mode", [TransferMode.DIRECT, TransferMode.KERNEL], ids=["direct", "kernel"])
+@pytest.mark.parametrize("mode", [TransferMode.DIRECT, TransferMode.KERNEL, TransferMode.ZEROCOPY],
+                         ids=["direct", "kernel", "zerocopy"])
 def test_save_and_load_of_another_process_caches(gpu, mode):
     layers, nb, seg, nseg = 6, 1024, 32768, 2          # 64 MiB per layer, K/V split
     n = 300
