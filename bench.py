@@ -828,6 +828,26 @@ def run_ref_transfer_bench(torch, np, args):
         print("bench.py: device bytes differ from the host image", file=sys.stderr)
         sys.exit(1)
     headline = next(r for r in rows if r["fragments"] == max_n and r["layout"] == "shuffled")
+    # The same kind of call timed from C++ (no interpreter between the calls): small
+    # block-ID transfers and the smallest row of the table above, with plain
+    # hipMemcpyAsync of the same sizes beside them.
+    native = None
+    native_bin = os.path.join(ROOT, "tests", "native", "small_transfers")
+    if os.path.exists(native_bin) and not args.ref_fragments:
+        import subprocess
+        for o in (xfer, stream, host):
+            o.close()
+        for b in backends.values():
+            b.close()
+        del device_buf
+        torch.cuda.empty_cache()
+        proc = subprocess.run([native_bin], capture_output=True, text=True, timeout=300)
+        lines = [ln for ln in proc.stdout.splitlines() if ln.startswith("{")]
+        if proc.returncode != 0 or not lines:
+            print("bench.py: tests/native/small_transfers failed:\n" + proc.stderr[-2000:],
+                  file=sys.stderr)
+            sys.exit(1)
+        native = json.loads(lines[-1])
     print(json.dumps({
         "metric": "descriptor backends at the shapes of the reference's transfer bench "
                   "(4 KiB fragments), GiB/s",
@@ -837,7 +857,7 @@ def run_ref_transfer_bench(torch, np, args):
         "config": {"workload": "benches/transfer_h2d.rs shapes: 4 KiB fragments, "
                                f"{counts[0]}..{max_n} per batch, contiguous/strided/shuffled, "
                                f"value = kernel backend, shuffled, {max_n} fragments, H2D"},
-        "table": rows}))
+        "table": rows, "native_small_transfers": native}))
 
 
 def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, payload,

@@ -29,6 +29,7 @@ typedef __attribute__((address_space(1))) unsigned char g_u8;
 // and page table: uniform constant loads become scalar loads.
 typedef __attribute__((address_space(4))) const uint32_t c_u32;
 typedef __attribute__((address_space(4))) const uint64_t c_u64;
+typedef __attribute__((address_space(4))) const BlockUnit c_unit;
 
 constexpr int kLanes = 256;
 
@@ -255,7 +256,6 @@ __global__ __launch_bounds__(kLanes) void block_units_kernel(const BlockUnit* __
 // and of ~90 us at 4 MiB).  `slab` is the first argument, so it starts at
 // offset 0 of the argument segment; a unit's `ids` / `far_table` hold byte
 // offsets into it.
-typedef __attribute__((address_space(4))) const BlockUnit c_unit;
 template <int U, bool TO_FAR>
 __global__ __launch_bounds__(kLanes) void block_units_args_kernel(ArgSlab slab, uint32_t first_unit,
                                                                   uint32_t n_units) {
@@ -279,12 +279,12 @@ __global__ __launch_bounds__(kLanes) void block_units_args_kernel(ArgSlab slab, 
 // UNITS_INNER: grid.y walks the (unit, segment) pairs and grid.z the list
 // positions, so workgroups that are dispatched together belong to one
 // position; otherwise grid.y walks the positions of one (unit, segment).
-template <int LT, bool TO_FAR, int SEGS, bool UNITS_INNER>
-__global__ __launch_bounds__(LT) void block_tiles_kernel(const BlockUnit* __restrict__ units) {
+template <int LT, bool TO_FAR, int SEGS, bool UNITS_INNER, typename UnitPtr>
+__device__ __forceinline__ void block_tiles_body(UnitPtr units) {
   constexpr uint32_t kTile = LT * 16;
   const uint32_t unit_seg = UNITS_INNER ? blockIdx.y : blockIdx.z;
   const uint32_t row = UNITS_INNER ? blockIdx.z : blockIdx.y;
-  const BlockUnit* __restrict__ up = units + (SEGS == 2 ? unit_seg >> 1 : unit_seg);
+  UnitPtr up = units + (SEGS == 2 ? unit_seg >> 1 : unit_seg);
   const uint32_t seg = SEGS == 2 ? (unit_seg & 1u) : 0u;
   if (row >= up->n_blocks) return;
   // Rows may visit the list positions in another order (see launch_block_tiles).
@@ -338,6 +338,23 @@ __global__ __launch_bounds__(LT) void block_tiles_kernel(const BlockUnit* __rest
       for (uint32_t j = lane; j < bytes; j += LT) db[j] = sb[j];
     }
   }
+}
+
+template <int LT, bool TO_FAR, int SEGS, bool UNITS_INNER>
+__global__ __launch_bounds__(LT) void block_tiles_kernel(const BlockUnit* __restrict__ units) {
+  block_tiles_body<LT, TO_FAR, SEGS, UNITS_INNER, const BlockUnit*>(units);
+}
+
+// One unit, passed by value: its fields arrive with the kernel's arguments
+// instead of behind a pointer, one dependent scalar load fewer before the id of
+// the workgroup's row is known (a workgroup lives for one load and one store, so
+// every level of that chain is a measurable part of its life).  The unit is the
+// first argument: offset 0 of the argument segment.
+template <int LT, bool TO_FAR, int SEGS>
+__global__ __launch_bounds__(LT) void block_tiles_one_kernel(BlockUnit unit) {
+  (void)unit;
+  block_tiles_body<LT, TO_FAR, SEGS, false, c_unit*>(
+      reinterpret_cast<c_unit*>(reinterpret_cast<uint64_t>(__builtin_amdgcn_kernarg_segment_ptr())));
 }
 
 // The two halves of streams_run_concurrently().  The wait is bounded by the
@@ -462,6 +479,35 @@ int launch_block_units_args(const ArgSlab& slab, uint32_t first_unit, uint32_t n
 #undef PF_LAUNCH_ARGS
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail_hip(e, "block_units_args_kernel launch");
+  return PF_OK;
+}
+
+int launch_block_tiles_one(const BlockUnit& unit, bool to_far, hipStream_t s) {
+  if (unit.n_blocks == 0 || unit.frag_bytes == 0) return PF_OK;
+  if (unit.n_seg != 1 && unit.n_seg != 2) {
+    return fail(PF_ERR_INVALID_ARGUMENT, "tile launch: %u segments per block", unit.n_seg);
+  }
+  constexpr uint64_t kTile = kTileLanes * 16;
+  const uint64_t gx = (unit.frag_bytes + kTile - 1) / kTile;
+  if (unit.n_blocks > kMaxTileBlocks || gx > 0x7FFFFFFFull) {
+    return fail(PF_ERR_INVALID_ARGUMENT, "tile launch out of range: %u blocks, %llu-byte fragments",
+                unit.n_blocks, static_cast<unsigned long long>(unit.frag_bytes));
+  }
+  dim3 grid(static_cast<uint32_t>(gx), unit.n_blocks, unit.n_seg);
+  dim3 block(kTileLanes, 1, 1);
+  if (unit.n_seg == 2) {
+    if (to_far) {
+      hipLaunchKernelGGL((block_tiles_one_kernel<kTileLanes, true, 2>), grid, block, 0, s, unit);
+    } else {
+      hipLaunchKernelGGL((block_tiles_one_kernel<kTileLanes, false, 2>), grid, block, 0, s, unit);
+    }
+  } else if (to_far) {
+    hipLaunchKernelGGL((block_tiles_one_kernel<kTileLanes, true, 1>), grid, block, 0, s, unit);
+  } else {
+    hipLaunchKernelGGL((block_tiles_one_kernel<kTileLanes, false, 1>), grid, block, 0, s, unit);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail_hip(e, "block_tiles_one_kernel launch");
   return PF_OK;
 }
 

@@ -76,6 +76,10 @@ constexpr uint32_t kMaxTileUnits = 32767;
 int launch_block_tiles(const BlockUnit* units, uint32_t n_units, uint32_t max_blocks,
                        uint64_t max_frag_bytes, uint32_t max_seg, bool to_far, hipStream_t s);
 
+// The same for a single unit, handed over by value (its `ids` / `order` are
+// device addresses as usual).
+int launch_block_tiles_one(const BlockUnit& unit, bool to_far, hipStream_t s);
+
 // Plain device copy kernel of the same tile shape, for calibrating counters
 // and measuring the HBM copy ceiling: copies `bytes` (multiple of 16).
 // unroll 0 selects the one-tile-per-workgroup form, 1/2/4/8 the grid-stride form.

@@ -147,8 +147,8 @@ int Xfer::launch_tiles(const BlockUnit* dev_unit, const BlockUnit& host_unit, bo
                        hipStream_t s) {
   int st = timing_begin(s);
   if (st != PF_OK) return st;
-  st = launch_block_tiles(dev_unit, 1, host_unit.n_blocks, host_unit.frag_bytes, host_unit.n_seg,
-                          to_far, s);
+  (void)dev_unit;
+  st = launch_block_tiles_one(host_unit, to_far, s);
   if (st != PF_OK) return st;
   return timing_end(s);
 }
