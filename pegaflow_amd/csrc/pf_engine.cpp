@@ -193,7 +193,7 @@ std::shared_ptr<InstanceContext> Engine::get_instance(const std::string& id, std
   std::lock_guard<std::mutex> lock(mu_);
   auto it = instances_.find(id);
   if (it == instances_.end()) {
-    if (err) *err = "instance " + id + " not registered";
+    if (err) *err = "instance " + id + " not found";  // lib.rs:92
     return nullptr;
   }
   return it->second;
@@ -299,7 +299,7 @@ int Engine::unregister_instance(const std::string& instance_id, std::string* err
     std::lock_guard<std::mutex> lock(mu_);
     auto it = instances_.find(instance_id);
     if (it == instances_.end()) {
-      return bad(err, PF_ERR_INSTANCE_MISSING, "instance " + instance_id + " not registered");
+      return bad(err, PF_ERR_INSTANCE_MISSING, "instance " + instance_id + " not found");
     }
     removed = it->second;
     instances_.erase(it);
@@ -498,7 +498,7 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
   auto gpu = instance->get_gpu(device_id);
   if (!gpu) {
     return bad(err, PF_ERR_WORKER_MISSING,
-               "instance " + instance_id + " has no worker for device " + std::to_string(device_id));
+               "device " + std::to_string(device_id) + " not found in instance " + instance_id);  // lib.rs:93-95
   }
   if (gpu->reg.tp_rank != tp_rank || gpu->reg.pp_rank != pp_rank) {
     return bad(err, PF_ERR_INVALID_ARGUMENT,
@@ -896,7 +896,7 @@ int Engine::batch_load_kv_blocks_multi_layer(
   auto gpu = instance->get_gpu(device_id);
   if (!gpu) {
     return bad(err, PF_ERR_WORKER_MISSING,
-               "instance " + instance_id + " has no worker for device " + std::to_string(device_id));
+               "device " + std::to_string(device_id) + " not found in instance " + instance_id);  // lib.rs:93-95
   }
   if (layer_groups.empty()) {
     return bad(err, PF_ERR_INVALID_ARGUMENT, "load requires at least one layer group");

@@ -5,18 +5,19 @@ that sit on the save / load path, a server over ``PegaEngine`` +
 Wire format: package ``pegaflow``, service ``Engine``, message and field
 numbers of pegaflow-proto/proto/engine.proto:5-197,251-270
 (RegisterContextBatch, Save, Load, QueryPrefetch, Release, UnregisterContext,
-Health, Shutdown).  The descriptors are built at import time with protobuf's
+Health, Shutdown, and the liveness stream Session).  The descriptors are built at import time with protobuf's
 descriptor API because the image has no protoc; the bytes on the wire are
 those a stub generated from engine.proto produces.  Handlers follow
 pegaflow-server/src/service.rs:85-96 (status codes), :110-160 (validation),
 :205-540 (register / save / load), :543-760 (query, release),
-:768-809 (unregister).
+:768-809 (unregister), :1017-1072 with session.rs (a worker's liveness stream:
+when it closes, the instance's mappings and registrations are dropped).
 
 Differences from the reference, on purpose:
   * ``wrapper_bytes`` carries ``HipIPCWrapper.to_bytes()`` records, not pickles;
   * a lease travels as 16 bytes (the reference's size) whose first 8 are this
     engine's 64-bit lease id;
-  * RDMA / MetaServer / Session RPCs are not served (UNIMPLEMENTED).
+  * RDMA / MetaServer RPCs are not served (UNIMPLEMENTED).
 """
 
 from __future__ import annotations
@@ -113,6 +114,9 @@ def _build_file() -> descriptor_pb2.FileDescriptorProto:
     message("ShutdownResponse", [("status", 1, "ResponseStatus")])
     message("HealthRequest", [])
     message("HealthResponse", [("status", 1, "ResponseStatus")])
+    message("SessionRequest", [("instance_id", 1, "string"), ("namespace", 2, "string"),
+                               ("tp_size", 3, "uint32"), ("world_size", 4, "uint32")])
+    message("SessionEvent", [])
     return f
 
 
@@ -135,6 +139,7 @@ ReleaseRequest, ReleaseResponse = _cls("ReleaseRequest"), _cls("ReleaseResponse"
 UnregisterRequest, UnregisterResponse = _cls("UnregisterRequest"), _cls("UnregisterResponse")
 ShutdownRequest, ShutdownResponse = _cls("ShutdownRequest"), _cls("ShutdownResponse")
 HealthRequest, HealthResponse = _cls("HealthRequest"), _cls("HealthResponse")
+SessionRequest, SessionEvent = _cls("SessionRequest"), _cls("SessionEvent")
 
 # method -> (request class, response class)
 METHODS = {
@@ -203,6 +208,11 @@ class EngineService:
         self.shutdown_requested = threading.Event()
         self._pending = []            # submitted loads whose handles are not yet released
         self._pending_lock = threading.Lock()
+        # session.rs: the current liveness session of each instance; a newer one
+        # supersedes the older, whose end then cleans nothing up
+        self._sessions = {}
+        self._sessions_lock = threading.Lock()
+        self._next_session = 0
 
     def _reap(self, wait: bool = False) -> None:
         """Release the handles of loads that have settled (their outcome went to
@@ -361,6 +371,41 @@ class EngineService:
     def Health(self, req):
         return HealthResponse(status=_ok())
 
+    # -- Session (service.rs:1017-1072, session.rs) ------------------------------
+    def Session(self, req, context):
+        """Server-streaming and silent: it lasts as long as the worker holds it.
+        When the stream ends (the worker closed it, or died and its socket
+        closed) the instance's mapped tensors and registrations are dropped,
+        unless a newer session has taken the instance over."""
+        if not req.instance_id:
+            context.abort(grpc.StatusCode.INVALID_ARGUMENT, "instance_id must not be empty")
+        with self._sessions_lock:
+            self._next_session += 1
+            token = self._next_session
+            self._sessions[req.instance_id] = token
+        ended = threading.Event()
+        context.add_callback(ended.set)
+        while not ended.wait(0.05):
+            if self.shutdown_requested.is_set() or not context.is_active():
+                break
+        with self._sessions_lock:
+            owned = self._sessions.get(req.instance_id) == token
+            if owned:
+                del self._sessions[req.instance_id]
+        if owned:
+            self.cleanup_instance(req.instance_id)
+        return
+        yield SessionEvent()  # pragma: no cover -- makes this a generator (a stream with no events)
+
+    def cleanup_instance(self, instance_id: str) -> None:
+        """service.rs cleanup_instance: what UnregisterContext does, without a caller
+        to report to."""
+        try:
+            self.engine.unregister_instance(instance_id)
+        except _lib.PegaHipError:
+            pass
+        self.registry.drop_instance(instance_id)
+
     def Shutdown(self, req):
         self.shutdown_requested.set()
         return ShutdownResponse(status=_ok())
@@ -380,11 +425,14 @@ class EngineService:
             handlers[name] = grpc.unary_unary_rpc_method_handler(
                 behavior, request_deserializer=req_cls.FromString,
                 response_serializer=resp_cls.SerializeToString)
+        handlers["Session"] = grpc.unary_stream_rpc_method_handler(
+            self.Session, request_deserializer=SessionRequest.FromString,
+            response_serializer=SessionEvent.SerializeToString)
         return grpc.method_handlers_generic_handler(SERVICE, handlers)
 
 
 def serve(engine: PegaEngine, address: str = DEFAULT_ENDPOINT, registry: TensorRegistry | None = None,
-          max_workers: int = 8):
+          max_workers: int = 32):
     """Start a server; returns (grpc.Server, EngineService, bound port)."""
     service = EngineService(engine, registry)
     server = grpc.server(futures.ThreadPoolExecutor(max_workers=max_workers),
@@ -398,6 +446,19 @@ def serve(engine: PegaEngine, address: str = DEFAULT_ENDPOINT, registry: TensorR
 
 class PegaFlowError(RuntimeError):
     """The server is unavailable or failed internally."""
+
+    def __init__(self, message: str, code: str = "UNKNOWN"):
+        super().__init__(message)
+        self.code = code
+
+
+class RpcRejected(ValueError):
+    """The server refused the request (INVALID_ARGUMENT or FAILED_PRECONDITION);
+    ``code`` is the gRPC status name, the text is the server's message."""
+
+    def __init__(self, message: str, code: str):
+        super().__init__(message)
+        self.code = code
 
 
 class EngineRpcClient:
@@ -420,7 +481,38 @@ class EngineRpcClient:
         return self._endpoint
 
     def close(self) -> None:
+        self.stop_session_watcher()
         self._channel.close()
+
+    def start_session_watcher(self, instance_id: str, namespace: str, tp_size: int,
+                              world_size: int) -> None:
+        """Open the liveness stream and hold it for the life of this client (or
+        process): when it ends, the server drops the instance.  Calling again
+        replaces the previous stream (pegaflow.pyi:290-315)."""
+        self.stop_session_watcher()
+        call = self._channel.unary_stream(
+            f"/{SERVICE}/Session", request_serializer=SessionRequest.SerializeToString,
+            response_deserializer=SessionEvent.FromString)(
+                SessionRequest(instance_id=instance_id, namespace=namespace, tp_size=tp_size,
+                               world_size=world_size))
+
+        def drain():
+            try:
+                for _event in call:
+                    pass
+            except grpc.RpcError:
+                pass
+
+        thread = threading.Thread(target=drain, name="pegaflow-session", daemon=True)
+        thread.start()
+        self._session = (call, thread)
+
+    def stop_session_watcher(self) -> None:
+        session = getattr(self, "_session", None)
+        if session is not None:
+            session[0].cancel()
+            session[1].join(timeout=5)
+            self._session = None
 
     def _call(self, name, request):
         try:
@@ -428,8 +520,8 @@ class EngineRpcClient:
         except grpc.RpcError as err:
             code, detail = err.code(), err.details()
             if code in (grpc.StatusCode.INVALID_ARGUMENT, grpc.StatusCode.FAILED_PRECONDITION):
-                raise ValueError(detail) from None
-            raise PegaFlowError(f"{code.name}: {detail}") from None
+                raise RpcRejected(detail, code.name) from None
+            raise PegaFlowError(f"{code.name}: {detail}", code.name) from None
 
     def health(self) -> tuple[bool, str]:
         r = self._call("Health", HealthRequest())

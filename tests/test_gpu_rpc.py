@@ -47,3 +47,55 @@ def test_worker_process_saves_and_loads_through_grpc(gpu, backend):
         service.close()
         service.registry.close()
         engine.close()
+
+
+def test_reference_rpc_scenarios(gpu):
+    """The cases of pegaflow-server/tests/mock_vllm_rpc_e2e.rs (line numbers
+    below), run by tests/rpc_scenarios_child.py against this process's server."""
+    from pegaflow_amd import rpc
+    scenarios = os.path.join(os.path.dirname(os.path.abspath(__file__)), "rpc_scenarios_child.py")
+    engine = PegaEngine(pool_size=64 << 20)
+    server, service, port = rpc.serve(engine, "127.0.0.1:0")
+    try:
+        proc = subprocess.run([sys.executable, "-u", scenarios, str(port)], capture_output=True,
+                              text=True, timeout=150)
+        assert proc.returncode == 0, proc.stderr[-3000:]
+        out = json.loads([ln for ln in proc.stdout.splitlines() if ln.startswith("{")][-1])
+        ok = [True, ""]
+        # :26-77 save / query / load round trip
+        assert out["register"] == ok and out["save"] == ok
+        assert out["cold_query"] == ["ready", 0, 0]
+        assert out["hit_query"] == ["ready", 4, 16]
+        assert out["load"] == [ok, 1] and out["roundtrip_matches"]
+        # :79-96
+        assert out["empty_req_id"] == ["INVALID_ARGUMENT", "req_id must not be empty"]
+        # :98-131 a lease is bound to its instance; the refused load settles its LoadState as an error
+        code, message = out["wrong_instance_load"][0]
+        assert "query lease belongs to instance" in message and out["wrong_instance_load"][1] < 0
+        # :133-171
+        assert out["first_release"] == ["accepted", ""]
+        assert out["second_release"] == ["FAILED_PRECONDITION", "query lease is unknown or expired"]
+        # :173-201 a partial prefix gives a lease over the prefix
+        assert out["prefix_save"] == ok and out["prefix_query"] == ["ready", 2, 16]
+        assert out["prefix_load"] == [ok, 1] and out["prefix_loaded_suffix_zero"]
+        # :203-240
+        assert out["mismatch_hits"] == 2
+        code, message = out["mismatch_load"][0]
+        assert code == "INVALID_ARGUMENT"
+        assert "query lease block count 2 does not match destination block count 4" in message
+        assert out["mismatch_load"][1] < 0
+        # :318-410 (two tensor-parallel workers) needs two GPUs; the reference skips it below two
+        # :242-316 the end of the liveness stream drops the instance
+        assert out["session_save"] == ok and out["session_hits"] == 4
+        for key in ("session_cleanup_probe", "session_save_after_cleanup"):
+            assert out[key][0] == "FAILED_PRECONDITION", out[key]
+            assert "instance mock-vllm-rpc-e2e-session not found" in out[key][1], out[key]
+        code, message = out["session_load_after_cleanup"][0]
+        assert code == "FAILED_PRECONDITION" and "not found" in message
+        assert out["session_load_after_cleanup"][1] < 0
+        assert out["first_instance_still_hits"] == 4
+    finally:
+        server.stop(grace=None)
+        service.close()
+        service.registry.close()
+        engine.close()
