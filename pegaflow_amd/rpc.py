@@ -134,7 +134,7 @@ SaveLayer, SaveRequest, SaveResponse = _cls("SaveLayer"), _cls("SaveRequest"), _
 LoadGroup, LoadBlockTarget, LoadBlockIds = _cls("LoadGroup"), _cls("LoadBlockTarget"), _cls("LoadBlockIds")
 LeaseLoad, LoadRequest, LoadResponse = _cls("LeaseLoad"), _cls("LoadRequest"), _cls("LoadResponse")
 QueryRequest, QueryResponse = _cls("QueryRequest"), _cls("QueryResponse")
-QueryLoading, QueryReady = _cls("QueryLoading"), _cls("QueryReady")
+QueryLoadingMsg, QueryReadyMsg = _cls("QueryLoading"), _cls("QueryReady")
 ReleaseRequest, ReleaseResponse = _cls("ReleaseRequest"), _cls("ReleaseResponse")
 UnregisterRequest, UnregisterResponse = _cls("UnregisterRequest"), _cls("UnregisterResponse")
 ShutdownRequest, ShutdownResponse = _cls("ShutdownRequest"), _cls("ShutdownResponse")
@@ -330,19 +330,19 @@ class EngineService:
                 positions = [i for i, hit in enumerate(present) if hit]
                 if req.wait_for_full_prefix and len(positions) != len(hashes):
                     # all-or-nothing want-set: a short answer carries no lease
-                    ready = QueryReady(num_hit_blocks=len(positions), lease=b"",
+                    ready = QueryReadyMsg(num_hit_blocks=len(positions), lease=b"",
                                        hit_positions=list(range(len(positions))))
                     return QueryResponse(ready=ready)
                 lease = b""
                 if positions:
                     lease = lease_to_bytes(self.engine.create_group_lease(
                         req.instance_id, req.group_id, [hashes[i] for i in positions]))
-                return QueryResponse(ready=QueryReady(num_hit_blocks=len(positions), lease=lease,
+                return QueryResponse(ready=QueryReadyMsg(num_hit_blocks=len(positions), lease=lease,
                                                       hit_positions=positions))
             hits, lease = self.engine.query_prefix(req.instance_id, hashes)
         except Exception as exc:
             raise _map_engine_error(exc)
-        return QueryResponse(ready=QueryReady(num_hit_blocks=hits,
+        return QueryResponse(ready=QueryReadyMsg(num_hit_blocks=hits,
                                               lease=lease_to_bytes(lease) if hits else b""))
 
     # -- Release (service.rs:738-766) -----------------------------------------
@@ -461,6 +461,27 @@ class RpcRejected(ValueError):
         self.code = code
 
 
+class QueryLoading:
+    """The query's backing fetch is still in progress (python/pegaflow/pegaflow.pyi:55-56)."""
+
+    def __repr__(self) -> str:
+        return "QueryLoading()"
+
+
+class QueryReady:
+    """pegaflow.pyi:58-67: the hit count, the lease over the hit blocks (empty on
+    0 hits) and, for membership queries, the hit positions."""
+
+    def __init__(self, num_hit_blocks: int, lease: bytes, hit_positions: Sequence[int] = ()):
+        self.num_hit_blocks = int(num_hit_blocks)
+        self.lease = bytes(lease)
+        self.hit_positions = list(hit_positions)
+
+    def __repr__(self) -> str:
+        return (f"QueryReady(num_hit_blocks={self.num_hit_blocks}, lease={self.lease.hex()}, "
+                f"hit_positions={self.hit_positions})")
+
+
 class EngineRpcClient:
     """Client with the method names, argument order and return values of the
     reference's ``EngineRpcClient`` (python/pegaflow/pegaflow.pyi:69-300)."""
@@ -574,13 +595,13 @@ class EngineRpcClient:
 
     def query_prefetch(self, instance_id: str, block_hashes: Sequence[bytes], req_id: str,
                        wait_for_full_prefix: bool = False, group_id: int = 0):
-        """-> ("loading",) or ("ready", num_hit_blocks, lease bytes, hit_positions)."""
+        """-> QueryLoading or QueryReady."""
         r = self._call("QueryPrefetch", QueryRequest(
             instance_id=instance_id, block_hashes=list(block_hashes), req_id=req_id,
             wait_for_full_prefix=wait_for_full_prefix, group_id=group_id))
         if r.WhichOneof("outcome") == "loading":
-            return ("loading",)
-        return ("ready", r.ready.num_hit_blocks, bytes(r.ready.lease), list(r.ready.hit_positions))
+            return QueryLoading()
+        return QueryReady(r.ready.num_hit_blocks, bytes(r.ready.lease), list(r.ready.hit_positions))
 
     def release(self, lease: bytes) -> None:
         self._call("Release", ReleaseRequest(lease=lease))

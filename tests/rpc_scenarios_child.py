@@ -87,10 +87,14 @@ def main():
     inst = "mock-vllm-rpc-e2e"
     out["register"] = list(register(inst, gpu))
     hs = hashes(17)
-    out["cold_query"] = list(client.query_prefetch(inst, hs, "mock-vllm-cold-query"))[:3]
-    out["cold_query"][2] = len(out["cold_query"][2])
+    def query(instance, hs_, req_id):
+        r = client.query_prefetch(instance, hs_, req_id)
+        return type(r).__name__, r.num_hit_blocks, r.lease, r.hit_positions
+
+    cold = query(inst, hs, "mock-vllm-cold-query")
+    out["cold_query"] = [cold[0], cold[1], len(cold[2])]
     out["save"] = list(save(inst, hs))
-    kind, hits, lease, _ = client.query_prefetch(inst, hs, "mock-vllm-hit-query")
+    kind, hits, lease, _ = query(inst, hs, "mock-vllm-hit-query")
     out["hit_query"] = [kind, hits, len(lease)]
     gpu.zero()
     out["load"] = load(inst, lease, len(hs))
@@ -102,7 +106,7 @@ def main():
     # mock_vllm_query_lease_is_bound_to_instance_id
     hs = hashes(37)
     save(inst, hs)
-    _k, _h, lease, _ = client.query_prefetch(inst, hs, "mock-vllm-instance-bound")
+    _k, _h, lease, _ = query(inst, hs, "mock-vllm-instance-bound")
     second = Gpu()
     register("mock-vllm-rpc-e2e-second", second)
     out["wrong_instance_load"] = load("mock-vllm-rpc-e2e-second", lease, len(hs))
@@ -111,14 +115,14 @@ def main():
     # mock_vllm_release_unknown_lease_returns_error
     hs = hashes(39)
     save(inst, hs)
-    _k, _h, lease, _ = client.query_prefetch(inst, hs, "mock-vllm-release-once")
+    _k, _h, lease, _ = query(inst, hs, "mock-vllm-release-once")
     out["first_release"] = rejected(lambda: client.release(lease))
     out["second_release"] = rejected(lambda: client.release(lease))
 
     # mock_vllm_prefix_partial_query_returns_prefix_lease
     hs = hashes(41)
     out["prefix_save"] = list(save(inst, hs[:2]))
-    kind, hits, lease, _ = client.query_prefetch(inst, hs, "mock-vllm-prefix-partial")
+    kind, hits, lease, _ = query(inst, hs, "mock-vllm-prefix-partial")
     out["prefix_query"] = [kind, hits, len(lease)]
     gpu.zero()
     out["prefix_load"] = load(inst, lease, 2)
@@ -127,7 +131,7 @@ def main():
     # mock_vllm_load_rejects_lease_block_count_mismatch
     hs = hashes(43)
     save(inst, hs[:2])
-    _k, hits, lease, _ = client.query_prefetch(inst, hs, "mock-vllm-load-count-mismatch")
+    _k, hits, lease, _ = query(inst, hs, "mock-vllm-load-count-mismatch")
     out["mismatch_hits"] = hits
     out["mismatch_load"] = load(inst, lease, len(hs))
 
@@ -141,7 +145,7 @@ def main():
     client.start_session_watcher(si, "mock-vllm", 1, 1)
     hs = hashes(47)
     out["session_save"] = list(save(si, hs))
-    _k, hits, lease, _ = client.query_prefetch(si, hs, "mock-vllm-session-cleanup-hit")
+    _k, hits, lease, _ = query(si, hs, "mock-vllm-session-cleanup-hit")
     out["session_hits"] = hits
     client.stop_session_watcher()              # the stream ends: the server cleans the instance up
     deadline = time.time() + 10
@@ -157,7 +161,7 @@ def main():
 
     # the first instance is still served after all of that
     hs = hashes(17)
-    _k, hits, lease, _ = client.query_prefetch(inst, hs, "still-there")
+    _k, hits, lease, _ = query(inst, hs, "still-there")
     out["first_instance_still_hits"] = hits
     client.release(lease)
     client.close()

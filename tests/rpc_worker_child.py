@@ -63,8 +63,9 @@ def main():
     for c in caches:
         c.zero_()
     torch.cuda.synchronize()
-    kind, hits, lease, positions = client.query_prefetch("rpc-inst", hashes + [b"missing"], "req-1")
-    out["query"] = [kind, hits, len(lease), positions]
+    ready = client.query_prefetch("rpc-inst", hashes + [b"missing"], "req-1")
+    hits, lease = ready.num_hit_blocks, ready.lease
+    out["query"] = [type(ready).__name__, hits, len(lease), ready.hit_positions]
     state = LoadState()
     # every second block of the lease goes nowhere (an absent target)
     targets = [int(b) if i % 2 == 0 else None for i, b in enumerate(dst)]
@@ -94,9 +95,9 @@ def main():
         out["release_consumed"] = "accepted"
     except ValueError as exc:
         out["release_consumed"] = str(exc)
-    kind, hits, lease2, _ = client.query_prefetch("rpc-inst", hashes[:3], "req-2")
-    client.release(lease2)
-    out["released"] = [kind, hits]
+    again = client.query_prefetch("rpc-inst", hashes[:3], "req-2")
+    client.release(again.lease)
+    out["released"] = [type(again).__name__, again.num_hit_blocks]
     try:
         client.release(b"short")
         out["bad_lease"] = "accepted"

@@ -34,11 +34,11 @@ def test_worker_process_saves_and_loads_through_grpc(gpu, backend):
         assert out["register"] == [True, ""] and out["save"] == [True, ""]
         assert "already registered" in out["second_register"]
         assert out["bad_save"].startswith("block_ids length 2 does not match block_hashes 1 for layer")
-        assert out["query"] == ["ready", n, 16, []]          # the trailing miss ends the prefix
+        assert out["query"] == ["QueryReady", n, 16, []]          # the trailing miss ends the prefix
         assert out["load"] == [True, ""] and out["load_state"] == 1
         assert out["problems"] == []
         assert out["release_consumed"] == "query lease is unknown or expired"
-        assert out["released"] == ["ready", 3]
+        assert out["released"] == ["QueryReady", 3]
         assert out["bad_lease"] == "query lease id must be 16 bytes, got 5"
         assert out["unregister"] == [True, ""]
         assert len(service.registry) == 0
@@ -64,8 +64,8 @@ def test_reference_rpc_scenarios(gpu):
         ok = [True, ""]
         # :26-77 save / query / load round trip
         assert out["register"] == ok and out["save"] == ok
-        assert out["cold_query"] == ["ready", 0, 0]
-        assert out["hit_query"] == ["ready", 4, 16]
+        assert out["cold_query"] == ["QueryReady", 0, 0]
+        assert out["hit_query"] == ["QueryReady", 4, 16]
         assert out["load"] == [ok, 1] and out["roundtrip_matches"]
         # :79-96
         assert out["empty_req_id"] == ["INVALID_ARGUMENT", "req_id must not be empty"]
@@ -76,7 +76,7 @@ def test_reference_rpc_scenarios(gpu):
         assert out["first_release"] == ["accepted", ""]
         assert out["second_release"] == ["FAILED_PRECONDITION", "query lease is unknown or expired"]
         # :173-201 a partial prefix gives a lease over the prefix
-        assert out["prefix_save"] == ok and out["prefix_query"] == ["ready", 2, 16]
+        assert out["prefix_save"] == ok and out["prefix_query"] == ["QueryReady", 2, 16]
         assert out["prefix_load"] == [ok, 1] and out["prefix_loaded_suffix_zero"]
         # :203-240
         assert out["mismatch_hits"] == 2
@@ -95,6 +95,46 @@ def test_reference_rpc_scenarios(gpu):
         assert out["session_load_after_cleanup"][1] < 0
         assert out["first_instance_still_hits"] == 4
     finally:
+        server.stop(grace=None)
+        service.close()
+        service.registry.close()
+        engine.close()
+
+
+def test_killed_worker_releases_its_tensors(gpu, tmp_path):
+    """python/tests/test_session_watcher.py:50-99: a worker that dies without
+    unregistering (SIGKILL) closes its liveness stream with its socket; the
+    server then drops the instance's mapped tensors and its registration."""
+    import signal
+    import time
+    from pegaflow_amd import _lib, rpc
+    child = os.path.join(os.path.dirname(os.path.abspath(__file__)), "rpc_crash_child.py")
+    engine = PegaEngine(pool_size=16 << 20)
+    server, service, port = rpc.serve(engine, "127.0.0.1:0")
+    instance = f"inst-crash-{os.getpid()}"
+    ready = tmp_path / "ready"
+    worker = subprocess.Popen([sys.executable, "-u", child, str(port), instance, str(ready)],
+                              stdout=subprocess.PIPE, stderr=subprocess.PIPE)
+    try:
+        deadline = time.monotonic() + 60
+        while not ready.exists():
+            assert worker.poll() is None, worker.stderr.read().decode(errors="replace")[-2000:]
+            assert time.monotonic() < deadline, "worker did not become ready"
+            time.sleep(0.05)
+        assert len(service.registry) == 1
+        assert engine.query_prefix(instance, [b"crash-a", b"crash-b"])[0] == 2
+        worker.send_signal(signal.SIGKILL)
+        worker.wait(timeout=5)
+        deadline = time.monotonic() + 10
+        while len(service.registry) != 0 and time.monotonic() < deadline:
+            time.sleep(0.05)
+        assert len(service.registry) == 0, "the dead worker's tensors are still mapped"
+        with pytest.raises(_lib.InstanceMissing, match=f"instance {instance} not found"):
+            engine.query_prefix(instance, [b"crash-a"])
+    finally:
+        if worker.poll() is None:
+            worker.kill()
+            worker.wait(timeout=5)
         server.stop(grace=None)
         service.close()
         service.registry.close()
