@@ -54,10 +54,10 @@ def test_load_request_absent_target_and_lease():
 
 
 def test_query_response_oneof():
-    ready = rpc.QueryResponse(ready=rpc.QueryReady(num_hit_blocks=3, lease=b"x" * 16,
+    ready = rpc.QueryResponse(ready=rpc.QueryReadyMsg(num_hit_blocks=3, lease=b"x" * 16,
                                                    hit_positions=[0, 2]))
     assert ready.SerializeToString() == bytes.fromhex("1218" "0803" "1210" + "78" * 16 + "1a020002")
-    loading = rpc.QueryResponse(loading=rpc.QueryLoading())
+    loading = rpc.QueryResponse(loading=rpc.QueryLoadingMsg())
     assert loading.SerializeToString() == bytes.fromhex("0a00")
     assert rpc.QueryResponse.FromString(bytes.fromhex("0a00")).WhichOneof("outcome") == "loading"
 
