@@ -257,9 +257,25 @@ int MemcpyBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_
   };
   std::vector<Run> runs;
   std::vector<std::pair<uint64_t, size_t>> open;  // host allocation -> index of its open run
+  // A batch whose small ranges add up to little is not worth the staging hop
+  // (pack kernel + copy + their hand-over): when every range has a device-visible
+  // host address the copy kernel moves them over the link directly, and at this
+  // size it is gone before it could matter to a kernel running beside it.
+  // Measured on MI355X, 4 KiB fragments shuffled, call + synchronise: 1024
+  // fragments 33 GiB/s staged against 42 through the kernel, 4096 fragments 43
+  // against 48.
+  uint64_t small_bytes = 0;
+  bool small_mapped = true;
+  for (const Range& r : ranges) {
+    if (r.size >= kLargeRange || r.size == 0) continue;
+    small_bytes += r.size;
+    small_mapped = small_mapped && r.host_device != 0;
+  }
+  const bool all_by_kernel = small_mapped && small_bytes <= kKernelBelowBytes;
   for (size_t i = 0; i < ranges.size(); ++i) {
     const Range& r = ranges[i];
     if (r.size >= kLargeRange || r.size == 0) continue;
+    if (all_by_kernel) continue;  // listed as isolated below, without a run record each
     size_t oi = 0;
     while (oi < open.size() && open[oi].first != r.host_allocation) ++oi;
     if (oi < open.size()) {
@@ -279,6 +295,12 @@ int MemcpyBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_
   std::vector<uint32_t> isolated;
   bool isolated_mapped = true;
   uint64_t staged_pieces = 0, max_staged_piece = 0, max_run_bytes = 0;
+  if (all_by_kernel) {
+    isolated.reserve(ranges.size());
+    for (size_t i = 0; i < ranges.size(); ++i) {
+      if (ranges[i].size < kLargeRange && ranges[i].size != 0) isolated.push_back(static_cast<uint32_t>(i));
+    }
+  }
   for (const Run& run : runs) {
     if (run.members.size() == 1) {
       isolated.push_back(run.members[0]);

@@ -87,6 +87,7 @@ class MemcpyBackend : public TransferBackend {
   static constexpr uint64_t kLargeRange = 4ull << 20;   // copied on its own from this size on
   static constexpr uint64_t kFewRanges = 8;             // batches up to this size: one copy per range
   static constexpr uint64_t kStagingBytes = 256ull << 20;
+  static constexpr uint64_t kKernelBelowBytes = 16ull << 20;  // small batches skip the staging hop
 
  private:
   int submit(const CopyDesc* copies, uint64_t n, bool host_is_src, hipStream_t s);
