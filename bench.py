@@ -90,10 +90,13 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["ref_transfer_bench"],
+    ap.add_argument("--workload",
+                    choices=sorted(WORKLOADS) + ["ref_transfer_bench", "ref_cpu_path"],
                     default="llama8b",
                     help="ref_transfer_bench = the shapes of the reference's own "
-                         "benches/transfer_h2d.rs through the descriptor backends")
+                         "benches/transfer_h2d.rs through the descriptor backends; "
+                         "ref_cpu_path = the engine-level groups of its benches/cpu_path.rs "
+                         "(long lists of 1 KiB blocks through save / query / load)")
     ap.add_argument("--path", choices=["auto", "staged", "zerocopy"], default="auto")
     ap.add_argument("--layers", type=int, default=0, help="override the layer count")
     ap.add_argument("--slot-mb", type=int, default=0)
@@ -155,6 +158,9 @@ def main():
         print("bench.py: this build runs on exactly one GPU (the path has no inter-GPU step); "
               f"--gpus {args.gpus} is not supported", file=sys.stderr)
         sys.exit(2)
+    if args.workload == "ref_cpu_path":  # a native program; nothing here touches the GPU
+        run_ref_cpu_path()
+        return
 
     import numpy as np
     import torch
@@ -858,6 +864,39 @@ def run_ref_transfer_bench(torch, np, args):
                                f"{counts[0]}..{max_n} per batch, contiguous/strided/shuffled, "
                                f"value = kernel backend, shuffled, {max_n} fragments, H2D"},
         "table": rows, "native_small_transfers": native}))
+
+
+def run_ref_cpu_path():
+    """The engine's CPU path on long block lists: tests/native/cpu_path.cpp, a C++
+    program over the C ABI with the groups and shapes of the reference's
+    pegaflow-core/benches/cpu_path.rs:389-774 (block counts 128..32768 of 1 KiB,
+    one layer or 61).  value = blocks per second through save + flush at 8192
+    unique blocks of one layer."""
+    import subprocess
+    native_bin = os.path.join(ROOT, "tests", "native", "cpu_path")
+    if not os.path.exists(native_bin):
+        print(f"bench.py: {native_bin} is missing: make -C pegaflow_amd/csrc", file=sys.stderr)
+        sys.exit(1)
+    proc = subprocess.run([native_bin], capture_output=True, text=True, timeout=900)
+    lines = [ln for ln in proc.stdout.splitlines() if ln.startswith("{")]
+    if proc.returncode != 0 or not lines:
+        print("bench.py: tests/native/cpu_path failed:\n" + proc.stdout[-2000:] + proc.stderr[-2000:],
+              file=sys.stderr)
+        sys.exit(1)
+    rows = json.loads(lines[-1])["rows"]
+    head = next(r for r in rows if r["group"] == "save_flush_unique" and r["case"] == "8192")
+    print(json.dumps({
+        "metric": "engine CPU path at the shapes of the reference's cpu_path bench, blocks/s "
+                  "(save + flush, 8192 unique 1 KiB blocks, one layer)",
+        "value": round(8192 / head["mean_us"] * 1e6, 1), "unit": "blocks/s", "n_gpus": 1,
+        "steps": 10, "warmup": 3, "ms_per_step": round(head["mean_us"] / 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
+        "data": "synthetic",
+        "config": {"workload": "benches/cpu_path.rs groups: save_flush_unique, "
+                               "save_flush_cpu_multilayer_61, save_flush_dtoh_multilayer_61, "
+                               "save/load_transfer_fragmentation, query_prefetch_lease, "
+                               "load_submit_wait"},
+        "table": rows}))
 
 
 def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, payload,

@@ -6,30 +6,58 @@
 #include <cstdint>
 #include <memory>
 #include <string>
+#include <string_view>
 #include <vector>
 
 #include "pf_pool.hpp"
 
 namespace pf {
 
-// pegaflow-common/src/block.rs:5-21.
+// pegaflow-common/src/block.rs:5-21: (namespace, hash bytes).  The namespace
+// is the small integer the engine assigned to its name, and the digest of the
+// pair is computed once, when the key (or a view of it) is built: a save looks
+// every key up twice and inserts it once, a query looks it up once.
+inline size_t block_key_digest(uint32_t ns, std::string_view hash) {
+  return std::hash<std::string_view>{}(hash) ^ (static_cast<size_t>(ns) * 0x9E3779B97F4A7C15ull);
+}
 struct BlockKey {
-  std::string ns;
+  uint32_t ns = 0;
   std::string hash;  // raw bytes
-  bool operator<(const BlockKey& o) const { return ns != o.ns ? ns < o.ns : hash < o.hash; }
-  bool operator==(const BlockKey& o) const { return ns == o.ns && hash == o.hash; }
+  size_t digest = 0;
+  BlockKey() = default;
+  BlockKey(uint32_t ns_id, std::string hash_bytes)
+      : ns(ns_id), hash(std::move(hash_bytes)), digest(block_key_digest(ns, hash)) {}
+};
+// The same without owning the bytes, for look-ups.
+struct BlockKeyView {
+  uint32_t ns = 0;
+  std::string_view hash;
+  size_t digest = 0;
+  BlockKeyView(uint32_t ns_id, std::string_view hash_bytes)
+      : ns(ns_id), hash(hash_bytes), digest(block_key_digest(ns, hash)) {}
+};
+struct BlockKeyHash {
+  using is_transparent = void;
+  size_t operator()(const BlockKey& k) const { return k.digest; }
+  size_t operator()(const BlockKeyView& k) const { return k.digest; }
+};
+struct BlockKeyEqual {
+  using is_transparent = void;
+  template <typename A, typename B>
+  bool operator()(const A& a, const B& b) const {
+    return a.digest == b.digest && a.ns == b.ns && std::string_view(a.hash) == std::string_view(b.hash);
+  }
 };
 
 // pegaflow-common/src/block.rs:30-43: group 0 keeps the raw hash, groups >= 1
 // append the big-endian group id.
-inline std::string group_hash(const std::string& hash, uint32_t group_id) {
+inline std::string group_hash(std::string hash, uint32_t group_id) {
   if (group_id == 0) return hash;
-  std::string out = hash;
-  out.push_back(static_cast<char>((group_id >> 24) & 0xFF));
-  out.push_back(static_cast<char>((group_id >> 16) & 0xFF));
-  out.push_back(static_cast<char>((group_id >> 8) & 0xFF));
-  out.push_back(static_cast<char>(group_id & 0xFF));
-  return out;
+  hash.push_back(static_cast<char>((group_id >> 24) & 0xFF));
+  hash.push_back(static_cast<char>((group_id >> 16) & 0xFF));
+  hash.push_back(static_cast<char>((group_id >> 8) & 0xFF));
+  hash.push_back(static_cast<char>(group_id & 0xFF));
+  return hash;
 }
 
 // block.rs:62-88: one contiguous range of pinned memory; keeps its allocation alive.
@@ -124,14 +152,23 @@ class SealedBlock {
 // block.rs:346-454: slots arrive one by one; seals when none remain.
 class InflightBlock {
  public:
-  explicit InflightBlock(size_t total_slots)
-      : slots_(total_slots), filled_(total_slots, false), remaining_(total_slots),
-        created_(std::chrono::steady_clock::now()) {}
+  using Clock = std::chrono::steady_clock;
+  // `created` lets a save that begins thousands of blocks read the clock once.
+  explicit InflightBlock(size_t total_slots, Clock::time_point created = Clock::now())
+      : slots_(total_slots), remaining_(total_slots), created_(created) {}
   enum class Insert { Inserted, Completed, Duplicate };
   Insert insert_slot(size_t slot_id, RawBlock block) {
-    if (slot_id >= slots_.size() || filled_[slot_id]) return Insert::Duplicate;
+    if (slot_id >= slots_.size() || filled(slot_id)) return Insert::Duplicate;
     slots_[slot_id] = std::move(block);
-    filled_[slot_id] = true;
+    --remaining_;
+    return remaining_ == 0 ? Insert::Completed : Insert::Inserted;
+  }
+  // The empty slot to build a block in, or null when it is taken or out of
+  // range; the caller confirms with slot_filled() once the block is in place.
+  RawBlock* empty_slot(size_t slot_id) {
+    return slot_id >= slots_.size() || filled(slot_id) ? nullptr : &slots_[slot_id];
+  }
+  Insert slot_filled() {
     --remaining_;
     return remaining_ == 0 ? Insert::Completed : Insert::Inserted;
   }
@@ -140,9 +177,7 @@ class InflightBlock {
   bool complete() const { return remaining_ == 0; }
   // Time since the first slot arrived (write_path.rs:302-330 collects blocks
   // that stay incomplete for too long).
-  std::chrono::steady_clock::duration age() const {
-    return std::chrono::steady_clock::now() - created_;
-  }
+  Clock::duration age() const { return Clock::now() - created_; }
   std::shared_ptr<SealedBlock> seal() { return std::make_shared<SealedBlock>(std::move(slots_)); }
   // Move every filled slot of `other` into this block (slots already filled
   // here are kept: a repeated slot is a duplicate, as in insert_slot).
@@ -150,7 +185,7 @@ class InflightBlock {
     Insert last = Insert::Duplicate;
     const size_t n = other.slots_.size() < slots_.size() ? other.slots_.size() : slots_.size();
     for (size_t i = 0; i < n; ++i) {
-      if (!other.filled_[i]) continue;
+      if (!other.filled(i)) continue;
       Insert r = insert_slot(i, std::move(other.slots_[i]));
       if (r == Insert::Completed) return r;
       if (r == Insert::Inserted) last = r;
@@ -159,10 +194,11 @@ class InflightBlock {
   }
 
  private:
+  // A slot that holds a block has at least one segment.
+  bool filled(size_t slot_id) const { return slots_[slot_id].num_segments() != 0; }
   std::vector<RawBlock> slots_;
-  std::vector<bool> filled_;
   size_t remaining_;
-  std::chrono::steady_clock::time_point created_;
+  Clock::time_point created_;
 };
 
 }  // namespace pf

@@ -186,7 +186,7 @@ Engine::~Engine() {
   leases_.clear();
   inflight_.clear();
   sealed_.clear();
-  lru_.clear();
+  lru_reset();
 }
 
 std::shared_ptr<InstanceContext> Engine::get_instance(const std::string& id, std::string* err) {
@@ -272,7 +272,8 @@ int Engine::register_context_layer_batch_strided(
       }
       instance = it->second;
     } else {
-      instance = std::make_shared<InstanceContext>(instance_id, ns, tp_size, world_size, page_first);
+      instance = std::make_shared<InstanceContext>(instance_id, ns, ns_id_locked(ns), tp_size,
+                                                   world_size, page_first);
       instances_[instance_id] = instance;
     }
   }
@@ -311,20 +312,42 @@ int Engine::unregister_instance(const std::string& instance_id, std::string* err
   return PF_OK;
 }
 
-void Engine::seal_insert(const BlockKey& key, std::shared_ptr<SealedBlock> block) {
-  // mu_ held by the caller; the key is not present.
-  lru_.push_back(key);
-  sealed_[key] = SealedEntry{std::move(block), std::prev(lru_.end())};
+uint32_t Engine::ns_id_locked(const std::string& ns) {
+  auto it = ns_ids_.find(ns);
+  if (it != ns_ids_.end()) return it->second;
+  const uint32_t id = static_cast<uint32_t>(ns_ids_.size());
+  ns_ids_.emplace(ns, id);
+  return id;
+}
+
+bool Engine::seal_insert(BlockKey&& key, std::shared_ptr<SealedBlock> block) {
+  auto [it, fresh] = sealed_.try_emplace(std::move(key));
+  if (!fresh) return false;
+  it->second.block = std::move(block);
+  it->second.key = &it->first;
+  lru_make_newest(&it->second);
+  return true;
+}
+
+Engine::SealedEntry* Engine::find_sealed(uint32_t ns, std::string_view hash, uint32_t group) {
+  SealedTable::iterator it;
+  if (group == 0) {
+    it = sealed_.find(BlockKeyView(ns, hash));
+  } else {
+    const std::string encoded = group_hash(std::string(hash), group);
+    it = sealed_.find(BlockKeyView(ns, encoded));
+  }
+  return it == sealed_.end() ? nullptr : &it->second;
 }
 
 bool Engine::evict_one() {
   // mu_ held by the caller.  Least recently used first; blocks that are
   // leased or being loaded (someone else holds a reference) stay.
-  for (auto it = lru_.begin(); it != lru_.end(); ++it) {
-    auto sit = sealed_.find(*it);
-    if (sit != sealed_.end() && sit->second.block.use_count() > 1) continue;
-    if (sit != sealed_.end()) sealed_.erase(sit);
-    lru_.erase(it);
+  for (SealedEntry* e = lru_.newer; e != &lru_; e = e->newer) {
+    if (e->block.use_count() > 1) continue;
+    lru_unlink(e);
+    auto it = sealed_.find(*e->key);
+    if (it != sealed_.end()) sealed_.erase(it);
     return true;
   }
   return false;
@@ -492,7 +515,7 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
   if (!instance) return PF_ERR_INSTANCE_MISSING;
   auto topo = instance->sealed_topology(err);
   if (!topo) return PF_ERR_INVALID_ARGUMENT;
-  const std::string ns = instance->ns();
+  const uint32_t ns = instance->ns_id();
 
   // ---- Phase 0: resolve metadata, bounds-check block ids ------------------
   auto gpu = instance->get_gpu(device_id);
@@ -573,15 +596,15 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
     for (SaveList& l : lists) {
       l.keys.reserve(l.n);
       for (size_t i = 0; i < l.n; ++i) {
-        l.keys.push_back(BlockKey{
+        l.keys.emplace_back(
             ns, group_hash(std::string(reinterpret_cast<const char*>(l.hashes[i]), l.lens[i]),
-                           l.group)});
+                           l.group));
       }
     }
     std::lock_guard<std::mutex> lock(mu_);
     for (SaveList& l : lists) {
       for (size_t i = 0; i < l.n; ++i) {
-        if (!sealed_.count(l.keys[i])) l.kept.push_back(static_cast<uint32_t>(i));
+        if (sealed_.find(l.keys[i]) == sealed_.end()) l.kept.push_back(static_cast<uint32_t>(i));
       }
       to_save += l.kept.size();
     }
@@ -686,7 +709,7 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
   std::future<TaskResult> pending = gpu->worker_pool->batch_save(std::move(gpu_layers));
 
   struct Assembled {
-    const BlockKey* key;
+    BlockKey* key;  // in its SaveList; moved into the store when the block is published
     InflightBlock block;
   };
   std::vector<Assembled> assembled;
@@ -695,7 +718,7 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
   if (!page_first) {
     assembled.reserve(to_save);
     for (size_t li = 0; li < lists.size() && prep_status == PF_OK; ++li) {
-      const SaveList& l = lists[li];
+      SaveList& l = lists[li];
       if (l.kept.empty()) continue;
       size_t total_slots = 0;
       std::string cause;
@@ -708,18 +731,21 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
       for (auto& ctx : ctxs) {
         if (ctx.list == li) members.push_back(&ctx);
       }
+      const auto created = Clock::now();
       for (size_t q = 0; q < l.kept.size() && prep_status == PF_OK; ++q) {
-        Assembled a{&l.keys[l.kept[q]], InflightBlock(total_slots)};
+        assembled.push_back(Assembled{&l.keys[l.kept[q]], InflightBlock(total_slots, created)});
+        InflightBlock& block = assembled.back().block;
         for (SaveLayerCtx* ctx : members) {
-          RawBlock raw;
-          if (!ctx->make_raw(q, cfg_.blockwise_alloc, &raw)) {
+          // Built in place; a slot named twice keeps its first block.
+          RawBlock* slot = block.empty_slot(ctx->slot_id);
+          if (slot == nullptr) continue;
+          if (!ctx->make_raw(q, cfg_.blockwise_alloc, slot)) {
             prep_status = PF_ERR_STORAGE;
             prep_err = "segment exceeds its pinned allocation";
             break;
           }
-          a.block.insert_slot(ctx->slot_id, std::move(raw));
+          block.slot_filled();
         }
-        assembled.push_back(std::move(a));
       }
     }
   }
@@ -734,9 +760,6 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
   t_phase = Clock::now();
   {
     std::lock_guard<std::mutex> lock(mu_);
-    auto seal = [&](const BlockKey& key, InflightBlock* b) {
-      seal_insert(key, b->seal());
-    };
     if (page_first) {
       const SaveList& l = lists[ctxs[0].list];
       const size_t slot_id = ctxs[0].slot_id;
@@ -746,10 +769,9 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
         Segment seg;
         Segment::create(pages[b]->as_ptr(), page_size, pages[b], &seg);
         // Page-first keys carry the raw hash (one group per shard page).
-        const std::string raw_hash(reinterpret_cast<const char*>(l.hashes[l.kept[b]]),
-                                   l.lens[l.kept[b]]);
-        BlockKey key{ns, raw_hash};
-        if (sealed_.count(key)) continue;
+        BlockKey key(ns, std::string(reinterpret_cast<const char*>(l.hashes[l.kept[b]]),
+                                     l.lens[l.kept[b]]));
+        if (sealed_.find(key) != sealed_.end()) continue;
         auto it = inflight_.find(key);
         if (it == inflight_.end()) {
           it = inflight_.emplace(key, InflightBlock(topo->total_slots())).first;
@@ -758,21 +780,25 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
         }
         if (it->second.insert_slot(slot_id, RawBlock::single_segment(std::move(seg))) ==
             InflightBlock::Insert::Completed) {
-          seal(key, &it->second);
+          auto sealed_block = it->second.seal();
           inflight_.erase(it);
+          seal_insert(std::move(key), std::move(sealed_block));
         }
       }
     } else {
       for (Assembled& a : assembled) {
-        const BlockKey& key = *a.key;
-        if (sealed_.count(key)) continue;
-        auto it = inflight_.find(key);
+        BlockKey& key = *a.key;
+        // Usually nothing is in flight and the save carries every slot of its
+        // blocks: one table operation per block.
+        auto it = inflight_.empty() ? inflight_.end() : inflight_.find(key);
         if (it == inflight_.end()) {
           if (a.block.complete()) {
-            seal(key, &a.block);
-          } else {
-            inflight_.emplace(key, std::move(a.block));
+            seal_insert(std::move(key), a.block.seal());  // no-op when sealed meanwhile
+          } else if (sealed_.find(key) == sealed_.end()) {
+            inflight_.emplace(std::move(key), std::move(a.block));
           }
+        } else if (sealed_.find(key) != sealed_.end()) {
+          continue;
         } else if (it->second.total_slots() != a.block.total_slots()) {
           // The block in flight was begun by an instance with another slot
           // count (a namespace shared by incompatible layouts): this save's
@@ -780,8 +806,9 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
           // (write_path.rs:147-165).
           continue;
         } else if (it->second.absorb(std::move(a.block)) == InflightBlock::Insert::Completed) {
-          seal(key, &it->second);
+          auto sealed_block = it->second.seal();
           inflight_.erase(it);
+          seal_insert(std::move(key), std::move(sealed_block));
         }
       }
     }
@@ -797,7 +824,7 @@ int Engine::batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank,
 }
 
 int Engine::query_group_membership(const std::string& instance_id, uint32_t group,
-                                   const std::vector<std::string>& hashes,
+                                   const std::vector<std::string_view>& hashes,
                                    std::vector<uint8_t>* present, std::string* err) {
   auto instance = get_instance(instance_id, err);
   if (!instance) return PF_ERR_INSTANCE_MISSING;
@@ -809,13 +836,13 @@ int Engine::query_group_membership(const std::string& instance_id, uint32_t grou
   present->assign(hashes.size(), 0);
   std::lock_guard<std::mutex> lock(mu_);
   for (size_t i = 0; i < hashes.size(); ++i) {
-    (*present)[i] = sealed_.count(BlockKey{instance->ns(), group_hash(hashes[i], group)}) ? 1 : 0;
+    (*present)[i] = find_sealed(instance->ns_id(), hashes[i], group) != nullptr ? 1 : 0;
   }
   return PF_OK;
 }
 
 int Engine::create_group_lease(const std::string& instance_id, uint32_t group,
-                               const std::vector<std::string>& hashes, uint64_t* out_lease,
+                               const std::vector<std::string_view>& hashes, uint64_t* out_lease,
                                std::string* err) {
   auto instance = get_instance(instance_id, err);
   if (!instance) return PF_ERR_INSTANCE_MISSING;
@@ -833,15 +860,16 @@ int Engine::create_group_lease(const std::string& instance_id, uint32_t group,
   lease.instance_id = instance_id;
   lease.remaining_consumers = std::max<size_t>(instance->world_size(), 1);
   lease.expires_at = lease_deadline();
+  lease.blocks.reserve(hashes.size());
   for (size_t i = 0; i < hashes.size(); ++i) {
-    auto it = sealed_.find(BlockKey{instance->ns(), group_hash(hashes[i], group)});
-    if (it == sealed_.end()) {
+    SealedEntry* hit = find_sealed(instance->ns_id(), hashes[i], group);
+    if (hit == nullptr) {
       return bad(err, PF_ERR_STORAGE,
                  "block " + std::to_string(i) + " of the lease is not resident in group " +
                      std::to_string(group));
     }
-    lease.blocks.push_back(it->second.block);
-    lru_.splice(lru_.end(), lru_, it->second.pos);
+    lease.blocks.push_back(hit->block);
+    lru_touch(hit);
   }
   *out_lease = next_lease_++;
   leases_[*out_lease] = std::move(lease);
@@ -853,7 +881,8 @@ SaveProfile Engine::last_save_profile() {
   return last_save_profile_;
 }
 
-int Engine::query_prefix(const std::string& instance_id, const std::vector<std::string>& hashes,
+int Engine::query_prefix(const std::string& instance_id,
+                         const std::vector<std::string_view>& hashes,
                          uint64_t* out_hits, uint64_t* out_lease, std::string* err) {
   auto instance = get_instance(instance_id, err);
   if (!instance) return PF_ERR_INSTANCE_MISSING;
@@ -863,11 +892,12 @@ int Engine::query_prefix(const std::string& instance_id, const std::vector<std::
   lease.instance_id = instance_id;
   lease.remaining_consumers = std::max<size_t>(instance->world_size(), 1);
   lease.expires_at = lease_deadline();
-  for (const std::string& h : hashes) {
-    auto it = sealed_.find(BlockKey{instance->ns(), h});
-    if (it == sealed_.end()) break;
-    lease.blocks.push_back(it->second.block);
-    lru_.splice(lru_.end(), lru_, it->second.pos);  // most recently used
+  lease.blocks.reserve(hashes.size());
+  for (std::string_view h : hashes) {
+    SealedEntry* hit = find_sealed(instance->ns_id(), h, 0);
+    if (hit == nullptr) break;
+    lease.blocks.push_back(hit->block);
+    lru_touch(hit);  // most recently used
   }
   *out_hits = lease.blocks.size();
   *out_lease = 0;
@@ -986,7 +1016,8 @@ int Engine::batch_load_kv_blocks_multi_layer(
         if (ids[si] >= 0) targets[gi].emplace_back(static_cast<uint64_t>(ids[si]), start + si);
       }
     }
-    block_cache.insert(block_cache.end(), blocks.begin(), blocks.end());
+    block_cache.insert(block_cache.end(), std::make_move_iterator(blocks.begin()),
+                       std::make_move_iterator(blocks.end()));
   }
   // One LayerTransferData per layer.
   struct PageList {
@@ -1074,7 +1105,7 @@ int Engine::batch_load_kv_blocks_multi_layer(
   // The leased blocks stay alive through the first layer of the task.
   if (!layers.empty()) {
     layers.front().keep.reserve(block_cache.size());
-    for (auto& b : block_cache) layers.front().keep.push_back(b);
+    for (auto& b : block_cache) layers.front().keep.push_back(std::move(b));
   }
   if (layers.empty()) {
     // Nothing to load: complete at once (lib.rs:885-890).

@@ -12,6 +12,7 @@
 #include <future>
 #include <list>
 #include <map>
+#include <unordered_map>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -71,10 +72,10 @@ struct GpuContext {
 // instance.rs:380-478,680-860.
 class InstanceContext {
  public:
-  InstanceContext(std::string id, std::string ns, size_t tp_size, size_t world_size,
-                  bool page_first)
-      : id_(std::move(id)), ns_(std::move(ns)), tp_size_(tp_size), world_size_(world_size),
-        page_first_(page_first) {}
+  InstanceContext(std::string id, std::string ns, uint32_t ns_id, size_t tp_size,
+                  size_t world_size, bool page_first)
+      : id_(std::move(id)), ns_(std::move(ns)), ns_id_(ns_id), tp_size_(tp_size),
+        world_size_(world_size), page_first_(page_first) {}
   int register_new_gpu(std::shared_ptr<GpuContext> ctx, std::string* err);
   // Fails while workers are still registering.
   std::shared_ptr<LayerTopology> sealed_topology(std::string* err);
@@ -82,6 +83,8 @@ class InstanceContext {
   std::string verify_topology(size_t tp_size, size_t world_size, bool page_first) const;
   const std::string& id() const { return id_; }
   const std::string& ns() const { return ns_; }
+  // The engine's number for the namespace: what block keys carry.
+  uint32_t ns_id() const { return ns_id_; }
   size_t tp_size() const { return tp_size_; }
   size_t world_size() const { return world_size_; }
   // Validation that must precede the (expensive) GPU context construction.
@@ -89,6 +92,7 @@ class InstanceContext {
 
  private:
   std::string id_, ns_;
+  uint32_t ns_id_;
   size_t tp_size_, world_size_;
   bool page_first_;
   std::mutex mu_;
@@ -119,18 +123,19 @@ class Engine {
   SaveProfile last_save_profile();
   // Longest cached prefix of `hashes` (group 0 keys) + a lease over those
   // blocks (lib.rs:506-546,614-629).
-  int query_prefix(const std::string& instance_id, const std::vector<std::string>& hashes,
+  int query_prefix(const std::string& instance_id, const std::vector<std::string_view>& hashes,
                    uint64_t* out_hits, uint64_t* out_lease, std::string* err);
   // lib.rs:593-611: per-position membership of `hashes` in one storage group
   // (no prefix rule, no lease).  An unknown group is an error.
   int query_group_membership(const std::string& instance_id, uint32_t group,
-                             const std::vector<std::string>& hashes, std::vector<uint8_t>* present,
+                             const std::vector<std::string_view>& hashes,
+                             std::vector<uint8_t>* present,
                              std::string* err);
   // lib.rs:614-628 over hashes instead of block handles: a lease that pins the
   // sealed blocks of exactly these hashes in `group`.  Fails when one of them
   // is not resident (it may have been evicted since the membership query).
   int create_group_lease(const std::string& instance_id, uint32_t group,
-                         const std::vector<std::string>& hashes, uint64_t* out_lease,
+                         const std::vector<std::string_view>& hashes, uint64_t* out_lease,
                          std::string* err);
   bool release_query_lease(uint64_t lease);
   // The periodic sweep of the reference's lease manager (lease.rs:66-80), for
@@ -155,7 +160,7 @@ class Engine {
   size_t evict_all();
 
  private:
-  Engine() = default;
+  Engine() { lru_reset(); }
   std::shared_ptr<InstanceContext> get_instance(const std::string& id, std::string* err);
   // storage/mod.rs:294-330: allocate, evicting oldest sealed blocks on pressure.
   std::shared_ptr<PinnedAllocation> allocate(uint64_t size, NumaNode numa);
@@ -169,17 +174,44 @@ class Engine {
   NumaTopology numa_;
   std::mutex mu_;  // instances, store, leases
   std::map<std::string, std::shared_ptr<InstanceContext>> instances_;
-  std::map<BlockKey, InflightBlock> inflight_;
-  // The read cache: sealed blocks in least-recently-used order (front = next
-  // to go; a prefix query moves its hits to the back), storage/mod.rs:482-554
-  // and storage/read_cache.rs of the reference without its admission policy.
+  std::map<std::string, uint32_t> ns_ids_;  // namespace name -> the number in block keys
+  uint32_t ns_id_locked(const std::string& ns);
+  std::unordered_map<BlockKey, InflightBlock, BlockKeyHash, BlockKeyEqual> inflight_;
+  // The read cache: sealed blocks in least-recently-used order (a prefix query
+  // makes its hits the most recently used), storage/mod.rs:482-554 and
+  // storage/read_cache.rs of the reference without its admission policy.  The
+  // order is a ring threaded through the table's own entries (their addresses
+  // do not change while they are in the table), so making a block the most
+  // recently used touches no allocator.
   struct SealedEntry {
     std::shared_ptr<SealedBlock> block;
-    std::list<BlockKey>::iterator pos;
+    const BlockKey* key = nullptr;  // the table's copy of the key
+    SealedEntry* older = nullptr;
+    SealedEntry* newer = nullptr;
   };
-  std::map<BlockKey, SealedEntry> sealed_;
-  std::list<BlockKey> lru_;
-  void seal_insert(const BlockKey& key, std::shared_ptr<SealedBlock> block);
+  using SealedTable = std::unordered_map<BlockKey, SealedEntry, BlockKeyHash, BlockKeyEqual>;
+  SealedTable sealed_;
+  // Ring head: lru_.newer is the least recently used entry, lru_.older the most.
+  SealedEntry lru_;
+  void lru_reset() { lru_.older = lru_.newer = &lru_; }
+  static void lru_unlink(SealedEntry* e) {
+    e->older->newer = e->newer;
+    e->newer->older = e->older;
+  }
+  void lru_make_newest(SealedEntry* e) {
+    e->older = lru_.older;
+    e->newer = &lru_;
+    lru_.older->newer = e;
+    lru_.older = e;
+  }
+  void lru_touch(SealedEntry* e) {
+    lru_unlink(e);
+    lru_make_newest(e);
+  }
+  // The sealed entry of (namespace, group-encoded hash), or null; mu_ held.
+  SealedEntry* find_sealed(uint32_t ns, std::string_view hash, uint32_t group);
+  // Enters a block under `key` unless the key is sealed already; mu_ held.
+  bool seal_insert(BlockKey&& key, std::shared_ptr<SealedBlock> block);
   // lease.rs:40-134: a lease serves one load per worker of the instance's
   // world size, then disappears.
   struct Lease {

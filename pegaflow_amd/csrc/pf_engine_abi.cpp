@@ -96,10 +96,6 @@ bool BorrowedBlocks::build(const pf_layer_transfer* layers, uint64_t n_layers,
   return true;
 }
 
-std::string hash_of(const uint8_t* p, uint32_t len) {
-  return std::string(reinterpret_cast<const char*>(p), len);
-}
-
 }  // namespace
 
 extern "C" {
@@ -381,8 +377,11 @@ int pf_engine_query_prefix(pf_engine_t e, const char* instance_id, const uint8_t
   PF_REQUIRE_PTR(instance_id);
   PF_REQUIRE_PTR(out_hits);
   PF_REQUIRE_PTR(out_lease);
-  std::vector<std::string> h;
-  for (uint64_t i = 0; i < n; ++i) h.push_back(hash_of(hashes[i], hash_lens[i]));
+  std::vector<std::string_view> h;
+  h.reserve(n);
+  for (uint64_t i = 0; i < n; ++i) {
+    h.emplace_back(reinterpret_cast<const char*>(hashes[i]), hash_lens[i]);
+  }
   std::string err;
   int st = reinterpret_cast<pf::Engine*>(e)->query_prefix(instance_id, h, out_hits, out_lease, &err);
   if (st != PF_OK) pf::last_error() = err;
@@ -486,8 +485,11 @@ int pf_engine_query_group_membership(pf_engine_t e, const char* instance_id, uin
     PF_REQUIRE_PTR(hash_lens);
     PF_REQUIRE_PTR(out_present);
   }
-  std::vector<std::string> h;
-  for (uint64_t i = 0; i < n; ++i) h.push_back(hash_of(hashes[i], hash_lens[i]));
+  std::vector<std::string_view> h;
+  h.reserve(n);
+  for (uint64_t i = 0; i < n; ++i) {
+    h.emplace_back(reinterpret_cast<const char*>(hashes[i]), hash_lens[i]);
+  }
   std::vector<uint8_t> present;
   std::string err;
   int st = reinterpret_cast<pf::Engine*>(e)->query_group_membership(instance_id, group, h, &present,
@@ -510,8 +512,11 @@ int pf_engine_create_group_lease(pf_engine_t e, const char* instance_id, uint32_
     PF_REQUIRE_PTR(hashes);
     PF_REQUIRE_PTR(hash_lens);
   }
-  std::vector<std::string> h;
-  for (uint64_t i = 0; i < n; ++i) h.push_back(hash_of(hashes[i], hash_lens[i]));
+  std::vector<std::string_view> h;
+  h.reserve(n);
+  for (uint64_t i = 0; i < n; ++i) {
+    h.emplace_back(reinterpret_cast<const char*>(hashes[i]), hash_lens[i]);
+  }
   std::string err;
   int st = reinterpret_cast<pf::Engine*>(e)->create_group_lease(instance_id, group, h, out_lease,
                                                                 &err);
