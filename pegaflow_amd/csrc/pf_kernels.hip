@@ -125,15 +125,27 @@ __device__ __forceinline__ void copy_tile_any(uint64_t dst, uint64_t src, uint32
 
 // Descriptor-table copy: table[3i..3i+2] = dst, src, size.  blockIdx.x strides
 // over descriptors, blockIdx.y over the tiles inside one descriptor, so a
-// batch of few large copies still spreads over the whole chip.
+// batch of few large copies still spreads over the whole chip.  The row a
+// workgroup handles next is fetched before the current one is copied: the
+// table may sit in mapped host memory (short batches skip the upload), where
+// a row is a couple of microseconds away.
 template <int U>
 __global__ __launch_bounds__(kLanes) void desc_copy_kernel(const uint64_t* __restrict__ table,
                                                            uint32_t n) {
   constexpr uint64_t kTile = static_cast<uint64_t>(U) * kLanes * 16;
-  for (uint32_t i = blockIdx.x; i < n; i += gridDim.x) {
-    const uint64_t dst = table[3ull * i + 0];
-    const uint64_t src = table[3ull * i + 1];
-    const uint64_t size = table[3ull * i + 2];
+  uint32_t i = blockIdx.x;
+  if (i >= n) return;
+  uint64_t dst = table[3ull * i + 0];
+  uint64_t src = table[3ull * i + 1];
+  uint64_t size = table[3ull * i + 2];
+  for (;;) {
+    const uint32_t next = i + gridDim.x;
+    uint64_t next_dst = 0, next_src = 0, next_size = 0;
+    if (next < n) {
+      next_dst = table[3ull * next + 0];
+      next_src = table[3ull * next + 1];
+      next_size = table[3ull * next + 2];
+    }
     const uint64_t n_tiles = (size + kTile - 1) / kTile;
     const bool vec = ((dst | src) & 15ull) == 0;
     for (uint64_t t = blockIdx.y; t < n_tiles; t += gridDim.y) {
@@ -146,6 +158,11 @@ __global__ __launch_bounds__(kLanes) void desc_copy_kernel(const uint64_t* __res
         copy_tile_any(dst + off, src + off, bytes);
       }
     }
+    if (next >= n) break;
+    i = next;
+    dst = next_dst;
+    src = next_src;
+    size = next_size;
   }
 }
 

@@ -160,6 +160,9 @@ int SlabPool::release_after(Slab* slab, hipStream_t s) {
   return PF_OK;
 }
 
+// Descriptor tables up to this size (4096 rows) are left in mapped host memory.
+constexpr uint64_t kHostTableBytes = 96 * 1024;
+
 // ---------------------------------------------------------------------------
 // MemcpyBackend
 // ---------------------------------------------------------------------------
@@ -393,8 +396,17 @@ int MemcpyBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_
       ++row;
     }
   }
-  PF_HIP(hipMemcpyAsync(slab->dev, slab->host, table_rows * 3 * sizeof(uint64_t),
-                        hipMemcpyHostToDevice, s));
+  // A short table of ranges that all go through the mapped-memory kernel is
+  // read where it was written (see KernelBackend::submit_impl); tables of
+  // packing launches stay in device memory, where the HBM-rate kernels read them.
+  if (staged_pieces == 0 && table_rows * 3 * sizeof(uint64_t) <= kHostTableBytes) {
+    void* alias = nullptr;
+    PF_HIP(hipHostGetDevicePointer(&alias, slab->host, 0));
+    table_dev = static_cast<const uint64_t*>(alias);
+  } else {
+    PF_HIP(hipMemcpyAsync(slab->dev, slab->host, table_rows * 3 * sizeof(uint64_t),
+                          hipMemcpyHostToDevice, s));
+  }
   row = 0;
   if (isolated_by_kernel) {
     st = launch_desc_copy(table_dev, isolated.size(), max_isolated, s,
@@ -464,9 +476,18 @@ int KernelBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_
     table[3 * i + 2] = c.size;
     max_size = std::max<uint64_t>(max_size, c.size);
   }
-  PF_HIP(hipMemcpyAsync(slab->dev, slab->host, bytes, hipMemcpyHostToDevice, s));
-  st = launch_desc_copy(static_cast<const uint64_t*>(slab->dev), n, max_size, s,
-                        host_link_workgroups(total_size, n));
+  // A short table is read where it was written, in mapped host memory: the
+  // upload would cost more than the rows' trip over the link, which the kernel
+  // hides behind the copy of the row before.
+  const uint64_t* table_dev = static_cast<const uint64_t*>(slab->dev);
+  if (bytes <= kHostTableBytes) {
+    void* alias = nullptr;
+    PF_HIP(hipHostGetDevicePointer(&alias, slab->host, 0));
+    table_dev = static_cast<const uint64_t*>(alias);
+  } else {
+    PF_HIP(hipMemcpyAsync(slab->dev, slab->host, bytes, hipMemcpyHostToDevice, s));
+  }
+  st = launch_desc_copy(table_dev, n, max_size, s, host_link_workgroups(total_size, n));
   if (st != PF_OK) return st;
   return slabs_.release_after(slab, s);
 }
