@@ -93,6 +93,9 @@ def main():
 
     cold = query(inst, hs, "mock-vllm-cold-query")
     out["cold_query"] = [cold[0], cold[1], len(cold[2])]
+    # python/tests/test_engine_client.py:20-44: a query without hashes is Ready(0) with no lease as well
+    empty = query(inst, [], "query-contract-empty_query")
+    out["empty_query"] = [empty[0], empty[1], empty[2] == b""]
     out["save"] = list(save(inst, hs))
     kind, hits, lease, _ = query(inst, hs, "mock-vllm-hit-query")
     out["hit_query"] = [kind, hits, len(lease)]

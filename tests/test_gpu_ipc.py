@@ -108,9 +108,9 @@ def test_save_and_load_of_another_process_caches(gpu, mode):
         state = LoadState(attach_to=zeroed["shm"])
         engine.batch_load_kv_blocks_multi_layer("ipc-inst", 0, 0, [names], lease,
                                                 [dst_ids.tolist()], state).wait()
-        verdict = worker.ask(op="await", src_ids=src_ids.tolist(), dst_ids=dst_ids.tolist())
-        assert verdict["state"] == 1, verdict
-        assert verdict["ok"], verdict["problems"]
+        answer = worker.ask(op="await", src_ids=src_ids.tolist(), dst_ids=dst_ids.tolist())
+        assert answer["state"] == 1, answer
+        assert answer["ok"], answer["problems"]
         state.close()
 
         # registry.rs:73-77: the same context cannot be registered twice

@@ -65,6 +65,7 @@ def test_reference_rpc_scenarios(gpu):
         # :26-77 save / query / load round trip
         assert out["register"] == ok and out["save"] == ok
         assert out["cold_query"] == ["QueryReady", 0, 0]
+        assert out["empty_query"] == ["QueryReady", 0, True]
         assert out["hit_query"] == ["QueryReady", 4, 16]
         assert out["load"] == [ok, 1] and out["roundtrip_matches"]
         # :79-96
