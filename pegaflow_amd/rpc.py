@@ -433,7 +433,9 @@ class EngineService:
 
 def serve(engine: PegaEngine, address: str = DEFAULT_ENDPOINT, registry: TensorRegistry | None = None,
           max_workers: int = 32):
-    """Start a server; returns (grpc.Server, EngineService, bound port)."""
+    """Start a server; returns (grpc.Server, EngineService, bound port).  An open
+    Session occupies one of the `max_workers` threads for as long as it lasts,
+    so keep `max_workers` well above the number of worker processes."""
     service = EngineService(engine, registry)
     server = grpc.server(futures.ThreadPoolExecutor(max_workers=max_workers),
                          options=[("grpc.max_receive_message_length", 256 << 20),
