@@ -173,10 +173,20 @@ template <int U, bool HOST_IS_SRC>
 __global__ __launch_bounds__(kLanes) void desc48_copy_kernel(
     const pf_copy_desc* __restrict__ table, uint32_t n) {
   constexpr uint64_t kTile = static_cast<uint64_t>(U) * kLanes * 16;
-  for (uint32_t i = blockIdx.x; i < n; i += gridDim.x) {
-    const uint64_t near_addr = table[i].device;
-    const uint64_t far_addr = table[i].host_device;
-    const uint64_t size = table[i].size;
+  uint32_t i = blockIdx.x;
+  if (i >= n) return;
+  uint64_t near_addr = table[i].device;
+  uint64_t far_addr = table[i].host_device;
+  uint64_t size = table[i].size;
+  for (;;) {
+    // The next row is on its way while this one is copied.
+    const uint32_t next = i + gridDim.x;
+    uint64_t next_near = 0, next_far = 0, next_size = 0;
+    if (next < n) {
+      next_near = table[next].device;
+      next_far = table[next].host_device;
+      next_size = table[next].size;
+    }
     const uint64_t dst = HOST_IS_SRC ? near_addr : far_addr;
     const uint64_t src = HOST_IS_SRC ? far_addr : near_addr;
     const uint64_t n_tiles = (size + kTile - 1) / kTile;
@@ -191,6 +201,11 @@ __global__ __launch_bounds__(kLanes) void desc48_copy_kernel(
         copy_tile_any(dst + off, src + off, bytes);
       }
     }
+    if (next >= n) break;
+    i = next;
+    near_addr = next_near;
+    far_addr = next_far;
+    size = next_size;
   }
 }
 
