@@ -424,7 +424,13 @@ int MemcpyBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_
       PF_HIP(hipMemcpyHtoDAsync(reinterpret_cast<hipDeviceptr_t>(in_staging), run.host_begin,
                                 run.bytes, s));
     }
-    st = launch_desc_copy(table_dev + 3 * row, run.members.size(), max_staged_piece, s);
+    // Many pieces of at most one tile: two rows per workgroup, so that the second
+    // row's descriptor is on its way while the first is copied (65 536 pieces of
+    // 4 KiB: 92 us instead of 98).
+    const uint64_t pieces = run.members.size();
+    const uint32_t pack_workgroups =
+        max_staged_piece <= 16384 && pieces >= 8192 ? static_cast<uint32_t>((pieces + 1) / 2) : 0;
+    st = launch_desc_copy(table_dev + 3 * row, pieces, max_staged_piece, s, pack_workgroups);
     if (st != PF_OK) return st;
     if (!host_is_src) {
       PF_HIP(hipMemcpyDtoHAsync(run.host_begin, reinterpret_cast<hipDeviceptr_t>(in_staging),
