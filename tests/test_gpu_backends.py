@@ -115,10 +115,13 @@ def test_unaligned_and_odd_sizes_match_oracle(backends, stream, direction):
     host.close()
 
 
-def test_shuffled_4k_fragments(backends, stream):
+@pytest.mark.parametrize("n", [4096, 16385])
+def test_shuffled_4k_fragments(backends, stream, n):
     """Shape of the reference's transfer bench (benches/transfer_h2d.rs):
-    4096-byte fragments in a seeded shuffled order, device strided by two."""
-    seg, n = 4096, 4096
+    4096-byte fragments in a seeded shuffled order, device strided by two.
+    The larger, odd count makes the direct backend's packing launch take two
+    fragments per workgroup with one left over."""
+    seg = 4096
     perm = xorshift_shuffle(n)
     assert sorted(perm) == list(range(n))
     rng = np.random.default_rng(3)
