@@ -647,26 +647,30 @@ def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_
 
     ticks = []   # (GEMMs launched so far, event on the GEMM stream), one per 64 GEMMs
 
-    def gemms(count, tick_pool=None, until=None):
+    def gemms(count, tick_pool=None, until=None, start=0):
         """Launch `count` GEMMs; with `until` (an event on another stream), keep
         launching in groups of 64 after that until the event has completed, so
-        that the GEMM stream stays busy for as long as that work takes.
-        Returns the number launched."""
-        del ticks[:]
-        launched = 0
+        that the GEMM stream stays busy for as long as that work takes.  `start`
+        continues the numbering (and the marks) of an earlier call.
+        Returns the number launched by this call."""
+        if start == 0:
+            del ticks[:]
+        launched = start
+        first = True
         with torch.cuda.stream(gemm_stream):
             g0.record()
             while True:
-                for _ in range(count if launched == 0 else 64):
+                for _ in range(count if first else 64):
                     torch.matmul(a, b, out=c)
                     launched += 1
                     if tick_pool is not None and launched % 64 == 0 and launched // 64 <= len(tick_pool):
                         tick_pool[launched // 64 - 1].record(gemm_native)
                         ticks.append((launched, tick_pool[launched // 64 - 1]))
+                first = False
                 if until is None or until.query() or launched > 60000:
                     break
             g1.record()
-        return launched
+        return launched - start
 
     gemms(50)
     torch.cuda.synchronize()
@@ -697,11 +701,11 @@ def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_
         # until the transfer's end event has completed: the GEMM stream is busy
         # from before the transfer starts until after it ends.
         m0.record(gemm_native)
-        gemms(1000)
+        backlog = gemms(960, tick_pool)           # 15 marks before and into the transfer
         e0.record(stream)
         fn(layers, stream, path)
         e1.record(stream)
-        count = gemms(64, tick_pool, until=e1)    # the GEMMs launched after the transfer call
+        count = gemms(64, tick_pool, until=e1, start=backlog)  # those launched after the call
         m1.record(gemm_native)
         e1.synchronize()
         torch.cuda.synchronize()
@@ -723,7 +727,16 @@ def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_
             during_ms = (inside[-1][1] - inside[0][1]) / (inside[-1][0] - inside[0][0])
             out[f"gemm_with_{name}_tflops"] = round(flop / (during_ms / 1e3) / 1e12, 1)
         else:
+            # Fewer than two marks inside: the GEMM stream all but stood still.  The
+            # GEMMs between the last mark before the transfer and the first after it
+            # bound what it did meanwhile.
             out[f"gemm_with_{name}_tflops"] = None
+            marks = [(k, m0.elapsed_ms(ev)) for k, ev in ticks]
+            before = [m for m in marks if m[1] < begin]
+            after = [m for m in marks if m[1] > end]
+            if before and after:
+                out[f"gemm_with_{name}_tflops_at_most"] = round(
+                    flop * (after[0][0] - before[-1][0]) / ((end - begin) / 1e3) / 1e12, 1)
         out[f"gemm_stream_with_{name}_tflops_whole_run"] = round(
             flop / (g0.elapsed_time(g1) / count / 1e3) / 1e12, 1)
         out[f"{name}_alone_gbps"] = round(payload / (alone_ms / 1e3) / 1e9, 2)
