@@ -408,6 +408,17 @@ def main():
     achieved = alg_bytes / (live_launch_ms / 1e3) / 1e9
     traffic, traffic_source = (measured_traffic(args.workload, alg_bytes) if staged_path
                                else (None, "zero-copy launches are not profiled for HBM traffic"))
+    # What a pair of events reads with nothing between them on that stream: the
+    # part of avg_launch_us that is the bracket itself, not the kernel (reported,
+    # not subtracted).
+    pair = [Event(timing=True), Event(timing=True)]
+    empty_pair_us = []
+    for _ in range(50):
+        pair[0].record(stream)
+        pair[1].record(stream)
+        pair[1].synchronize()
+        empty_pair_us.append(pair[0].elapsed_ms(pair[1]) * 1e3)
+    empty_pair_us.sort()
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                 "traffic": traffic, "traffic_source": traffic_source,
@@ -416,6 +427,7 @@ def main():
                 "measured": f"HIP events around each of the {live['launches']} launches of the "
                             f"{args.steps} timed steps",
                 "launches": launches, "avg_launch_us": round(live_launch_ms * 1e3, 2),
+                "empty_event_pair_us": round(empty_pair_us[len(empty_pair_us) // 2], 2),
                 "alg_bytes_per_launch": int(alg_bytes),
                 "launches_alone": {
                     "avg_launch_us": round(alone_launch_ms * 1e3, 2),
