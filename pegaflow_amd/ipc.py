@@ -90,14 +90,17 @@ class HipIPCWrapper:
             raise ValueError("not a HipIPCWrapper record")
         if len(data) != _FIXED.size + n:
             raise ValueError("IPC record has a truncated metadata tail")
-        meta = json.loads(data[_FIXED.size:].decode())
         self = cls.__new__(cls)
         self.handle, self.alloc_size, self.offset, self.size_bytes = handle, alloc_size, offset, size
         self.device_uuid = uuid
-        self.dtype = str(meta["dtype"])
-        self.shape = tuple(int(x) for x in meta["shape"])
-        self.stride = tuple(int(x) for x in meta["stride"])
-        self.storage_offset = int(meta.get("storage_offset", 0))
+        try:
+            meta = json.loads(data[_FIXED.size:].decode())
+            self.dtype = str(meta["dtype"])
+            self.shape = tuple(int(x) for x in meta["shape"])
+            self.stride = tuple(int(x) for x in meta["stride"])
+            self.storage_offset = int(meta.get("storage_offset", 0))
+        except (KeyError, TypeError, AttributeError, UnicodeDecodeError, ValueError) as exc:
+            raise ValueError(f"IPC record has a malformed metadata tail: {exc}") from None
         return self
 
     def c_record(self) -> "_lib.PfIpcTensor":
