@@ -270,6 +270,11 @@ class EngineService:
                              exc.message if exc.message.startswith("register tensor failed")
                              else f"register tensor failed: {exc.message}")
             raise _map_engine_error(exc)
+        except ValueError as exc:
+            # a wrapper that cannot be read (engine errors, some of which are
+            # ValueErrors too, are handled above): the reference fails to
+            # unpickle it and answers INTERNAL (service.rs:286-296)
+            raise _Abort(grpc.StatusCode.INTERNAL, f"register tensor failed: {exc}")
         return RegisterContextResponse(status=_ok())
 
     # -- Save (service.rs:360-437) ------------------------------------------

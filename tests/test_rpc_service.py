@@ -130,6 +130,10 @@ def test_register_validation_codes(served):
         ("INVALID_ARGUMENT", "tp_rank 1 out of range (tp_size 1)")
     code, text = _rejected(lambda: client.register_context_batch(**{**args, "num_blocks_list": []}))
     assert code == "INVALID_ARGUMENT" and "same non-zero length" in text
+    # a wrapper the server cannot read is its own failure class, as a failed unpickle is
+    with pytest.raises(rpc.PegaFlowError) as err:
+        client.register_context_batch(**args)
+    assert err.value.code == "INTERNAL" and "register tensor failed" in str(err.value)
     # a client of another release is refused before anything is touched (service.rs:212-222)
     service.version = "9.9.9"
     code, text = _rejected(lambda: client.register_context_batch(**args))
