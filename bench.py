@@ -107,6 +107,8 @@ def parse_args():
                     help="staged path: 0 default, 1 link copies on a side stream, 2 in order on "
                          "the caller's stream (kernels then never overlap a copy)")
     ap.add_argument("--no-overlap", action="store_true", help="skip the GEMM-overlap section")
+    ap.add_argument("--gemm-m", type=int, default=4096,
+                    help="edge of the square bf16 GEMMs of the overlap section (BASELINE: 4096)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-engine", action="store_true", help="skip the save/query/load engine section")
     ap.add_argument("--engine-mode", choices=["direct", "kernel", "zerocopy"], default="direct",
@@ -467,7 +469,7 @@ def main():
     overlap = None
     if not args.no_overlap:
         overlap = run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_layers,
-                              checker, pool)
+                              checker, pool, m=args.gemm_m)
 
     # ---- both directions at once (the worker pool runs a load thread and a
     # save thread per GPU: gpu_worker.rs:116-345 of the reference) ----------
@@ -640,14 +642,13 @@ class ByteChecker:
 
 
 def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_layers, checker,
-                pool):
+                pool, m=4096):
     """Transfer alone, GEMM stream alone, then both at once (load and save).
     The pass that runs next to the GEMM stream starts from a cleared target and
     is byte-checked on every layer; the GEMM's result is compared with the one
     it gives alone."""
     from pegaflow_amd.runtime import Event, Stream
     dev = torch.device("cuda:0")
-    m = 4096
     a = torch.randn(m, m, device=dev, dtype=torch.bfloat16)
     b = torch.randn(m, m, device=dev, dtype=torch.bfloat16)
     c = torch.empty(m, m, device=dev, dtype=torch.bfloat16)
@@ -693,7 +694,7 @@ def run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_
     m0, m1 = Event(timing=True), Event(timing=True)
     tick_pool = [Event(timing=True) for _ in range(1024)]
     c_alone = c.clone()
-    out = {"gemm": "4096x4096x4096 bf16, back to back on its own stream",
+    out = {"gemm": f"{m}x{m}x{m} bf16, back to back on its own stream",
            "gemm_alone_tflops": round(flop / (gemm_alone_ms / 1e3) / 1e12, 1)}
     gemm_ok = True
     for name, fn, layers in (("load", xfer.load, load_layers), ("save", xfer.save, save_layers)):

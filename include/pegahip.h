@@ -584,6 +584,10 @@ typedef struct pf_engine_config {
   uint32_t use_descriptor_backends;  /* see pf_worker_pool_spawn */
   uint64_t unit_size_hint;
   uint64_t lease_ttl_ms;             /* lease.rs:11: 0 = default (600 000 ms) */
+  uint64_t auto_staged_min_bytes;    /* workers: smallest dense transfer that is staged instead of
+                                        moved by the resident zero-copy kernel; 0 = default (16 MiB per layer).
+                                        Lower it where short model kernels run beside the transfers:
+                                        a resident copy kernel costs them far more than a staged copy. */
 } pf_engine_config;
 
 typedef struct pf_layer_save {       /* LayerSave, block.rs:20-25 */

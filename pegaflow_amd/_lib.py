@@ -121,7 +121,7 @@ class PfEngineConfig(C.Structure):
     _fields_ = [("pool_size", u64), ("use_hugepages", u32), ("numa_aware", u32),
                 ("pool_shards", u32), ("blockwise_alloc", u32), ("ssd_enabled", u32),
                 ("use_descriptor_backends", u32), ("unit_size_hint", u64),
-                ("lease_ttl_ms", u64)]
+                ("lease_ttl_ms", u64), ("auto_staged_min_bytes", u64)]
 
 
 class PfIpcTensor(C.Structure):

@@ -289,7 +289,8 @@ int Engine::register_context_layer_batch_strided(
   std::string werr;
   int wstatus = PF_ERR_DEVICE_INIT;
   ctx->worker_pool = GpuWorkerPool::spawn(device_id, ctx->preferred_numa, mode,
-                                          cfg_.use_descriptor_backends, &werr, &wstatus);
+                                          cfg_.use_descriptor_backends, &werr, &wstatus,
+                                          cfg_.auto_staged_min_bytes);
   if (!ctx->worker_pool) return bad(err, wstatus, werr);
   return instance->register_new_gpu(std::move(ctx), err);
 }

@@ -36,6 +36,8 @@ struct EngineConfig {
   uint64_t unit_size_hint = 0;
   // lease.rs:11: a lease that nobody consumes stops pinning its blocks after this long.
   uint64_t lease_ttl_ms = 600000;
+  // PF_PATH_AUTO threshold of the workers' transfer engines; 0 = the engine's default.
+  uint64_t auto_staged_min_bytes = 0;
 };
 
 // block.rs:20-25, as a view of the caller's arrays (valid for the call).

@@ -271,6 +271,7 @@ int pf_engine_create(const pf_engine_config* cfg, pf_engine_t* out) {
   c.use_descriptor_backends = cfg->use_descriptor_backends != 0;
   c.unit_size_hint = cfg->unit_size_hint;
   if (cfg->lease_ttl_ms != 0) c.lease_ttl_ms = cfg->lease_ttl_ms;
+  c.auto_staged_min_bytes = cfg->auto_staged_min_bytes;
   std::string err;
   int status = PF_ERR_STORAGE;
   auto e = pf::Engine::create(c, &err, &status);

@@ -282,11 +282,12 @@ bool to_block_form(const std::vector<LayerTransferData>& all_layers, size_t begi
 std::unique_ptr<GpuWorkerPool> GpuWorkerPool::spawn(int device_id, NumaNode numa_node,
                                                     TransferMode mode,
                                                     bool use_descriptor_backends, std::string* err,
-                                                    int* status) {
+                                                    int* status, uint64_t auto_staged_min_bytes) {
   std::unique_ptr<GpuWorkerPool> pool(new GpuWorkerPool());
   pool->device_id_ = device_id;
   pool->mode_ = mode;
   pool->use_descriptors_ = use_descriptor_backends;
+  pool->auto_staged_min_bytes_ = auto_staged_min_bytes;
   std::promise<TaskResult> load_ready, save_ready;
   auto lf = load_ready.get_future();
   auto sf = save_ready.get_future();
@@ -553,6 +554,7 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
       pf_xfer_config cfg;
       std::memset(&cfg, 0, sizeof(cfg));
       cfg.copy_stream = 2;
+      cfg.auto_staged_min_bytes = auto_staged_min_bytes_;
       xfer = Xfer::create(&cfg);
       if (!xfer) {
         init.status = PF_ERR_DEVICE_INIT;

@@ -95,7 +95,7 @@ class GpuWorkerPool {
   // choosing the link path (Direct = staged when possible, Kernel = zero-copy).
   static std::unique_ptr<GpuWorkerPool> spawn(int device_id, NumaNode numa_node, TransferMode mode,
                                               bool use_descriptor_backends, std::string* err,
-                                              int* status);
+                                              int* status, uint64_t auto_staged_min_bytes = 0);
   ~GpuWorkerPool();
   // gpu_worker.rs:204-212: fire and forget; the future (and the LoadState, if
   // named) is signalled when the task settles.
@@ -135,6 +135,7 @@ class GpuWorkerPool {
   int device_id_ = 0;
   TransferMode mode_ = TransferMode::Direct;
   bool use_descriptors_ = false;
+  uint64_t auto_staged_min_bytes_ = 0;  // 0 = the transfer engine's default
   Worker load_;
   Worker save_;
   size_t queue_clashes_ = 0;

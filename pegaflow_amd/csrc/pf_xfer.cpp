@@ -894,16 +894,26 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     const BlockUnit& u = units_host[ui];
     const bool last_of_layer =
         ui + 1 == unit_refs.size() || unit_refs[ui + 1].plan != unit_refs[ui].plan;
+    // K and V cross the link as one copy when V follows K both in staging and
+    // in the host image (the engine allocates a layer's K and V buffers one
+    // after the other): a copy costs ~10 us beyond its bytes.
+    uint64_t link_bytes = r.count * p.frag_bytes;
+    uint32_t link_copies = p.n_seg;
+    if (p.n_seg == 2 && u.far_base[1] == u.far_base[0] + link_bytes &&
+        p.host[1] + r.first * p.host_stride == p.host[0] + r.first * p.host_stride + link_bytes) {
+      link_bytes *= 2;
+      link_copies = 1;
+    }
     if (save) {
       if (sl.used) PF_HIP(hipStreamWaitEvent(s, sl.freed, 0));
       st = launch_tiles(units_dev + ui, u, true, s);
       if (st != PF_OK) return st;
       PF_HIP(hipEventRecord(sl.ready, s));
       PF_HIP(hipStreamWaitEvent(side, sl.ready, 0));
-      for (uint32_t sgm = 0; sgm < p.n_seg; ++sgm) {
+      for (uint32_t sgm = 0; sgm < link_copies; ++sgm) {
         PF_HIP(hipMemcpyAsync(p.host[sgm] + r.first * p.host_stride,
                               reinterpret_cast<const void*>(u.far_base[sgm]),
-                              r.count * p.frag_bytes, hipMemcpyDeviceToHost, side));
+                              link_bytes, hipMemcpyDeviceToHost, side));
       }
       PF_HIP(hipEventRecord(sl.freed, side));
       sl.used = true;
@@ -913,9 +923,9 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
       }
     } else {
       if (sl.used) PF_HIP(hipStreamWaitEvent(side, sl.freed, 0));
-      for (uint32_t sgm = 0; sgm < p.n_seg; ++sgm) {
+      for (uint32_t sgm = 0; sgm < link_copies; ++sgm) {
         PF_HIP(hipMemcpyAsync(reinterpret_cast<void*>(u.far_base[sgm]),
-                              p.host[sgm] + r.first * p.host_stride, r.count * p.frag_bytes,
+                              p.host[sgm] + r.first * p.host_stride, link_bytes,
                               hipMemcpyHostToDevice, side));
       }
       PF_HIP(hipEventRecord(sl.ready, side));

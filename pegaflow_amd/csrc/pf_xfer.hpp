@@ -33,8 +33,16 @@ constexpr uint32_t kDefaultSlots = 2;
 // one call favour it even more (8 x 4 MiB: 50.3 against 37.3).  Loads are
 // faster zero-copy at every size (128 MiB: 56.9 against 55.1 GB/s), but a
 // long zero-copy transfer slows kernels that run beside it, which a staged
-// one does not, so large loads are staged as well.
-constexpr uint64_t kDefaultAutoStagedMin = 64ull << 20;
+// one does not, so large loads are staged as well.  What it costs them
+// decides the threshold: a back-to-back stream of 2048^3 bf16 GEMMs (23 us
+// each) runs at 104-109 TFLOP/s beside a 16-workgroup zero-copy transfer and
+// at 687-713 beside a staged one (591 alone, launch-bound), a 1024^3 stream at
+// 28 against 110; a staged layer costs ~30 us beyond its bytes (through the
+// engine's workers, 32 layers: 16 MiB per layer 49.4 / 51.3 GB/s staged
+// against 54.1 / 56.0 zero-copy, 32 MiB 51.7 / 53.5 against 53.9 / 56.1, 4 MiB
+// 40.1 / 41.7 against 51.0 / 54.7).  From 16 MiB per layer on a transfer
+// outlasts 280 us and gives up less than a tenth of its rate by staging.
+constexpr uint64_t kDefaultAutoStagedMin = 16ull << 20;
 constexpr int kDefaultUnroll = 4;
 // Zero-copy launches are capped to a few workgroups: the host link, not the
 // GPU, is the bound, and every workgroup that stays resident for the length of

@@ -233,13 +233,17 @@ class PegaEngine:
     def __init__(self, pool_size: int, use_hugepages: bool = False, numa_aware: bool = False,
                  pool_shards: int = 1, blockwise_alloc: bool = False, ssd_enabled: bool = False,
                  use_descriptor_backends: bool = False, unit_size_hint: int = 0,
-                 lease_ttl_ms: int = 0):
+                 lease_ttl_ms: int = 0, auto_staged_min_bytes: int = 0):
         """``lease_ttl_ms``: how long an unconsumed query lease pins its blocks
-        (0 = the reference's 600 s, lease.rs:11)."""
+        (0 = the reference's 600 s, lease.rs:11).  ``auto_staged_min_bytes``: the
+        smallest dense transfer the workers stage through device memory instead
+        of moving it with the resident zero-copy kernel (0 = 16 MiB per layer); lower it
+        where short model kernels run beside the transfers."""
         self._lib = _lib.load()
         cfg = _lib.PfEngineConfig(pool_size, int(use_hugepages), int(numa_aware), pool_shards,
                                   int(blockwise_alloc), int(ssd_enabled),
-                                  int(use_descriptor_backends), unit_size_hint, lease_ttl_ms)
+                                  int(use_descriptor_backends), unit_size_hint, lease_ttl_ms,
+                                  auto_staged_min_bytes)
         h = C.c_void_p()
         check(self._lib.pf_engine_create(C.byref(cfg), C.byref(h)))
         self.handle = h

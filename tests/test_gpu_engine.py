@@ -833,3 +833,29 @@ def test_partially_cached_save_stores_only_the_new_blocks(engine):
     for dst, src in zip(range(10, 16), [0, 1, 2, 3, 7, 6]):
         want[dst * 1024:(dst + 1) * 1024] = layer.expected[src * 1024:(src + 1) * 1024]
     layer.assert_gpu_matches(want)
+
+
+def test_lower_staging_threshold_moves_the_same_bytes(gpu):
+    """pf_engine_config.auto_staged_min_bytes: with the workers' threshold at
+    1 MiB a 6 MiB save and load go through device staging instead of the
+    resident zero-copy kernel; the bytes are the same."""
+    e = PegaEngine(pool_size=64 << 20, auto_staged_min_bytes=1 << 20)
+    layers = [Layer(f"layer_{i}", 64, 16384, split_kv_stride=64 * 16384) for i in range(3)]
+    register(e, "staged-small", layers)
+    hashes = make_block_hashes(48, 3)
+    ids = list(range(8, 56))
+    e.batch_save_kv_blocks("staged-small", 0, 0, 0, [LayerSave(l.name, ids, hashes) for l in layers])
+    for l in layers:
+        l.zero_gpu()
+    hits, lease = e.query_prefix("staged-small", hashes)
+    assert hits == 48
+    dest = list(range(0, 48))
+    e.batch_load_kv_blocks_multi_layer("staged-small", 0, 0, [[l.name for l in layers]], lease,
+                                       [dest]).wait()
+    for l in layers:
+        want = np.zeros_like(l.expected)
+        view = want.reshape(2, 64, 16384)
+        src = l.expected.reshape(2, 64, 16384)
+        view[:, dest] = src[:, ids]
+        l.assert_gpu_matches(want)
+    e.close()
