@@ -750,15 +750,47 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
 
   // ---- 3. staging slots ---------------------------------------------------
   std::vector<uint32_t> unit_slot(unit_refs.size(), 0);
-  if (max_unit_bytes != 0) {
-    for (auto& sl : slots_) {
-      st = ensure_slot(sl, max_unit_bytes);
-      if (st != PF_OK) return st;
-    }
-  }
   BlockUnit* units_host = reinterpret_cast<BlockUnit*>(slab_host);
   const BlockUnit* units_dev = reinterpret_cast<const BlockUnit*>(slab_dev);
   uint32_t slot_cursor = next_slot_;
+  // Small staged units that follow one another share a slot: one gather (or
+  // scatter) launch serves the whole group, which saves a launch and its
+  // hand-offs per layer (~12 of the ~30 us a staged layer costs beyond its
+  // bytes).  group_end[ui] is one past the last unit of the group that starts
+  // at ui (0 for units inside a group and for zero-copy units).
+  std::vector<size_t> group_end(unit_refs.size(), 0);
+  std::vector<uint64_t> unit_slot_off(unit_refs.size(), 0);
+  {
+    const uint64_t group_cap = std::min<uint64_t>(kStagedGroupBytes, slot_bytes_);
+    size_t ui = 0;
+    while (ui < unit_refs.size()) {
+      if (!plans[unit_refs[ui].plan].staged) {
+        ++ui;
+        continue;
+      }
+      uint64_t used = 0;
+      size_t ue = ui;
+      while (ue < unit_refs.size() && plans[unit_refs[ue].plan].staged &&
+             ue - ui < kStagedGroupUnits) {
+        const LayerPlan& q = plans[unit_refs[ue].plan];
+        const uint64_t bytes = (unit_refs[ue].count * q.frag_bytes * q.n_seg + 255) & ~255ull;
+        if (ue > ui && used + bytes > group_cap) break;
+        unit_slot_off[ue] = used;
+        used += bytes;
+        ++ue;
+      }
+      group_end[ui] = ue;
+      max_unit_bytes = std::max(max_unit_bytes, used);
+      ui = ue;
+    }
+    if (max_unit_bytes != 0) {
+      for (auto& sl : slots_) {
+        st = ensure_slot(sl, max_unit_bytes);
+        if (st != PF_OK) return st;
+      }
+    }
+  }
+  uint32_t group_slot = 0;
   for (size_t ui = 0; ui < unit_refs.size(); ++ui) {
     const UnitRef& r = unit_refs[ui];
     const LayerPlan& p = plans[r.plan];
@@ -778,10 +810,12 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     u.n_seg = p.n_seg;
     u.tiles_per_frag = static_cast<uint32_t>((p.frag_bytes + tile - 1) / tile);
     if (p.staged) {
-      uint32_t slot = slot_cursor;
-      slot_cursor = (slot_cursor + 1) % n_slots_;
-      unit_slot[ui] = slot;
-      const uint64_t base = reinterpret_cast<uint64_t>(slots_[slot].buf);
+      if (group_end[ui] != 0) {  // first unit of a group: the next slot
+        group_slot = slot_cursor;
+        slot_cursor = (slot_cursor + 1) % n_slots_;
+      }
+      unit_slot[ui] = group_slot;
+      const uint64_t base = reinterpret_cast<uint64_t>(slots_[group_slot].buf) + unit_slot_off[ui];
       u.far_base[0] = base;
       u.far_base[1] = base + r.count * p.frag_bytes;
       u.far_stride = p.frag_bytes;
@@ -886,62 +920,93 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
       continue;
     }
 
-    // Staged unit.
+    // Staged group: the units [ui, ue) share one slot.
     st = fork_side();
     if (st != PF_OK) return st;
-    const UnitRef& r = unit_refs[ui];
+    const size_t ue = group_end[ui];
     Slot& sl = slots_[unit_slot[ui]];
-    const BlockUnit& u = units_host[ui];
-    const bool last_of_layer =
-        ui + 1 == unit_refs.size() || unit_refs[ui + 1].plan != unit_refs[ui].plan;
-    // K and V cross the link as one copy when V follows K both in staging and
-    // in the host image (the engine allocates a layer's K and V buffers one
-    // after the other): a copy costs ~10 us beyond its bytes.
-    uint64_t link_bytes = r.count * p.frag_bytes;
-    uint32_t link_copies = p.n_seg;
-    if (p.n_seg == 2 && u.far_base[1] == u.far_base[0] + link_bytes &&
-        p.host[1] + r.first * p.host_stride == p.host[0] + r.first * p.host_stride + link_bytes) {
-      link_bytes *= 2;
-      link_copies = 1;
-    }
+    // K and V of a unit cross the link as one copy when V follows K both in
+    // staging and in the host image (the engine allocates a layer's K and V
+    // buffers one after the other): a copy costs ~10 us beyond its bytes.
+    auto link_copies = [&](size_t k, bool to_host) -> int {
+      const UnitRef& r = unit_refs[k];
+      const LayerPlan& q = plans[r.plan];
+      const BlockUnit& u = units_host[k];
+      uint64_t bytes = r.count * q.frag_bytes;
+      uint32_t copies = q.n_seg;
+      if (q.n_seg == 2 && u.far_base[1] == u.far_base[0] + bytes &&
+          q.host[1] + r.first * q.host_stride == q.host[0] + r.first * q.host_stride + bytes) {
+        bytes *= 2;
+        copies = 1;
+      }
+      for (uint32_t sgm = 0; sgm < copies; ++sgm) {
+        uint8_t* host_ptr = q.host[sgm] + r.first * q.host_stride;
+        void* staged = reinterpret_cast<void*>(u.far_base[sgm]);
+        if (to_host) {
+          PF_HIP(hipMemcpyAsync(host_ptr, staged, bytes, hipMemcpyDeviceToHost, side));
+        } else {
+          PF_HIP(hipMemcpyAsync(staged, host_ptr, bytes, hipMemcpyHostToDevice, side));
+        }
+      }
+      return PF_OK;
+    };
+    auto launch_group = [&](bool to_far) -> int {
+      if (ue - ui == 1) return launch_tiles(units_dev + ui, units_host[ui], to_far, s);
+      uint32_t max_blocks = 0, max_seg = 0;
+      uint64_t max_frag = 0;
+      for (size_t k = ui; k < ue; ++k) {
+        max_blocks = std::max(max_blocks, units_host[k].n_blocks);
+        max_seg = std::max(max_seg, units_host[k].n_seg);
+        max_frag = std::max(max_frag, units_host[k].frag_bytes);
+      }
+      int rc = timing_begin(s);
+      if (rc != PF_OK) return rc;
+      rc = launch_block_tiles(units_dev + ui, static_cast<uint32_t>(ue - ui), max_blocks, max_frag,
+                              max_seg, to_far, s);
+      if (rc != PF_OK) return rc;
+      return timing_end(s);
+    };
+    // The events of every layer that ends inside the group fire behind it.
+    const uint64_t last_layer = plans[unit_refs[ue - 1].plan].src_index;
+    const bool ends_a_layer =
+        ue == unit_refs.size() || unit_refs[ue].plan != unit_refs[ue - 1].plan;
+    const uint64_t fire_through = ends_a_layer ? last_layer : (last_layer == 0 ? UINT64_MAX : last_layer - 1);
     if (save) {
       if (sl.used) PF_HIP(hipStreamWaitEvent(s, sl.freed, 0));
-      st = launch_tiles(units_dev + ui, u, true, s);
+      st = launch_group(true);
       if (st != PF_OK) return st;
       PF_HIP(hipEventRecord(sl.ready, s));
       PF_HIP(hipStreamWaitEvent(side, sl.ready, 0));
-      for (uint32_t sgm = 0; sgm < link_copies; ++sgm) {
-        PF_HIP(hipMemcpyAsync(p.host[sgm] + r.first * p.host_stride,
-                              reinterpret_cast<const void*>(u.far_base[sgm]),
-                              link_bytes, hipMemcpyDeviceToHost, side));
+      for (size_t k = ui; k < ue; ++k) {
+        st = link_copies(k, true);
+        if (st != PF_OK) return st;
       }
       PF_HIP(hipEventRecord(sl.freed, side));
       sl.used = true;
-      if (last_of_layer) {
-        st = fire_events_through(p.src_index, side);
+      if (fire_through != UINT64_MAX) {
+        st = fire_events_through(fire_through, side);
         if (st != PF_OK) return st;
       }
     } else {
       if (sl.used) PF_HIP(hipStreamWaitEvent(side, sl.freed, 0));
-      for (uint32_t sgm = 0; sgm < link_copies; ++sgm) {
-        PF_HIP(hipMemcpyAsync(reinterpret_cast<void*>(u.far_base[sgm]),
-                              p.host[sgm] + r.first * p.host_stride, link_bytes,
-                              hipMemcpyHostToDevice, side));
+      for (size_t k = ui; k < ue; ++k) {
+        st = link_copies(k, false);
+        if (st != PF_OK) return st;
       }
       PF_HIP(hipEventRecord(sl.ready, side));
       st = upload_orders();
       if (st != PF_OK) return st;
       PF_HIP(hipStreamWaitEvent(s, sl.ready, 0));
-      st = launch_tiles(units_dev + ui, u, false, s);
+      st = launch_group(false);
       if (st != PF_OK) return st;
       PF_HIP(hipEventRecord(sl.freed, s));
       sl.used = true;
-      if (last_of_layer) {
-        st = fire_events_through(p.src_index, s);
+      if (fire_through != UINT64_MAX) {
+        st = fire_events_through(fire_through, s);
         if (st != PF_OK) return st;
       }
     }
-    ++ui;
+    ui = ue;
   }
   if (side_used && save) {
     // Join: everything the side stream drained is ordered before whatever the

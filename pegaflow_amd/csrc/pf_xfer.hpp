@@ -37,12 +37,19 @@ constexpr uint32_t kDefaultSlots = 2;
 // decides the threshold: a back-to-back stream of 2048^3 bf16 GEMMs (23 us
 // each) runs at 104-109 TFLOP/s beside a 16-workgroup zero-copy transfer and
 // at 687-713 beside a staged one (591 alone, launch-bound), a 1024^3 stream at
-// 28 against 110; a staged layer costs ~30 us beyond its bytes (through the
-// engine's workers, 32 layers: 16 MiB per layer 49.4 / 51.3 GB/s staged
-// against 54.1 / 56.0 zero-copy, 32 MiB 51.7 / 53.5 against 53.9 / 56.1, 4 MiB
-// 40.1 / 41.7 against 51.0 / 54.7).  From 16 MiB per layer on a transfer
-// outlasts 280 us and gives up less than a tenth of its rate by staging.
+// 28 against 110; a staged layer costs 10-30 us beyond its bytes (through the
+// engine's workers, 32 layers: 16 MiB per layer 50.0 / 52.0 GB/s staged
+// against 54.1 / 56.0 zero-copy, 32 MiB 51.3 / 53.0 against 53.9 / 56.1, 4 MiB
+// 44.7 / 46.4 against 51.0 / 54.7, 1 MiB 29.1 / 32.6 against 42.5 / 49.6).  From
+// 16 MiB per layer on a transfer outlasts 280 us and gives up less than a
+// tenth of its rate by staging.
 constexpr uint64_t kDefaultAutoStagedMin = 16ull << 20;
+// Staged units that follow one another share a staging slot, and one gather or
+// scatter launch, while together they stay below this size and count: the
+// copies of a group still take well under a millisecond, so the pipeline
+// keeps its grain.
+constexpr uint64_t kStagedGroupBytes = 32ull << 20;
+constexpr size_t kStagedGroupUnits = 16;
 constexpr int kDefaultUnroll = 4;
 // Zero-copy launches are capped to a few workgroups: the host link, not the
 // GPU, is the bound, and every workgroup that stays resident for the length of

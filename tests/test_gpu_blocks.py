@@ -502,3 +502,88 @@ def test_page_packing_is_refused_when_it_would_touch_foreign_bytes(xfer, stream)
     for c in cases:
         c.close()
     pool.close()
+
+
+@pytest.mark.parametrize("copy_stream", [0, 2], ids=["side_stream", "in_order"])
+def test_small_staged_layers_share_slots_and_launches(stream, copy_stream):
+    """Staged layers that are small share a staging slot and one gather /
+    scatter launch per group.  Nine layers of unlike shapes in one call -
+    split and contiguous, 4 KiB to 48 KiB fragments, one with a size that is
+    no multiple of 16, one empty, counts from 1 to 300 - so that groups close
+    on the unit count and on the byte cap; checked against the oracle both
+    ways, with per-layer events and untouched bytes."""
+    rng = np.random.default_rng(77)
+    shapes = [dict(num_blocks=512, seg=32768, segments=2, n_ids=300),   # 18.75 MiB: fills most of a group
+              dict(num_blocks=256, seg=16384, segments=2, n_ids=200),   # closes the first group on bytes
+              dict(num_blocks=128, seg=4096, segments=2, n_ids=97),
+              dict(num_blocks=64, seg=49152, segments=1, n_ids=33),
+              dict(num_blocks=64, seg=4104, segments=2, n_ids=20),      # byte tail in every fragment
+              dict(num_blocks=64, seg=8192, segments=2, n_ids=1),
+              dict(num_blocks=64, seg=8192, segments=1, n_ids=1),
+              dict(num_blocks=300, seg=16384, segments=2, n_ids=299),
+              dict(num_blocks=128, seg=32768, segments=1, n_ids=128)]
+    cases = [Case(rng, **kw) for kw in shapes]
+    cases[6].ids = np.zeros(0, dtype=np.uint32)                          # an empty layer inside a group
+    hosts, layers, Ls = [], [], []
+    for li, c in enumerate(cases):
+        L = c.product_layout()
+        Ls.append(L)
+        nseg = 2 if L.is_split else 1
+        # K and V buffers adjacent for even layers (one link copy), apart for odd ones
+        gap = 0 if li % 2 == 0 else 4096
+        n, stride = len(c.ids), L.host_stride
+        h = PinnedMemory(max(1, nseg * n * stride + gap))
+        h.as_numpy()[:] = SENT
+        hosts.append((h, gap))
+        c.dev.copy_from_host(c.cache0)
+        lb = _dense_layer(c, L, h, c.ids)
+        if nseg == 2 and gap:
+            buf = n * stride
+            lb.host = (h.host_ptr, h.host_ptr + buf + gap)
+            lb.host_device = (h.device_ptr, h.device_ptr + buf + gap)
+        lb.layer_name = f"layer_{li}"
+        layers.append(lb)
+    xfer = BlockTransfer(auto_staged_min_bytes=1, copy_stream=copy_stream)
+    events = [Event() for _ in cases]
+    xfer.set_layer_events(events)
+    xfer.save(layers, stream, TransferPath.AUTO)
+    for e in events:
+        e.synchronize()
+    stream.synchronize()
+    assert xfer.last_path == ST
+    images = []
+    for c, L, (h, gap) in zip(cases, Ls, hosts):
+        n, stride = len(c.ids), L.host_stride
+        if n == 0:
+            images.append((None, None))
+            continue
+        oc = c.cache0.copy()
+        ok = np.full(n * stride, SENT, dtype=np.uint8)
+        ov = np.full(n * stride, SENT, dtype=np.uint8) if L.is_split else None
+        O.transfer_layer(c.oracle_layout(oc), c.ids, ok, ov, host_is_src=False)
+        hv = h.as_numpy()
+        assert np.array_equal(hv[: n * stride], ok), c.args
+        if ov is not None:
+            assert (hv[n * stride: n * stride + gap] == SENT).all()
+            assert np.array_equal(hv[n * stride + gap: 2 * n * stride + gap], ov), c.args
+        images.append((ok, ov))
+    # load into other slots of sentinel-filled caches
+    for li, c in enumerate(cases):
+        c.dev.fill(SENT)
+        if len(c.ids):
+            layers[li].block_ids = rng.choice(c.num_blocks, len(c.ids), replace=False).astype(np.uint32)
+    xfer.load(layers, stream, TransferPath.AUTO)
+    for e in events:
+        e.synchronize()
+    stream.synchronize()
+    for li, (c, L) in enumerate(zip(cases, Ls)):
+        oc = np.full_like(c.cache0, SENT)
+        if len(c.ids):
+            ok, ov = images[li]
+            O.transfer_layer(c.oracle_layout(oc), layers[li].block_ids, ok, ov, host_is_src=True)
+        assert np.array_equal(c.dev.copy_to_host(), oc), li
+    xfer.set_layer_events(None)
+    xfer.close()
+    for c, (h, _gap) in zip(cases, hosts):
+        c.close()
+        h.close()
