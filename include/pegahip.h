@@ -584,10 +584,12 @@ typedef struct pf_engine_config {
   uint32_t use_descriptor_backends;  /* see pf_worker_pool_spawn */
   uint64_t unit_size_hint;
   uint64_t lease_ttl_ms;             /* lease.rs:11: 0 = default (600 000 ms) */
-  uint64_t auto_staged_min_bytes;    /* workers: smallest dense transfer that is staged instead of
-                                        moved by the resident zero-copy kernel; 0 = default (16 MiB per layer).
-                                        Lower it where short model kernels run beside the transfers:
-                                        a resident copy kernel costs them far more than a staged copy. */
+  uint64_t auto_staged_min_bytes;    /* workers: smallest dense layer that is staged instead of
+                                        moved by the resident zero-copy kernel; 0 = default (4 MiB;
+                                        a lone pf_xfer stages from 16 MiB).  Model kernels that run
+                                        beside the resident kernel slow down for as long as it runs,
+                                        a staged copy leaves them alone: lower it to favour the model,
+                                        UINT64_MAX = never stage (offload while the GPU is idle). */
 } pf_engine_config;
 
 typedef struct pf_layer_save {       /* LayerSave, block.rs:20-25 */

@@ -925,27 +925,40 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     if (st != PF_OK) return st;
     const size_t ue = group_end[ui];
     Slot& sl = slots_[unit_slot[ui]];
-    // K and V of a unit cross the link as one copy when V follows K both in
-    // staging and in the host image (the engine allocates a layer's K and V
-    // buffers one after the other): a copy costs ~10 us beyond its bytes.
-    auto link_copies = [&](size_t k, bool to_host) -> int {
+    // The link copies of the group, coalesced: pieces that follow one another
+    // both in staging and in the host image cross as one copy (a copy costs
+    // ~10 us beyond its bytes).  V follows K when the engine allocated a
+    // layer's K and V buffers one after the other, and the next layer follows
+    // when its buffers were allocated right behind: a group of small layers
+    // saved by one call is then a single copy.
+    struct LinkCopy {
+      uint8_t* host;
+      uint64_t staged;
+      uint64_t bytes;
+    };
+    std::vector<LinkCopy> group_copies;
+    for (size_t k = ui; k < ue; ++k) {
       const UnitRef& r = unit_refs[k];
       const LayerPlan& q = plans[r.plan];
       const BlockUnit& u = units_host[k];
-      uint64_t bytes = r.count * q.frag_bytes;
-      uint32_t copies = q.n_seg;
-      if (q.n_seg == 2 && u.far_base[1] == u.far_base[0] + bytes &&
-          q.host[1] + r.first * q.host_stride == q.host[0] + r.first * q.host_stride + bytes) {
-        bytes *= 2;
-        copies = 1;
-      }
-      for (uint32_t sgm = 0; sgm < copies; ++sgm) {
-        uint8_t* host_ptr = q.host[sgm] + r.first * q.host_stride;
-        void* staged = reinterpret_cast<void*>(u.far_base[sgm]);
-        if (to_host) {
-          PF_HIP(hipMemcpyAsync(host_ptr, staged, bytes, hipMemcpyDeviceToHost, side));
+      for (uint32_t sgm = 0; sgm < q.n_seg; ++sgm) {
+        LinkCopy c{q.host[sgm] + r.first * q.host_stride, u.far_base[sgm], r.count * q.frag_bytes};
+        if (!group_copies.empty() &&
+            group_copies.back().host + group_copies.back().bytes == c.host &&
+            group_copies.back().staged + group_copies.back().bytes == c.staged) {
+          group_copies.back().bytes += c.bytes;
         } else {
-          PF_HIP(hipMemcpyAsync(staged, host_ptr, bytes, hipMemcpyHostToDevice, side));
+          group_copies.push_back(c);
+        }
+      }
+    }
+    auto link_copies = [&](bool to_host) -> int {
+      for (const LinkCopy& c : group_copies) {
+        void* staged = reinterpret_cast<void*>(c.staged);
+        if (to_host) {
+          PF_HIP(hipMemcpyAsync(c.host, staged, c.bytes, hipMemcpyDeviceToHost, side));
+        } else {
+          PF_HIP(hipMemcpyAsync(staged, c.host, c.bytes, hipMemcpyHostToDevice, side));
         }
       }
       return PF_OK;
@@ -977,10 +990,8 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
       if (st != PF_OK) return st;
       PF_HIP(hipEventRecord(sl.ready, s));
       PF_HIP(hipStreamWaitEvent(side, sl.ready, 0));
-      for (size_t k = ui; k < ue; ++k) {
-        st = link_copies(k, true);
-        if (st != PF_OK) return st;
-      }
+      st = link_copies(true);
+      if (st != PF_OK) return st;
       PF_HIP(hipEventRecord(sl.freed, side));
       sl.used = true;
       if (fire_through != UINT64_MAX) {
@@ -989,10 +1000,8 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
       }
     } else {
       if (sl.used) PF_HIP(hipStreamWaitEvent(side, sl.freed, 0));
-      for (size_t k = ui; k < ue; ++k) {
-        st = link_copies(k, false);
-        if (st != PF_OK) return st;
-      }
+      st = link_copies(false);
+      if (st != PF_OK) return st;
       PF_HIP(hipEventRecord(sl.ready, side));
       st = upload_orders();
       if (st != PF_OK) return st;

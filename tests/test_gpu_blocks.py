@@ -524,25 +524,35 @@ def test_small_staged_layers_share_slots_and_launches(stream, copy_stream):
               dict(num_blocks=128, seg=32768, segments=1, n_ids=128)]
     cases = [Case(rng, **kw) for kw in shapes]
     cases[6].ids = np.zeros(0, dtype=np.uint32)                          # an empty layer inside a group
+    # One pinned pool, the layers' images one behind the other as the engine's
+    # allocations of one save are: even layers have V right behind K and start
+    # right behind the layer before (pieces that cross the link as one copy),
+    # odd ones keep a gap before V and after themselves.
+    sizes = []
+    for li, c in enumerate(cases):
+        L = c.product_layout()
+        nseg = 2 if L.is_split else 1
+        sizes.append(nseg * len(c.ids) * L.host_stride + (0 if li % 2 == 0 else 2 * 4096))
+    pool = PinnedMemory(sum(sizes) + 4096)
+    pool.as_numpy()[:] = SENT
     hosts, layers, Ls = [], [], []
+    cursor = 0
     for li, c in enumerate(cases):
         L = c.product_layout()
         Ls.append(L)
         nseg = 2 if L.is_split else 1
-        # K and V buffers adjacent for even layers (one link copy), apart for odd ones
         gap = 0 if li % 2 == 0 else 4096
         n, stride = len(c.ids), L.host_stride
-        h = PinnedMemory(max(1, nseg * n * stride + gap))
-        h.as_numpy()[:] = SENT
-        hosts.append((h, gap))
+        buf = n * stride
+        hosts.append((cursor, gap))
         c.dev.copy_from_host(c.cache0)
-        lb = _dense_layer(c, L, h, c.ids)
-        if nseg == 2 and gap:
-            buf = n * stride
-            lb.host = (h.host_ptr, h.host_ptr + buf + gap)
-            lb.host_device = (h.device_ptr, h.device_ptr + buf + gap)
-        lb.layer_name = f"layer_{li}"
+        lb = LayerBlocks(
+            layout=L, block_ids=c.ids,
+            host=tuple(pool.host_ptr + cursor + s_ * (buf + gap) for s_ in range(nseg)),
+            host_device=tuple(pool.device_ptr + cursor + s_ * (buf + gap) for s_ in range(nseg)),
+            host_len=tuple(buf for _ in range(nseg)), host_stride=stride, layer_name=f"layer_{li}")
         layers.append(lb)
+        cursor += sizes[li]
     xfer = BlockTransfer(auto_staged_min_bytes=1, copy_stream=copy_stream)
     events = [Event() for _ in cases]
     xfer.set_layer_events(events)
@@ -552,7 +562,8 @@ def test_small_staged_layers_share_slots_and_launches(stream, copy_stream):
     stream.synchronize()
     assert xfer.last_path == ST
     images = []
-    for c, L, (h, gap) in zip(cases, Ls, hosts):
+    expect_pool = np.full(pool.as_numpy().size, SENT, dtype=np.uint8)
+    for c, L, (at, gap) in zip(cases, Ls, hosts):
         n, stride = len(c.ids), L.host_stride
         if n == 0:
             images.append((None, None))
@@ -561,12 +572,16 @@ def test_small_staged_layers_share_slots_and_launches(stream, copy_stream):
         ok = np.full(n * stride, SENT, dtype=np.uint8)
         ov = np.full(n * stride, SENT, dtype=np.uint8) if L.is_split else None
         O.transfer_layer(c.oracle_layout(oc), c.ids, ok, ov, host_is_src=False)
-        hv = h.as_numpy()
+        expect_pool[at: at + n * stride] = ok
+        if ov is not None:
+            expect_pool[at + n * stride + gap: at + 2 * n * stride + gap] = ov
+        hv = pool.as_numpy()[at:]
         assert np.array_equal(hv[: n * stride], ok), c.args
         if ov is not None:
             assert (hv[n * stride: n * stride + gap] == SENT).all()
             assert np.array_equal(hv[n * stride + gap: 2 * n * stride + gap], ov), c.args
         images.append((ok, ov))
+    assert np.array_equal(pool.as_numpy(), expect_pool)      # gaps and the pool's tail untouched
     # load into other slots of sentinel-filled caches
     for li, c in enumerate(cases):
         c.dev.fill(SENT)
@@ -584,6 +599,6 @@ def test_small_staged_layers_share_slots_and_launches(stream, copy_stream):
         assert np.array_equal(c.dev.copy_to_host(), oc), li
     xfer.set_layer_events(None)
     xfer.close()
-    for c, (h, _gap) in zip(cases, hosts):
+    for c in cases:
         c.close()
-        h.close()
+    pool.close()
