@@ -75,6 +75,7 @@ int main(){
   rc|=run(true,1,false,false,1,5,128,8192,60,64);
   rc|=run(true,0,false,false,1,5,2048,65536,1500,1200);   // page-first, whole-page staging (>64 MiB)
   rc|=run(false,0,false,false,2,20,4096,32768,2500,4000); // staged, two-part conversion on load
+  rc|=run(false,0,false,false,2,12,1024,32768,200,600);   // 12.5 MiB layers: staged in groups that share a slot and a launch
   rc|=run(false,1,false,false,2,8,4096,32768,2500,2000);  // kernel mode at the same size: the engine picks the path, as in direct mode
   rc|=run(false,2,false,false,2,8,4096,32768,2500,2000);  // PF_MODE_ZEROCOPY at the same size: zero-copy both ways
   rc|=run(true,2,false,false,1,5,128,8192,60,64);         // PF_MODE_ZEROCOPY over page-first pages
