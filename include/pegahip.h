@@ -585,7 +585,7 @@ typedef struct pf_engine_config {
   uint64_t unit_size_hint;
   uint64_t lease_ttl_ms;             /* lease.rs:11: 0 = default (600 000 ms) */
   uint64_t auto_staged_min_bytes;    /* workers: smallest dense layer that is staged instead of
-                                        moved by the resident zero-copy kernel; 0 = default (4 MiB;
+                                        moved by the resident zero-copy kernel; 0 = default (1 MiB;
                                         a lone pf_xfer stages from 16 MiB).  Model kernels that run
                                         beside the resident kernel slow down for as long as it runs,
                                         a staged copy leaves them alone: lower it to favour the model,

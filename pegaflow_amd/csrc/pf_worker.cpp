@@ -555,12 +555,13 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
       std::memset(&cfg, 0, sizeof(cfg));
       cfg.copy_stream = 2;
       // The workers move KV beside a running model: they stage from a lower
-      // size than a lone transfer engine does.  Through these workers, 32
-      // layers per call, staged against zero-copy: 4 MiB per layer 48.9 / 51.0
-      // against 51.0 / 54.7 GB/s save / load, 1 MiB 39.0 / 44.0 against
-      // 42.7 / 51.0 - and short kernels beside the zero-copy kernel run at a
-      // sixth to a quarter of their rate for as long as it is resident.
-      constexpr uint64_t kWorkerAutoStagedMin = 4ull << 20;
+      // size than a lone transfer engine does.  A stream of 2048^3 bf16 GEMMs
+      // beside an unbroken loop of saves and loads through these workers, 32
+      // layers per call, keeps 0.94-0.95 of its rate when the layers are
+      // staged and 0.21 (4 MiB layers), 0.36 (1 MiB), 0.58 (256 KiB) when they
+      // go through the resident zero-copy kernel; staging costs the transfers
+      // themselves 6 % at 4 MiB and 1 MiB per layer and 20 % at 256 KiB.
+      constexpr uint64_t kWorkerAutoStagedMin = 1ull << 20;
       cfg.auto_staged_min_bytes =
           auto_staged_min_bytes_ != 0 ? auto_staged_min_bytes_ : kWorkerAutoStagedMin;
       xfer = Xfer::create(&cfg);

@@ -237,7 +237,7 @@ class PegaEngine:
         """``lease_ttl_ms``: how long an unconsumed query lease pins its blocks
         (0 = the reference's 600 s, lease.rs:11).  ``auto_staged_min_bytes``: the
         smallest dense transfer the workers stage through device memory instead
-        of moving it with the resident zero-copy kernel (0 = 4 MiB per layer); lower it
+        of moving it with the resident zero-copy kernel (0 = 1 MiB per layer); lower it
         where short model kernels run beside the transfers."""
         self._lib = _lib.load()
         cfg = _lib.PfEngineConfig(pool_size, int(use_hugepages), int(numa_aware), pool_shards,
