@@ -313,7 +313,8 @@ typedef struct pf_xfer_config {
   uint32_t staging_slots;      /* 0 = default (2) */
   uint32_t zerocopy_max_workgroups; /* workgroups of a zero-copy launch; 0 = default (16 for
                                        fragments of 16 KiB and more, up to 64 for smaller ones) */
-  uint64_t auto_staged_min_bytes;   /* 0 = default threshold for PF_PATH_AUTO */
+  uint64_t auto_staged_min_bytes;   /* PF_PATH_AUTO stages a dense layer of this size or more;
+                                       0 = default (16 MiB) */
   uint32_t tile_unroll;             /* zero-copy kernel: 16-byte loads in flight per lane:
                                        1,2,4,8; 0 = default (4) */
   uint32_t copy_stream;             /* staged path: where the link copies run.
@@ -321,6 +322,11 @@ typedef struct pf_xfer_config {
                                        one staged unit), 1 = a side stream of the engine (the
                                        copy of one unit overlaps the gather of the next),
                                        2 = the caller's stream (in order, no second queue) */
+  uint64_t auto_staged_min_call_bytes; /* PF_PATH_AUTO also stages every dense layer (of 32 KiB or
+                                       more) of a call whose dense layers add up to this much;
+                                       0 = off.  For engines that move KV beside running kernels:
+                                       the resident zero-copy kernel costs those for as long as
+                                       the call lasts. */
 } pf_xfer_config;
 
 typedef struct pf_xfer_s* pf_xfer_t;
@@ -584,12 +590,13 @@ typedef struct pf_engine_config {
   uint32_t use_descriptor_backends;  /* see pf_worker_pool_spawn */
   uint64_t unit_size_hint;
   uint64_t lease_ttl_ms;             /* lease.rs:11: 0 = default (600 000 ms) */
-  uint64_t auto_staged_min_bytes;    /* workers: smallest dense layer that is staged instead of
-                                        moved by the resident zero-copy kernel; 0 = default (1 MiB;
-                                        a lone pf_xfer stages from 16 MiB).  Model kernels that run
-                                        beside the resident kernel slow down for as long as it runs,
-                                        a staged copy leaves them alone: lower it to favour the model,
-                                        UINT64_MAX = never stage (offload while the GPU is idle). */
+  uint64_t auto_staged_min_bytes;    /* workers: a task whose dense layers add up to this much is
+                                        staged through device memory instead of moved by the
+                                        resident zero-copy kernel (layers of 16 MiB and more are
+                                        staged in any case); 0 = default (8 MiB).  Model kernels
+                                        that run beside the resident kernel slow down for as long as
+                                        it runs, a staged copy leaves them alone: 1 = stage whatever
+                                        can be staged, UINT64_MAX = only the large layers. */
 } pf_engine_config;
 
 typedef struct pf_layer_save {       /* LayerSave, block.rs:20-25 */

@@ -554,16 +554,17 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
       pf_xfer_config cfg;
       std::memset(&cfg, 0, sizeof(cfg));
       cfg.copy_stream = 2;
-      // The workers move KV beside a running model: they stage from a lower
-      // size than a lone transfer engine does.  A stream of 2048^3 bf16 GEMMs
-      // beside an unbroken loop of saves and loads through these workers, 32
-      // layers per call, keeps 0.94-0.95 of its rate when the layers are
-      // staged and 0.21 (4 MiB layers), 0.36 (1 MiB), 0.58 (256 KiB) when they
-      // go through the resident zero-copy kernel; staging costs the transfers
-      // themselves 6 % at 4 MiB and 1 MiB per layer and 20 % at 256 KiB.
-      constexpr uint64_t kWorkerAutoStagedMin = 1ull << 20;
-      cfg.auto_staged_min_bytes =
-          auto_staged_min_bytes_ != 0 ? auto_staged_min_bytes_ : kWorkerAutoStagedMin;
+      // The workers move KV beside a running model, so they also stage tasks
+      // of small layers once the task is long enough for the resident
+      // zero-copy kernel to matter to the kernels beside it.  A stream of
+      // 2048^3 bf16 GEMMs beside an unbroken loop of saves and loads through
+      // these workers, 32 layers per call, keeps 0.94-0.96 of its rate when
+      // the layers are staged and 0.21 (4 MiB layers), 0.36 (1 MiB), 0.58
+      // (256 KiB), 0.84 (64 KiB) beside the resident kernel; staging costs
+      // such a call 50-70 us, the length of a 3-4 MiB transfer.
+      constexpr uint64_t kWorkerStagedCallBytes = 8ull << 20;
+      cfg.auto_staged_min_call_bytes =
+          auto_staged_min_bytes_ != 0 ? auto_staged_min_bytes_ : kWorkerStagedCallBytes;
       xfer = Xfer::create(&cfg);
       if (!xfer) {
         init.status = PF_ERR_DEVICE_INIT;

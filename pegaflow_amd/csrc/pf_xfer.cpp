@@ -46,6 +46,7 @@ struct LayerPlan {
   const uint64_t* page_host = nullptr; // host addresses of the same pages
   uint64_t page_offset = 0;
   bool staged = false;
+  bool dense = false;           // uniform host image at the fragment's own stride
   bool vec_ok = false;
   uint64_t ids_slab_off = 0;    // byte offset of the id list inside the slab
   uint64_t table_slab_off = 0;  // byte offset of the page table inside the slab
@@ -269,6 +270,7 @@ int Xfer::plan_layer(const pf_layer_blocks& in, size_t index, int path, LayerPla
   p.vec_ok = near_aligned && far_aligned && (p.n_seg == 1 || !paged || aligned16(p.frag_bytes));
 
   const bool dense = !paged && in.host_stride == p.frag_bytes;
+  p.dense = dense;
   switch (path) {
     case PF_PATH_ZEROCOPY:
       p.staged = false;
@@ -288,7 +290,7 @@ int Xfer::plan_layer(const pf_layer_blocks& in, size_t index, int path, LayerPla
       break;
     case PF_PATH_AUTO:
       p.staged = dense && p.layer_bytes >= auto_min_;
-      break;
+      break;  // run() may still stage it: see the call-size rule there
     default:
       return fail(PF_ERR_INVALID_ARGUMENT, "unknown transfer path %d", path);
   }
@@ -573,6 +575,17 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     int st = plan_layer(layers[li], li, path, &p, &skip);
     if (st != PF_OK) return st;
     if (!skip) plans.push_back(std::move(p));
+  }
+  // A call that moves enough dense bytes is staged whatever the size of its
+  // layers: what the resident zero-copy kernel costs the kernels beside it
+  // grows with the length of the call, and small layers share staging slots
+  // and link copies.
+  if (path == PF_PATH_AUTO && call_min_ != 0) {
+    uint64_t dense_bytes = 0;
+    for (const LayerPlan& p : plans) dense_bytes += p.dense ? p.layer_bytes : 0;
+    if (dense_bytes >= call_min_) {
+      for (LayerPlan& p : plans) p.staged = p.staged || (p.dense && p.layer_bytes >= kMinStagedLayerBytes);
+    }
   }
   const bool want_events = !layer_events_.empty();
   if (plans.empty()) {

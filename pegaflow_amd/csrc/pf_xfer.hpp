@@ -48,6 +48,9 @@ constexpr uint64_t kDefaultAutoStagedMin = 16ull << 20;
 // scatter launch, while together they stay below this size and count: the
 // copies of a group still take well under a millisecond, so the pipeline
 // keeps its grain.
+// Layers below this size stay with the zero-copy kernel even in a call that
+// is staged for its total size.
+constexpr uint64_t kMinStagedLayerBytes = 32ull << 10;
 constexpr uint64_t kStagedGroupBytes = 32ull << 20;
 constexpr size_t kStagedGroupUnits = 16;
 constexpr int kDefaultUnroll = 4;
@@ -79,6 +82,7 @@ class Xfer {
       if (cfg->staging_slots) n_slots_ = cfg->staging_slots;
       if (cfg->zerocopy_max_workgroups) zc_max_wg_ = cfg->zerocopy_max_workgroups;
       if (cfg->auto_staged_min_bytes) auto_min_ = cfg->auto_staged_min_bytes;
+      call_min_ = cfg->auto_staged_min_call_bytes;
       if (cfg->tile_unroll) unroll_ = static_cast<int>(cfg->tile_unroll);
       if (cfg->copy_stream) copy_stream_ = cfg->copy_stream;
     }
@@ -208,6 +212,7 @@ class Xfer {
   uint32_t n_slots_ = kDefaultSlots;
   uint32_t zc_max_wg_ = 0;  // 0 = by fragment size (zero_copy_workgroups)
   uint64_t auto_min_ = kDefaultAutoStagedMin;
+  uint64_t call_min_ = 0;  // PF_PATH_AUTO: stage every dense layer of a call that moves this much (0 = off)
   int unroll_ = kDefaultUnroll;
 
   hipStream_t side_ = nullptr;

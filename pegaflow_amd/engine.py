@@ -235,10 +235,12 @@ class PegaEngine:
                  use_descriptor_backends: bool = False, unit_size_hint: int = 0,
                  lease_ttl_ms: int = 0, auto_staged_min_bytes: int = 0):
         """``lease_ttl_ms``: how long an unconsumed query lease pins its blocks
-        (0 = the reference's 600 s, lease.rs:11).  ``auto_staged_min_bytes``: the
-        smallest dense transfer the workers stage through device memory instead
-        of moving it with the resident zero-copy kernel (0 = 1 MiB per layer); lower it
-        where short model kernels run beside the transfers."""
+        (0 = the reference's 600 s, lease.rs:11).  ``auto_staged_min_bytes``: a
+        task whose dense layers add up to this much is staged through device
+        memory by the workers instead of moved with the resident zero-copy
+        kernel (0 = 8 MiB; layers of 16 MiB and more are staged in any case);
+        1 = stage whatever can be staged, for servers that would rather
+        lengthen small loads than disturb the model's kernels."""
         self._lib = _lib.load()
         cfg = _lib.PfEngineConfig(pool_size, int(use_hugepages), int(numa_aware), pool_shards,
                                   int(blockwise_alloc), int(ssd_enabled),

@@ -602,3 +602,49 @@ def test_small_staged_layers_share_slots_and_launches(stream, copy_stream):
     for c in cases:
         c.close()
     pool.close()
+
+
+def test_call_size_rule_stages_small_layers_of_a_long_call(stream):
+    """auto_staged_min_call_bytes: PF_PATH_AUTO stages the dense layers of a
+    call whose dense bytes reach the threshold even though no layer reaches
+    the per-layer threshold; a shorter call stays zero-copy; the bytes are
+    the oracle's either way."""
+    rng = np.random.default_rng(91)
+    xfer = BlockTransfer(auto_staged_min_call_bytes=2 << 20)   # per-layer default: 16 MiB
+    for n_ids, want in ((40, ST), (8, ZC)):                       # 4 x 640 KiB = 2.5 MiB | 4 x 128 KiB
+        cases = [Case(rng, num_blocks=64, seg=8192, segments=2, n_ids=n_ids) for _ in range(4)]
+        hosts, layers = [], []
+        for li, c in enumerate(cases):
+            L = c.product_layout()
+            h = PinnedMemory(2 * n_ids * L.host_stride)
+            h.as_numpy()[:] = SENT
+            hosts.append(h)
+            c.dev.copy_from_host(c.cache0)
+            layers.append(_dense_layer(c, L, h, c.ids))
+        xfer.save(layers, stream, TransferPath.AUTO)
+        stream.synchronize()
+        assert xfer.last_path == want
+        for c, h in zip(cases, hosts):
+            L = c.product_layout()
+            n, stride = n_ids, L.host_stride
+            oc = c.cache0.copy()
+            ok = np.full(n * stride, SENT, dtype=np.uint8)
+            ov = np.full(n * stride, SENT, dtype=np.uint8)
+            O.transfer_layer(c.oracle_layout(oc), c.ids, ok, ov, host_is_src=False)
+            assert np.array_equal(h.as_numpy()[: n * stride], ok)
+            assert np.array_equal(h.as_numpy()[n * stride:], ov)
+            c.dev.fill(SENT)
+        xfer.load(layers, stream, TransferPath.AUTO)
+        stream.synchronize()
+        assert xfer.last_path == want
+        for c, h in zip(cases, hosts):
+            L = c.product_layout()
+            n, stride = n_ids, L.host_stride
+            oc = np.full_like(c.cache0, SENT)
+            hv = h.as_numpy()
+            O.transfer_layer(c.oracle_layout(oc), c.ids, hv[: n * stride].copy(),
+                             hv[n * stride:].copy(), host_is_src=True)
+            assert np.array_equal(c.dev.copy_to_host(), oc)
+            c.close()
+            h.close()
+    xfer.close()
