@@ -1028,7 +1028,85 @@ def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, pa
     out["load_gbps_all"] = [round(payload / t / 1e9, 2) for t in load_s]
     out["query_ms"] = round(min(query_s) * 1e3, 2)
     out["blocks"] = n
+    if not w["page_first"]:
+        out["small_tasks_beside_short_kernels"] = engine_beside_short_kernels(
+            torch, eng, names, save_ids, n_layers * nseg * seg)
     eng.close()
+    return out
+
+
+def engine_beside_short_kernels(torch, eng, names, save_ids, bytes_per_block, blocks=64, m=2048,
+                                seconds=0.8):
+    """What the engine's small tasks cost kernels that run beside them: a stream of
+    back-to-back m^3 bf16 GEMMs (23 us each at 2048) alone, then beside an unbroken
+    loop of save -> query -> load of `blocks` blocks per layer through the engine
+    (4 MiB per layer at the Llama shape).  The workers of a `direct` / `kernel`
+    instance stage such a task, those of a `zerocopy` instance move it with the
+    resident kernel; the bench line carries both."""
+    import threading
+    from pegaflow_amd.engine import LayerSave
+    dev = torch.device("cuda:0")
+    a = torch.randn(m, m, device=dev, dtype=torch.bfloat16)
+    b = torch.randn(m, m, device=dev, dtype=torch.bfloat16)
+    c = torch.empty(m, m, device=dev, dtype=torch.bfloat16)
+    gemm_stream = torch.cuda.Stream()
+    ids = [int(i) for i in save_ids[:blocks]]
+    stop = threading.Event()
+    moved = {"bytes": 0, "seconds": 0.0, "error": None}
+
+    def mover():
+        salt = 0
+        t0 = time.perf_counter()
+        try:
+            while not stop.is_set():
+                salt += 1
+                hashes = [b"k" + salt.to_bytes(4, "little") + i.to_bytes(4, "little") + bytes(23)
+                          for i in range(len(ids))]
+                eng.batch_save_kv_blocks("bench-src", 0, 0, 0,
+                                         [LayerSave(nm, ids, hashes) for nm in names])
+                hits, lease = eng.query_prefix("bench-dst", hashes)
+                task = eng.batch_load_kv_blocks_multi_layer("bench-dst", 0, 0, [names], lease, [ids])
+                task.wait()
+                task.close()
+                moved["bytes"] += 2 * len(ids) * bytes_per_block
+                if salt % 64 == 0:
+                    eng.evict_all()
+        except Exception as exc:  # reported, the bench goes on
+            moved["error"] = str(exc)
+        moved["seconds"] = time.perf_counter() - t0
+
+    def gemm_tflops(span):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        count = 0
+        with torch.cuda.stream(gemm_stream):
+            e0.record()
+            t0 = time.perf_counter()
+            while time.perf_counter() - t0 < span:
+                for _ in range(256):
+                    torch.matmul(a, b, out=c)
+                count += 256
+                if count % 4096 == 0:
+                    gemm_stream.synchronize()   # keep the backlog bounded
+            e1.record()
+        e1.synchronize()
+        return 2.0 * m ** 3 * count / (e0.elapsed_time(e1) / 1e3) / 1e12
+
+    gemm_tflops(0.2)
+    alone = gemm_tflops(seconds)
+    thread = threading.Thread(target=mover)
+    thread.start()
+    time.sleep(0.1)
+    beside = gemm_tflops(seconds)
+    stop.set()
+    thread.join()
+    eng.evict_all()
+    out = {"gemm": f"{m}x{m}x{m} bf16", "blocks_per_layer": len(ids),
+           "task_mib": round(len(ids) * bytes_per_block / 2 ** 20, 1),
+           "gemm_alone_tflops": round(alone, 1), "gemm_beside_tflops": round(beside, 1),
+           "gemm_share_kept": round(beside / alone, 3),
+           "engine_save_plus_load_gbps": round(moved["bytes"] / max(moved["seconds"], 1e-9) / 1e9, 2)}
+    if moved["error"]:
+        out["error"] = moved["error"]
     return out
 
 
