@@ -683,7 +683,7 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
       }
       // Staged loads visit each unit's positions in ascending destination id
       // (launch_block_tiles); layers with the same ids and unit size share it.
-      if (!save && p.staged && p.n_blocks > 1) {
+      if (!save && p.staged && p.n_blocks > 1 && p.layer_bytes >= kRowOrderFromBytes) {
         p.ordered = true;
         for (size_t pj = 0; pj < pi; ++pj) {
           if (plans[pj].ordered && plans[pj].ids_slab_off == p.ids_slab_off &&

@@ -51,6 +51,10 @@ constexpr uint64_t kDefaultAutoStagedMin = 16ull << 20;
 // Layers below this size stay with the zero-copy kernel even in a call that
 // is staged for its total size.
 constexpr uint64_t kMinStagedLayerBytes = 32ull << 10;
+// Staged loads of layers from this size on scatter in ascending destination id
+// (an HBM-rate matter); below it the order array's upload costs more than the
+// scatter could gain.
+constexpr uint64_t kRowOrderFromBytes = 4ull << 20;
 constexpr uint64_t kStagedGroupBytes = 32ull << 20;
 constexpr size_t kStagedGroupUnits = 16;
 constexpr int kDefaultUnroll = 4;
