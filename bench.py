@@ -91,12 +91,15 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload",
-                    choices=sorted(WORKLOADS) + ["ref_transfer_bench", "ref_cpu_path"],
+                    choices=sorted(WORKLOADS) + ["ref_transfer_bench", "ref_cpu_path",
+                                                 "link_after_free"],
                     default="llama8b",
                     help="ref_transfer_bench = the shapes of the reference's own "
                          "benches/transfer_h2d.rs through the descriptor backends; "
                          "ref_cpu_path = the engine-level groups of its benches/cpu_path.rs "
-                         "(long lists of 1 KiB blocks through save / query / load)")
+                         "(long lists of 1 KiB blocks through save / query / load); "
+                         "link_after_free = what a large hipFree does to the link copies that "
+                         "follow it")
     ap.add_argument("--path", choices=["auto", "staged", "zerocopy"], default="auto")
     ap.add_argument("--layers", type=int, default=0, help="override the layer count")
     ap.add_argument("--slot-mb", type=int, default=0)
@@ -120,12 +123,18 @@ def parse_args():
                          "the descriptor backends, as the reference's workers do")
     ap.add_argument("--engine-child", action="store_true",
                     help="(internal) run only the engine section and print its JSON")
+    ap.add_argument("--engine-lazy-staging", action="store_true",
+                    help="engine section: the workers allocate their staging slots on the first "
+                         "staged task instead of at registration (pf_engine_config.lazy_staging)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--ref-fragments", type=int, default=0,
                     help="ref_transfer_bench: only this fragment count (default: 1024..65536)")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--settle-max", type=int, default=8,
-                    help="upper bound on the untimed passes run after the warmup until two agree")
+    ap.add_argument("--no-extra-workloads", action="store_true",
+                    help="default run only: skip the configs[3] and configs[4] workloads that "
+                         "follow the headline one (the `workloads` key)")
+    ap.add_argument("--free-gib", type=int, default=40,
+                    help="link_after_free: GiB of device memory to allocate, touch and free")
     return ap.parse_args()
 
 
@@ -167,23 +176,159 @@ def main():
     import numpy as np
     import torch
 
+    from pegaflow_amd import runtime
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    runtime.set_device(0)
+
+    if args.workload == "ref_transfer_bench":
+        run_ref_transfer_bench(torch, np, args)
+        return
+    if args.workload == "link_after_free":
+        print(json.dumps(run_link_after_free(runtime, args.free_gib)))
+        return
+    if args.engine_child:
+        print(json.dumps(run_workload(args, args.workload, {"engine_child"}, torch, np)))
+        return
+    sections = set()
+    if not args.no_overlap:
+        sections |= {"overlap", "duplex"}
+    if not args.no_engine:
+        sections.add("engine")
+    if not args.no_cpu:
+        sections.add("cpu")
+    result = run_workload(args, args.workload, sections, torch, np)
+    # The other two GPU configurations of the benchmark in the same run, as the
+    # reference's own transfer bench sweeps its shapes in one run
+    # (benches/transfer_h2d.rs:62-109): timed steps, byte check, link and kernel
+    # roofline each; the headline keys above stay those of the first workload.
+    default_run = (args.workload == "llama8b" and args.path == "auto" and not args.layers
+                   and not args.no_extra_workloads)
+    if default_run:
+        keys = ("value", "save_gbps", "load_gbps", "ms_per_step", "step_save_load_ms", "config",
+                "roofline", "link", "link_settle", "byte_checks", "verified")
+        workloads = {"llama8b": {k: result[k] for k in keys}}
+        for name in ("llama70b_fp8", "dsv3_mla"):
+            extra = run_workload(args, name, set(), torch, np)
+            workloads[name] = {k: extra[k] for k in keys}
+        result["workloads"] = workloads
+    print(json.dumps(result))
+
+
+_SETTLE = {}
+
+
+def wait_for_link(runtime, limit_s=20.0):
+    """Wait until host -> device copies run at the link's rate again.
+
+    Freeing device memory is followed by a stretch during which the runtime's
+    host -> device copies run at half their rate while device -> host copies
+    and kernels that read host memory are unaffected (`--workload
+    link_after_free` shows it: about 50 ms per GiB freed, in the freeing process
+    and in any other).  A process that starts right after another one released
+    tens of GiB -- this bench's own engine child, or the bench after a test run
+    -- would otherwise time that aftermath.  Copies of 256 MiB each way until
+    three host -> device copies in a row reach 0.95 of the device -> host rate;
+    no workload bytes move.  Returns what it saw."""
+    from pegaflow_amd.runtime import DeviceBuffer, Event, PinnedMemory, Stream
+    size = 256 << 20
+    if not _SETTLE:   # kept for the life of the process: freeing them would restart the effect
+        _SETTLE.update(pin=PinnedMemory(2 * size), dev=DeviceBuffer(2 * size), stream=Stream(),
+                       ev=[Event(timing=True), Event(timing=True), Event(timing=True)])
+    pin, dev, stream, ev = _SETTLE["pin"], _SETTLE["dev"], _SETTLE["stream"], _SETTLE["ev"]
+    t0 = time.perf_counter()
+    first = None
+    good = samples = 0
+    while True:
+        ev[0].record(stream)
+        runtime.memcpy_d2h_async(pin.host_ptr, dev.ptr, size, stream)
+        ev[1].record(stream)
+        runtime.memcpy_h2d_async(dev.ptr + size, pin.host_ptr + size, size, stream)
+        ev[2].record(stream)
+        ev[2].synchronize()
+        d2h = size / ev[0].elapsed_ms(ev[1]) / 1e6
+        h2d = size / ev[1].elapsed_ms(ev[2]) / 1e6
+        samples += 1
+        if samples == 1:
+            continue   # the first copy of a stream carries its set-up
+        if first is None:
+            first = h2d
+        good = good + 1 if h2d >= 0.95 * d2h else 0
+        waited = time.perf_counter() - t0
+        if good >= 3 or waited > limit_s:
+            return {"waited_ms": round(waited * 1e3, 1), "copies": samples,
+                    "first_h2d_gbps": round(first, 2), "last_h2d_gbps": round(h2d, 2),
+                    "d2h_gbps": round(d2h, 2), "settled": good >= 3}
+
+
+def run_link_after_free(runtime, gib):
+    """Allocate, touch and free `gib` GiB of device memory, then time 327 MB
+    copies each way, one at a time, for a few seconds: how long and how much the
+    copies that follow a large hipFree are slowed."""
+    from pegaflow_amd.runtime import DeviceBuffer, Event, PinnedMemory, Stream
+    piece = 327_680_000
+    pin, dev = PinnedMemory(2 * piece), DeviceBuffer(2 * piece)
+    sa, sb = Stream(), Stream()
+    ev = [Event(timing=True) for _ in range(4)]
+
+    def sample(seconds):
+        rows, t0 = [], time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            ev[0].record(sa)
+            runtime.memcpy_d2h_async(pin.host_ptr, dev.ptr, piece, sa)
+            ev[1].record(sa)
+            ev[1].synchronize()
+            ev[2].record(sb)
+            runtime.memcpy_h2d_async(dev.ptr + piece, pin.host_ptr + piece, piece, sb)
+            ev[3].record(sb)
+            ev[3].synchronize()
+            rows.append((time.perf_counter() - t0, ev[0].elapsed_ms(ev[1]), ev[2].elapsed_ms(ev[3])))
+        return rows
+
+    sample(0.2)
+    before = sample(0.5)
+    bufs = []
+    for i in range(gib):
+        b = DeviceBuffer(1 << 30)
+        b.fill(i + 1)
+        bufs.append(b)
+    runtime.device_synchronize()
+    t0 = time.perf_counter()
+    for b in bufs:
+        b.close()
+    free_s = time.perf_counter() - t0
+    after = sample(max(3.0, 0.12 * gib))
+    norm_h2d = sorted(r[2] for r in before)[len(before) // 2]
+    norm_d2h = sorted(r[1] for r in before)[len(before) // 2]
+    slow = [r for r in after if r[2] > 1.2 * norm_h2d]
+    return {"metric": "link copies after hipFree", "unit": "ms per 327.68 MB copy",
+            "freed_gib": gib, "free_call_s": round(free_s, 3),
+            "before": {"h2d_ms": round(norm_h2d, 2), "d2h_ms": round(norm_d2h, 2)},
+            "after": {"h2d_ms_max": round(max(r[2] for r in after), 2),
+                      "d2h_ms_max": round(max(r[1] for r in after), 2),
+                      "slow_h2d_copies": len(slow),
+                      "last_slow_h2d_at_s": round(slow[-1][0], 2) if slow else 0.0,
+                      "slow_h2d_ms_median": round(sorted(r[2] for r in slow)[len(slow) // 2], 2)
+                      if slow else None},
+            "device": runtime.device_name(0)}
+
+
+def run_workload(args, workload, sections, torch, np):
+    """One workload of WORKLOADS end to end: inputs, timed steps, byte check,
+    link peak, kernel roofline and the sections asked for ("overlap", "duplex",
+    "engine", "cpu"); returns the result line as a dict.  {"engine_child"} runs
+    only the engine section in this process and returns its dict."""
     from pegaflow_amd import _lib, runtime
     from pegaflow_amd.layout import KVCacheLayout
     from pegaflow_amd.pool import LayerTopology, WorkerLayers
     from pegaflow_amd.runtime import Event, PinnedMemory, Stream
     from pegaflow_amd.transfer import BlockTransfer, LayerBlocks, TransferPath
 
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
-    torch.cuda.set_device(0)
-    runtime.set_device(0)
     dev = torch.device("cuda:0")
     path = {"auto": TransferPath.AUTO, "staged": TransferPath.STAGED,
             "zerocopy": TransferPath.ZEROCOPY}[args.path]
-
-    if args.workload == "ref_transfer_bench":
-        run_ref_transfer_bench(torch, np, args)
-        return
-    w = WORKLOADS[args.workload]
+    w = WORKLOADS[workload]
     n_layers = args.layers or w["layers"]
     nb, seg, n = w["num_blocks"], w["seg"], w["n"]
     nseg = 2 if w["split"] else 1
@@ -214,15 +359,16 @@ def main():
     dst_cache = [new_cache(False) for _ in range(n_layers)]
     save_ids = make_ids(np, w["ids"], nb, n, args.seed)
     load_ids = make_ids(np, "permutation", nb, n, args.seed + 1)
-    if args.engine_child:
+    if "engine_child" in sections:
         torch.cuda.synchronize()
-        print(json.dumps(run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids,
-                                    payload, args.engine_mode, args.engine_descriptors)))
-        return
+        return run_engine(torch, np, runtime, w, names, src_cache, dst_cache, save_ids, load_ids,
+                          payload, args.engine_mode, args.engine_descriptors,
+                          args.engine_lazy_staging)
     t0 = time.time()
     pool = PinnedMemory(payload)
     pool_alloc_s = time.time() - t0
     torch.cuda.synchronize()
+    link_settle = wait_for_link(runtime)
 
     def layouts_for(caches):
         kv = nb * seg if w["split"] else 0
@@ -288,17 +434,6 @@ def main():
 
     for _ in range(args.warmup):
         one_step()
-    # A process that starts right after another one released tens of GiB of
-    # device and pinned memory sees the driver's clean-up of that memory as
-    # slower passes for a second or two.  Untimed passes until two in a row
-    # agree (bounded) keep that out of the timed steps; the count is reported.
-    settle_steps, prev = 0, None
-    while settle_steps < args.settle_max:
-        cur = sum(one_step())
-        settle_steps += 1
-        if prev is not None and abs(cur - prev) <= 0.015 * min(cur, prev):
-            break
-        prev = cur
     torch.cuda.synchronize()
     stream.synchronize()
     save_ms = load_ms = 0.0
@@ -408,7 +543,7 @@ def main():
     staged_path = used_path == "staged"
     alg_bytes = (2 if staged_path else 1) * bytes_per_launch
     achieved = alg_bytes / (live_launch_ms / 1e3) / 1e9
-    traffic, traffic_source = (measured_traffic(args.workload, alg_bytes) if staged_path
+    traffic, traffic_source = (measured_traffic(workload, alg_bytes) if staged_path
                                else (None, "zero-copy launches are not profiled for HBM traffic"))
     # What a pair of events reads with nothing between them on that stream: the
     # part of avg_launch_us that is the bracket itself, not the kernel (reported,
@@ -467,14 +602,14 @@ def main():
 
     # ---- compute overlap (configs[2]): transfers next to a GEMM stream ----
     overlap = None
-    if not args.no_overlap:
+    if "overlap" in sections:
         overlap = run_overlap(torch, xfer, save_layers, load_layers, stream, path, payload, n_layers,
                               checker, pool, m=args.gemm_m)
 
     # ---- both directions at once (the worker pool runs a load thread and a
     # save thread per GPU: gpu_worker.rs:116-345 of the reference) ----------
     duplex = None
-    if not args.no_overlap:
+    if "duplex" in sections:
         pool2 = PinnedMemory(payload)
         duplex = run_duplex(layers_for(src_cache, save_ids, pool2), load_layers, path, payload, args,
                             checker, pool, pool2, runtime)
@@ -491,15 +626,18 @@ def main():
     stream.close()
     pool.close()
     engine = None
-    if not args.no_engine:
+    del src_cache, dst_cache, save_layers, load_layers, scratch, scratch2
+    gc.collect()
+    torch.cuda.empty_cache()
+    if "engine" in sections:
         import subprocess
-        del src_cache, dst_cache, save_layers, load_layers, scratch, scratch2
-        torch.cuda.empty_cache()
         def engine_run(mode):
             cmd = [sys.executable, os.path.abspath(__file__), "--engine-child", "--workload",
-                   args.workload, "--seed", str(args.seed), "--engine-mode", mode]
+                   workload, "--seed", str(args.seed), "--engine-mode", mode]
             if args.engine_descriptors:
                 cmd.append("--engine-descriptors")
+            if args.engine_lazy_staging:
+                cmd.append("--engine-lazy-staging")
             if args.layers:
                 cmd += ["--layers", str(args.layers)]
             proc = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
@@ -517,7 +655,7 @@ def main():
 
     # ---- CPU baseline: the oracle's memcpy executor on the host cores -----
     cpu = None
-    if not args.no_cpu:
+    if "cpu" in sections:
         cpu = run_cpu_baseline(np, w, save_ids, load_ids, args.cpu_seconds, args.seed)
 
     result = {
@@ -542,7 +680,7 @@ def main():
                    "copy_stream": args.copy_stream},
         "save_gbps": round(save_gbps, 3),
         "step_save_load_ms": step_times[:16],
-        "settle_steps": settle_steps,
+        "link_settle": link_settle,
         "load_gbps": round(load_gbps, 3),
         "roofline": roofline,
         "link": link,
@@ -551,10 +689,11 @@ def main():
         "duplex": duplex,
         "engine": engine,
         "byte_checks": byte_checks,
+        "verified": True,   # a failed byte check ends the run with exit status 1
         "pool_alloc_s": round(pool_alloc_s, 2),
         "device": runtime.device_name(0),
     }
-    print(json.dumps(result))
+    return result
 
 
 class ByteChecker:
@@ -925,19 +1064,22 @@ def run_ref_cpu_path():
         "table": rows}))
 
 
-def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, payload,
-               mode_name="direct", descriptors=False):
+def run_engine(torch, np, runtime, w, names, src_cache, dst_cache, save_ids, load_ids, payload,
+               mode_name="direct", descriptors=False, lazy_staging=False):
     """End to end through pf_engine_*: registration, batch_save (host image
     allocation in the pinned pool, one worker task, block bookkeeping), prefix
     query, batch_load into a second instance of the same namespace.  Times are
-    wall clock around the C calls with the arguments packed beforehand."""
+    wall clock around the C calls with the arguments packed beforehand.  The
+    first repetition is the first task each worker ever sees; `*_gbps` are
+    medians, `*_gbps_first` and `*_gbps_all` are beside them, and every load
+    carries its phase profile (pf_task_result)."""
     from pegaflow_amd.engine import LayerSave, LoadState, PackedSaves, PegaEngine
     from pegaflow_amd.transfer import TransferMode
     nb, seg, n = w["num_blocks"], w["seg"], w["n"]
     nseg = 2 if w["split"] else 1
     n_layers = len(names)
     eng = PegaEngine(pool_size=int(payload * 2.3) + (256 << 20),
-                     use_descriptor_backends=descriptors)
+                     use_descriptor_backends=descriptors, lazy_staging=lazy_staging)
     kv = nb * seg if nseg == 2 else 0
     for inst, caches in (("bench-src", src_cache), ("bench-dst", dst_cache)):
         eng.register_context_layer_batch(
@@ -950,9 +1092,14 @@ def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, pa
     for t in dst_cache:
         t.zero_()
     torch.cuda.synchronize()
-    out = {"transfer_mode": mode_name, "worker_form": "descriptors" if descriptors else "block ids"}
-    reps = 3
-    save_s, load_s, query_s = [], [], []
+    # This process starts right after the parent released its caches.
+    link_settle = wait_for_link(runtime)
+    out = {"transfer_mode": mode_name, "worker_form": "descriptors" if descriptors else "block ids",
+           "link_settle": link_settle,
+           "staging_mib_after_registration": eng.staging_bytes >> 20,
+           "lazy_staging": bool(lazy_staging)}
+    reps = 5
+    save_s, load_s, query_s, load_profiles = [], [], [], []
     for rep in range(reps):
         hashes = [bytes([rep]) + int(i).to_bytes(4, "little") + bytes(27) for i in range(n)]
         packed = PackedSaves([LayerSave(nm, save_ids, hashes) for nm in names])
@@ -970,6 +1117,10 @@ def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, pa
         res = task.wait()   # raises if the load failed
         load_s.append(time.perf_counter() - t0)
         assert res.done and state.get() == 1, "engine load did not complete"
+        load_profiles.append({"paths": list(res.paths), "staged_groups": res.staged_groups,
+                              "zero_copy_launches": res.zero_copy_launches,
+                              "elapsed_ms": round(res.elapsed_ms, 2),
+                              **{k: round(v, 2) for k, v in res.phases_ms.items()}})
         task.close()
         state.close()
         if rep == reps - 1:
@@ -1022,11 +1173,19 @@ def run_engine(torch, np, w, names, src_cache, dst_cache, save_ids, load_ids, pa
             "aggregate_gbps": round(2 * payload / span / 1e9, 2)}
     except Exception as exc:  # pool too small for two images, etc.: report, do not fail the bench
         out["concurrent_save_and_load"] = {"error": str(exc)}
-    out["save_gbps"] = round(payload / min(save_s) / 1e9, 2)
-    out["load_gbps"] = round(payload / min(load_s) / 1e9, 2)
+    median = lambda xs: sorted(xs)[len(xs) // 2]
+    out["save_gbps"] = round(payload / median(save_s) / 1e9, 2)
+    out["load_gbps"] = round(payload / median(load_s) / 1e9, 2)
+    out["save_gbps_first"] = round(payload / save_s[0] / 1e9, 2)
+    out["load_gbps_first"] = round(payload / load_s[0] / 1e9, 2)
+    out["first_over_median"] = {"save": round(median(save_s) / save_s[0], 4),
+                                "load": round(median(load_s) / load_s[0], 4)}
     out["save_gbps_all"] = [round(payload / t / 1e9, 2) for t in save_s]
     out["load_gbps_all"] = [round(payload / t / 1e9, 2) for t in load_s]
-    out["query_ms"] = round(min(query_s) * 1e3, 2)
+    out["load_profile_first"] = load_profiles[0]
+    out["load_profile_median_rep"] = load_profiles[load_s.index(median(load_s))]
+    out["staging_mib"] = eng.staging_bytes >> 20
+    out["query_ms"] = round(median(query_s) * 1e3, 2)
     out["blocks"] = n
     if not w["page_first"]:
         out["small_tasks_beside_short_kernels"] = engine_beside_short_kernels(

@@ -196,12 +196,23 @@ typedef struct pf_merged_range {
   uint64_t size;
 } pf_merged_range;
 
-#define PF_MODE_DIRECT 0 /* one DMA copy per merged range ("direct") */
-#define PF_MODE_KERNEL 1 /* one copy kernel over mapped host memory ("kernel") */
+/* As descriptor backends (pf_backend_create) the first two are the reference's:
+ * "direct" issues DMA copies of the merged ranges, "kernel" one copy kernel
+ * over mapped host memory.  As the mode of a worker pool or of an engine
+ * registration they DEVIATE from the reference (gpu_worker.rs:264-276, where
+ * Kernel selects the copy-kernel backend): both let the block-ID engine pick
+ * the way across the link per task (PF_PATH_AUTO), because a copy kernel that
+ * stays resident for a long transfer slows the model's kernels beside it; the
+ * bytes moved are the same.  pf_task_result.paths says which way a task went,
+ * the pool logs its choice once when it is spawned, and
+ * pf_engine_config.kernel_mode_zerocopy gives PF_MODE_KERNEL registrations the
+ * reference's behaviour. */
+#define PF_MODE_DIRECT 0
+#define PF_MODE_KERNEL 1
 /* Worker pools and engine registrations only (not a descriptor backend, not a
- * name the connector sends): always the zero-copy kernel, whatever the size.
- * For instances that offload while the GPU is otherwise idle; see
- * pf_worker_pool_spawn. */
+ * name the connector sends): always the zero-copy kernel, whatever the size,
+ * and no staging memory.  For instances that offload while the GPU is otherwise
+ * idle; see pf_worker_pool_spawn. */
 #define PF_MODE_ZEROCOPY 2
 
 typedef struct pf_backend_s* pf_backend_t;
@@ -520,11 +531,35 @@ int pf_load_state_set(pf_load_state_t s, int64_t state); /* 1 or -1 */
 typedef struct pf_worker_pool_s* pf_worker_pool_t;
 typedef struct pf_task_s* pf_task_t;
 
+/* Ways a task's bytes crossed the link (bits of pf_task_result.paths; a task of
+ * mixed layers can carry more than one). */
+#define PF_TASK_PATH_STAGED 1u      /* device gather/scatter + DMA copies of a staging slot */
+#define PF_TASK_PATH_ZEROCOPY 2u    /* block-ID kernel over mapped host memory */
+#define PF_TASK_PATH_DESCRIPTORS 4u /* per-fragment descriptors through a transfer backend */
+
+/* What a settled task reports: the reference's workers log bytes, duration and
+ * bandwidth per task (gpu_worker.rs:458-474,505-520); the rest says which way
+ * the bytes went and where the task's time was spent, phase by phase. */
 typedef struct pf_task_result {
   int32_t status;      /* PF_OK or an error status */
   int32_t done;        /* 0 while pending (only from pf_task_wait with a timeout) */
   uint64_t bytes;      /* payload bytes moved */
   double elapsed_ms;   /* descriptor/plan construction + enqueue + synchronise */
+  uint32_t paths;              /* PF_TASK_PATH_* bits */
+  uint32_t staged_groups;      /* staging-slot fills: one gather or scatter launch each */
+  uint32_t zero_copy_launches; /* launches of the block-ID kernel over host memory */
+  uint32_t link_copies;        /* DMA copies of the staged path */
+  double resolve_ms;       /* engine loads: leases -> host blocks on the calling thread */
+  double queue_ms;         /* submitted -> picked up by the worker thread */
+  double convert_ms;       /* worker: host blocks -> block-ID form or descriptors */
+  double plan_ms;          /* transfer engine: validation, unit and slab layout */
+  double staging_alloc_ms; /* device staging (re)allocated inside the task; 0 once the
+                              pool's slots fit (they are allocated when it is spawned) */
+  double enqueue_ms;       /* issuing copies and launches (row-order sort included) */
+  double sync_ms;          /* last enqueue -> completion event */
+  double device_first_ms;  /* on the device: first command of the task -> first staging
+                              slot filled (load) or drained (save), or first kernel done */
+  double device_ms;        /* on the device: first command -> last command done */
 } pf_task_result;
 
 /* GpuWorkerPool::spawn, gpu_worker.rs:131-201: a load thread and a save thread
@@ -540,6 +575,27 @@ typedef struct pf_task_result {
  * Initialisation errors are returned here, synchronously. */
 int pf_worker_pool_spawn(int device_id, int numa_node, int transfer_mode,
                          int use_descriptor_backends, pf_worker_pool_t* out);
+/* The same with the pool's knobs.  Each worker of a staging pool (block-ID
+ * engine, mode direct or kernel) holds two staging slots in device memory,
+ * allocated here -- everything a worker needs exists before its first task, as
+ * in init_worker (gpu_worker.rs:278-298) -- so a pool costs
+ * 2 workers x 2 x staging_slot_bytes of device memory (2 GiB at the default)
+ * for as long as it lives, plus 64 MiB each of device and pinned memory for
+ * priming the two copy directions. */
+typedef struct pf_worker_pool_config {
+  int32_t device_id;
+  int32_t numa_node;                /* < 0 = no pinning */
+  int32_t transfer_mode;            /* PF_MODE_* */
+  uint32_t use_descriptor_backends;
+  uint64_t staging_slot_bytes;      /* 0 = default (512 MiB); a task's layer larger than a
+                                       slot is moved in several fills */
+  uint64_t auto_staged_min_bytes;   /* 0 = default (8 MiB), see pf_engine_config */
+  uint32_t lazy_staging;            /* 1 = allocate the slots on the first staged task */
+  uint32_t reserved;
+} pf_worker_pool_config;
+int pf_worker_pool_spawn_ex(const pf_worker_pool_config* cfg, pf_worker_pool_t* out);
+/* Device memory the pool's workers hold for staging right now. */
+uint64_t pf_worker_pool_staging_bytes(pf_worker_pool_t p);
 int pf_worker_pool_destroy(pf_worker_pool_t p);
 /* A process's streams share a few hardware queues (GPU_MAX_HW_QUEUES, 4 by
  * default), and kernels of two streams on one queue run one after the other.
@@ -597,6 +653,19 @@ typedef struct pf_engine_config {
                                         that run beside the resident kernel slow down for as long as
                                         it runs, a staged copy leaves them alone: 1 = stage whatever
                                         can be staged, UINT64_MAX = only the large layers. */
+  uint64_t staging_slot_bytes;       /* upper bound of a worker's staging slot; 0 = default
+                                        (512 MiB).  Every registered context (instance, GPU)
+                                        holds 2 workers x 2 slots of min(this, what its layers
+                                        can fill: the largest layer, or a block's page for
+                                        page-first instances) in device memory from registration
+                                        on -- memory the serving framework's own budget does not
+                                        know about. */
+  uint32_t lazy_staging;             /* 1 = workers allocate their slots on the first staged
+                                        task instead of at registration (that task is slower) */
+  uint32_t kernel_mode_zerocopy;     /* 1 = a PF_MODE_KERNEL registration gets zero-copy workers
+                                        (PF_MODE_ZEROCOPY), which is what the reference's kernel
+                                        mode does (gpu_worker.rs:264-276); 0 = the per-task
+                                        choice described at PF_MODE_DIRECT */
 } pf_engine_config;
 
 typedef struct pf_layer_save {       /* LayerSave, block.rs:20-25 */
@@ -631,6 +700,13 @@ typedef struct pf_save_profile {
   uint64_t bytes;
 } pf_save_profile;
 int pf_engine_last_save_profile(pf_engine_t e, pf_save_profile* out);
+/* The load task that settled last on any worker pool of the engine: bytes,
+ * duration (what the reference logs per load, gpu_worker.rs:458-474), the way
+ * it crossed the link and its phases.  PF_ERR_STORAGE when no load has settled
+ * yet.  The same figures come back from pf_task_wait for the task itself. */
+int pf_engine_last_load_profile(pf_engine_t e, pf_task_result* out);
+/* Device memory the worker pools of all registered contexts hold for staging. */
+uint64_t pf_engine_staging_bytes(pf_engine_t e);
 /* Longest cached prefix of the hashes and a lease over those blocks (0 = none). */
 int pf_engine_query_prefix(pf_engine_t e, const char* instance_id,
                            const uint8_t* const* hashes, const uint32_t* hash_lens, uint64_t n,

@@ -34,6 +34,10 @@ PF_PATH_AUTO = 0
 PF_PATH_ZEROCOPY = 1
 PF_PATH_STAGED = 2
 
+PF_TASK_PATH_STAGED = 1
+PF_TASK_PATH_ZEROCOPY = 2
+PF_TASK_PATH_DESCRIPTORS = 4
+
 u64 = C.c_uint64
 u32 = C.c_uint32
 vp = C.c_void_p
@@ -115,14 +119,27 @@ class PfWorkerLayers(C.Structure):
 
 class PfTaskResult(C.Structure):
     _fields_ = [("status", C.c_int32), ("done", C.c_int32), ("bytes", u64),
-                ("elapsed_ms", C.c_double)]
+                ("elapsed_ms", C.c_double), ("paths", u32), ("staged_groups", u32),
+                ("zero_copy_launches", u32), ("link_copies", u32),
+                ("resolve_ms", C.c_double), ("queue_ms", C.c_double), ("convert_ms", C.c_double),
+                ("plan_ms", C.c_double), ("staging_alloc_ms", C.c_double),
+                ("enqueue_ms", C.c_double), ("sync_ms", C.c_double),
+                ("device_first_ms", C.c_double), ("device_ms", C.c_double)]
+
+
+class PfWorkerPoolConfig(C.Structure):
+    _fields_ = [("device_id", C.c_int32), ("numa_node", C.c_int32), ("transfer_mode", C.c_int32),
+                ("use_descriptor_backends", u32), ("staging_slot_bytes", u64),
+                ("auto_staged_min_bytes", u64), ("lazy_staging", u32), ("reserved", u32)]
 
 
 class PfEngineConfig(C.Structure):
     _fields_ = [("pool_size", u64), ("use_hugepages", u32), ("numa_aware", u32),
                 ("pool_shards", u32), ("blockwise_alloc", u32), ("ssd_enabled", u32),
                 ("use_descriptor_backends", u32), ("unit_size_hint", u64),
-                ("lease_ttl_ms", u64), ("auto_staged_min_bytes", u64)]
+                ("lease_ttl_ms", u64), ("auto_staged_min_bytes", u64),
+                ("staging_slot_bytes", u64), ("lazy_staging", u32),
+                ("kernel_mode_zerocopy", u32)]
 
 
 class PfIpcTensor(C.Structure):
@@ -252,6 +269,8 @@ PROTOTYPES = {
     "pf_load_state_get": (C.c_int64, [vp]),
     "pf_load_state_set": (C.c_int, [vp, C.c_int64]),
     "pf_worker_pool_spawn": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(vp)]),
+    "pf_worker_pool_spawn_ex": (C.c_int, [C.POINTER(PfWorkerPoolConfig), C.POINTER(vp)]),
+    "pf_worker_pool_staging_bytes": (u64, [vp]),
     "pf_worker_pool_destroy": (C.c_int, [vp]),
     "pf_worker_submit_load": (C.c_int, [vp, C.POINTER(PfLayerTransfer), u64, C.c_char_p,
                                         C.POINTER(vp)]),
@@ -278,6 +297,8 @@ PROTOTYPES = {
                                        C.POINTER(C.POINTER(C.c_int64)), u64, C.c_char_p,
                                        C.POINTER(vp)]),
     "pf_engine_last_save_profile": (C.c_int, [vp, C.POINTER(PfSaveProfile)]),
+    "pf_engine_last_load_profile": (C.c_int, [vp, C.POINTER(PfTaskResult)]),
+    "pf_engine_staging_bytes": (u64, [vp]),
     "pf_engine_batch_load_multi": (C.c_int, [vp, C.c_char_p, u64, C.c_int, u64,
                                              C.POINTER(C.POINTER(C.c_char_p)), C.POINTER(u64),
                                              C.POINTER(PfLoadRequest), u64, C.c_char_p,

@@ -23,6 +23,15 @@ int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 // hipError_t as a positive status.
 int fail_hip(hipError_t e, const char* what);
 
+// Diagnostics on stderr, one line per call, prefixed "pegahip:".  The level comes
+// from the environment variable PEGAHIP_LOG when the library is first used:
+// "off", "info" (the default: one line per worker pool that is spawned) or
+// "debug" (also one line per task, as the reference's workers log at debug
+// level, gpu_worker.rs:465-474,511-520).
+enum class LogLevel { Off = 0, Info = 1, Debug = 2 };
+LogLevel log_level();
+void log_line(LogLevel level, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
 struct Stream {
   hipStream_t s = nullptr;
   bool owned = false;

@@ -139,6 +139,13 @@ std::shared_ptr<LayerTopology> InstanceContext::sealed_topology(std::string* err
   return topology_;
 }
 
+std::vector<std::shared_ptr<GpuContext>> InstanceContext::gpus() {
+  std::lock_guard<std::mutex> lock(mu_);
+  std::vector<std::shared_ptr<GpuContext>> out;
+  for (auto& kv : gpus_) out.push_back(kv.second);
+  return out;
+}
+
 std::shared_ptr<GpuContext> InstanceContext::get_gpu(int device_id) {
   std::lock_guard<std::mutex> lock(mu_);
   auto it = gpus_.find(device_id);
@@ -288,9 +295,28 @@ int Engine::register_context_layer_batch_strided(
   if (st != PF_OK) return st;
   std::string werr;
   int wstatus = PF_ERR_DEVICE_INIT;
-  ctx->worker_pool = GpuWorkerPool::spawn(device_id, ctx->preferred_numa, mode,
-                                          cfg_.use_descriptor_backends, &werr, &wstatus,
-                                          cfg_.auto_staged_min_bytes);
+  WorkerPoolOptions options;
+  options.use_descriptor_backends = cfg_.use_descriptor_backends;
+  options.auto_staged_min_bytes = cfg_.auto_staged_min_bytes;
+  options.lazy_staging = cfg_.lazy_staging;
+  // A staging slot never holds more than one layer's blocks (layer-first) or
+  // the pages of one call (page-first: every layer's slice of a block), so a
+  // context of small layers gets small slots.  Small layers that follow one
+  // another share up to 32 MiB of a slot: that is the floor.
+  {
+    uint64_t fill = 0;
+    for (const auto& kv : ctx->reg.kv_caches) {
+      const uint64_t bytes = kv.second.block_bytes() * kv.second.num_blocks();
+      fill = page_first ? fill + bytes : std::max(fill, bytes);
+    }
+    constexpr uint64_t kSlotFloor = 32ull << 20, kSlotDefault = 512ull << 20;
+    const uint64_t cap = cfg_.staging_slot_bytes ? cfg_.staging_slot_bytes : kSlotDefault;
+    fill = (std::max(fill, kSlotFloor) + 0xFFFFFull) & ~0xFFFFFull;
+    options.staging_slot_bytes = std::min(cap, fill);
+  }
+  if (mode == TransferMode::Kernel && cfg_.kernel_mode_zerocopy) mode = TransferMode::ZeroCopy;
+  ctx->worker_pool = GpuWorkerPool::spawn(device_id, ctx->preferred_numa, mode, options, &werr,
+                                          &wstatus);
   if (!ctx->worker_pool) return bad(err, wstatus, werr);
   return instance->register_new_gpu(std::move(ctx), err);
 }
@@ -877,6 +903,43 @@ int Engine::create_group_lease(const std::string& instance_id, uint32_t group,
   return PF_OK;
 }
 
+bool Engine::last_load_profile(TaskResult* out) {
+  std::vector<std::shared_ptr<InstanceContext>> instances;
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    for (auto& kv : instances_) instances.push_back(kv.second);
+  }
+  bool found = false;
+  std::chrono::steady_clock::time_point newest;
+  for (auto& instance : instances) {
+    for (auto& gpu : instance->gpus()) {
+      TaskResult r;
+      std::chrono::steady_clock::time_point when;
+      if (gpu->worker_pool && gpu->worker_pool->last_load(&r, &when) && (!found || when > newest)) {
+        found = true;
+        newest = when;
+        *out = std::move(r);
+      }
+    }
+  }
+  return found;
+}
+
+uint64_t Engine::staging_bytes() {
+  std::vector<std::shared_ptr<InstanceContext>> instances;
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    for (auto& kv : instances_) instances.push_back(kv.second);
+  }
+  uint64_t total = 0;
+  for (auto& instance : instances) {
+    for (auto& gpu : instance->gpus()) {
+      if (gpu->worker_pool) total += gpu->worker_pool->staging_bytes();
+    }
+  }
+  return total;
+}
+
 SaveProfile Engine::last_save_profile() {
   std::lock_guard<std::mutex> lock(mu_);
   return last_save_profile_;
@@ -920,6 +983,7 @@ int Engine::batch_load_kv_blocks_multi_layer(
     const std::vector<std::vector<std::string>>& layer_groups,
     const std::vector<LoadRequest>& loads, const std::string& load_state_shm,
     std::future<TaskResult>* out, std::string* err) {
+  const auto t_resolve = std::chrono::steady_clock::now();
   auto instance = get_instance(instance_id, err);
   if (!instance) return PF_ERR_INSTANCE_MISSING;
   auto topo = instance->sealed_topology(err);
@@ -1121,6 +1185,8 @@ int Engine::batch_load_kv_blocks_multi_layer(
   }
   LoadCompletion completion;
   completion.load_state_shm = load_state_shm;
+  completion.resolve_ms = std::chrono::duration<double, std::milli>(
+                              std::chrono::steady_clock::now() - t_resolve).count();
   *out = gpu->worker_pool->submit_load(std::move(layers), std::move(completion));
   return PF_OK;
 }

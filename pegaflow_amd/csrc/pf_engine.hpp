@@ -38,6 +38,15 @@ struct EngineConfig {
   uint64_t lease_ttl_ms = 600000;
   // PF_PATH_AUTO threshold of the workers' transfer engines; 0 = the engine's default.
   uint64_t auto_staged_min_bytes = 0;
+  // Upper bound of one staging slot of a worker (0 = 512 MiB).  A context's
+  // pool holds 2 workers x 2 slots of min(this, what its layers can fill).
+  uint64_t staging_slot_bytes = 0;
+  // Workers allocate their staging on the first staged task, not at registration.
+  bool lazy_staging = false;
+  // Registrations that ask for TransferMode::Kernel get zero-copy workers (the
+  // reference's meaning of that mode: one copy kernel over mapped host memory,
+  // gpu_worker.rs:264-276) instead of the per-task choice.
+  bool kernel_mode_zerocopy = false;
 };
 
 // block.rs:20-25, as a view of the caller's arrays (valid for the call).
@@ -82,6 +91,7 @@ class InstanceContext {
   // Fails while workers are still registering.
   std::shared_ptr<LayerTopology> sealed_topology(std::string* err);
   std::shared_ptr<GpuContext> get_gpu(int device_id);
+  std::vector<std::shared_ptr<GpuContext>> gpus();
   std::string verify_topology(size_t tp_size, size_t world_size, bool page_first) const;
   const std::string& id() const { return id_; }
   const std::string& ns() const { return ns_; }
@@ -123,6 +133,12 @@ class Engine {
   int batch_save_kv_blocks(const std::string& instance_id, size_t tp_rank, size_t pp_rank,
                            int device_id, const std::vector<LayerSaveView>& saves, std::string* err);
   SaveProfile last_save_profile();
+  // The load task that settled last on any of the engine's worker pools (what
+  // the reference logs per load, gpu_worker.rs:458-474, plus its phases); false
+  // when none has.
+  bool last_load_profile(TaskResult* out);
+  // Device memory the worker pools of all registered contexts hold for staging.
+  uint64_t staging_bytes();
   // Longest cached prefix of `hashes` (group 0 keys) + a lease over those
   // blocks (lib.rs:506-546,614-629).
   int query_prefix(const std::string& instance_id, const std::vector<std::string_view>& hashes,

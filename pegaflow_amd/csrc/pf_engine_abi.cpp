@@ -149,25 +149,47 @@ int pf_load_state_set(pf_load_state_t s, int64_t state) {
 
 // ---- worker pool --------------------------------------------------------------
 
-int pf_worker_pool_spawn(int device_id, int numa_node, int transfer_mode,
-                         int use_descriptor_backends, pf_worker_pool_t* out) {
+int pf_worker_pool_spawn_ex(const pf_worker_pool_config* cfg, pf_worker_pool_t* out) {
+  PF_REQUIRE_PTR(cfg);
   PF_REQUIRE_PTR(out);
-  if (device_id < 0) return pf::fail(PF_ERR_INVALID_ARGUMENT, "device_id %d must be >= 0", device_id);
-  if (transfer_mode != PF_MODE_DIRECT && transfer_mode != PF_MODE_KERNEL &&
-      transfer_mode != PF_MODE_ZEROCOPY) {
-    return pf::fail(PF_ERR_INVALID_ARGUMENT, "unknown transfer mode %d", transfer_mode);
+  if (cfg->device_id < 0) {
+    return pf::fail(PF_ERR_INVALID_ARGUMENT, "device_id %d must be >= 0", cfg->device_id);
   }
+  if (cfg->transfer_mode != PF_MODE_DIRECT && cfg->transfer_mode != PF_MODE_KERNEL &&
+      cfg->transfer_mode != PF_MODE_ZEROCOPY) {
+    return pf::fail(PF_ERR_INVALID_ARGUMENT, "unknown transfer mode %d", cfg->transfer_mode);
+  }
+  pf::WorkerPoolOptions options;
+  options.use_descriptor_backends = cfg->use_descriptor_backends != 0;
+  options.staging_slot_bytes = cfg->staging_slot_bytes;
+  options.auto_staged_min_bytes = cfg->auto_staged_min_bytes;
+  options.lazy_staging = cfg->lazy_staging != 0;
   std::string err;
   int status = PF_ERR_DEVICE_INIT;
-  auto pool = pf::GpuWorkerPool::spawn(device_id, pf::NumaNode::from_int(numa_node),
-                                       static_cast<pf::TransferMode>(transfer_mode),
-                                       use_descriptor_backends != 0, &err, &status);
+  auto pool = pf::GpuWorkerPool::spawn(cfg->device_id, pf::NumaNode::from_int(cfg->numa_node),
+                                       static_cast<pf::TransferMode>(cfg->transfer_mode), options,
+                                       &err, &status);
   if (!pool) {
     pf::last_error() = err;
     return status;
   }
   *out = reinterpret_cast<pf_worker_pool_t>(pool.release());
   return PF_OK;
+}
+
+int pf_worker_pool_spawn(int device_id, int numa_node, int transfer_mode,
+                         int use_descriptor_backends, pf_worker_pool_t* out) {
+  pf_worker_pool_config cfg;
+  std::memset(&cfg, 0, sizeof(cfg));
+  cfg.device_id = device_id;
+  cfg.numa_node = numa_node;
+  cfg.transfer_mode = transfer_mode;
+  cfg.use_descriptor_backends = use_descriptor_backends != 0 ? 1u : 0u;
+  return pf_worker_pool_spawn_ex(&cfg, out);
+}
+
+uint64_t pf_worker_pool_staging_bytes(pf_worker_pool_t p) {
+  return p ? reinterpret_cast<pf::GpuWorkerPool*>(p)->staging_bytes() : 0;
 }
 
 uint64_t pf_worker_pool_queue_clashes(pf_worker_pool_t p) {
@@ -190,6 +212,27 @@ int pf_worker_stream_report(int device, uint64_t* out_streams, uint64_t* out_cla
 int pf_worker_pool_destroy(pf_worker_pool_t p) {
   delete reinterpret_cast<pf::GpuWorkerPool*>(p);
   return PF_OK;
+}
+
+static void fill_task_result(const pf::TaskResult& r, pf_task_result* out) {
+  std::memset(out, 0, sizeof(*out));
+  out->status = r.status;
+  out->done = 1;
+  out->bytes = r.bytes;
+  out->elapsed_ms = r.elapsed_ms;
+  out->paths = r.paths;
+  out->staged_groups = r.staged_groups;
+  out->zero_copy_launches = r.zero_copy_launches;
+  out->link_copies = r.link_copies;
+  out->resolve_ms = r.resolve_ms;
+  out->queue_ms = r.queue_ms;
+  out->convert_ms = r.convert_ms;
+  out->plan_ms = r.plan_ms;
+  out->staging_alloc_ms = r.staging_alloc_ms;
+  out->enqueue_ms = r.enqueue_ms;
+  out->sync_ms = r.sync_ms;
+  out->device_first_ms = r.device_first_ms;
+  out->device_ms = r.device_ms;
 }
 
 static int submit(pf_worker_pool_t p, const pf_layer_transfer* layers, uint64_t n_layers,
@@ -239,12 +282,7 @@ int pf_task_wait(pf_task_t t, int timeout_ms, pf_task_result* out) {
     h->result = h->fut.get();
     h->settled = true;
   }
-  if (out) {
-    out->status = h->result.status;
-    out->done = 1;
-    out->bytes = h->result.bytes;
-    out->elapsed_ms = h->result.elapsed_ms;
-  }
+  if (out) fill_task_result(h->result, out);
   if (h->result.status != PF_OK) pf::last_error() = h->result.message;
   return h->result.status;
 }
@@ -272,6 +310,9 @@ int pf_engine_create(const pf_engine_config* cfg, pf_engine_t* out) {
   c.unit_size_hint = cfg->unit_size_hint;
   if (cfg->lease_ttl_ms != 0) c.lease_ttl_ms = cfg->lease_ttl_ms;
   c.auto_staged_min_bytes = cfg->auto_staged_min_bytes;
+  c.staging_slot_bytes = cfg->staging_slot_bytes;
+  c.lazy_staging = cfg->lazy_staging != 0;
+  c.kernel_mode_zerocopy = cfg->kernel_mode_zerocopy != 0;
   std::string err;
   int status = PF_ERR_STORAGE;
   auto e = pf::Engine::create(c, &err, &status);
@@ -369,6 +410,21 @@ int pf_engine_last_save_profile(pf_engine_t e, pf_save_profile* out) {
   out->total_ms = p.total_ms;
   out->bytes = p.bytes;
   return PF_OK;
+}
+
+int pf_engine_last_load_profile(pf_engine_t e, pf_task_result* out) {
+  PF_REQUIRE_PTR(e);
+  PF_REQUIRE_PTR(out);
+  pf::TaskResult r;
+  if (!reinterpret_cast<pf::Engine*>(e)->last_load_profile(&r)) {
+    return pf::fail(PF_ERR_STORAGE, "no load task has settled on this engine yet");
+  }
+  fill_task_result(r, out);
+  return PF_OK;
+}
+
+uint64_t pf_engine_staging_bytes(pf_engine_t e) {
+  return e ? reinterpret_cast<pf::Engine*>(e)->staging_bytes() : 0;
 }
 
 int pf_engine_query_prefix(pf_engine_t e, const char* instance_id, const uint8_t* const* hashes,

@@ -1,5 +1,6 @@
 // Device, stream, event and raw device-memory entry points of the C ABI.
 // These are thin: they exist so that a host-side binding needs no HIP headers.
+#include <cstdlib>
 #include <cstring>
 #include <fstream>
 
@@ -33,6 +34,27 @@ int fail_hip(hipError_t e, const char* what) {
   // unrelated later call.
   (void)hipGetLastError();
   return static_cast<int>(e);
+}
+
+LogLevel log_level() {
+  static const LogLevel level = [] {
+    const char* v = std::getenv("PEGAHIP_LOG");
+    if (v == nullptr) return LogLevel::Info;
+    if (std::strcmp(v, "off") == 0 || std::strcmp(v, "0") == 0) return LogLevel::Off;
+    if (std::strcmp(v, "debug") == 0) return LogLevel::Debug;
+    return LogLevel::Info;
+  }();
+  return level;
+}
+
+void log_line(LogLevel level, const char* fmt, ...) {
+  if (static_cast<int>(level) > static_cast<int>(log_level())) return;
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  fprintf(stderr, "pegahip: %s\n", buf);
 }
 
 }  // namespace pf

@@ -10,6 +10,12 @@
 
 namespace pf {
 
+namespace {
+// The workers move KV beside a running model: a task whose dense layers add up
+// to this much is staged whatever the size of its layers (see run()).
+constexpr uint64_t kWorkerStagedCallBytes = 8ull << 20;
+}  // namespace
+
 bool build_copy_descs(const std::vector<LayerTransferData>& layers, std::vector<CopyDesc>* out,
                       uint64_t* total_bytes, std::string* err, size_t begin, size_t end) {
   out->clear();
@@ -281,13 +287,12 @@ bool to_block_form(const std::vector<LayerTransferData>& all_layers, size_t begi
 
 std::unique_ptr<GpuWorkerPool> GpuWorkerPool::spawn(int device_id, NumaNode numa_node,
                                                     TransferMode mode,
-                                                    bool use_descriptor_backends, std::string* err,
-                                                    int* status, uint64_t auto_staged_min_bytes) {
+                                                    const WorkerPoolOptions& options,
+                                                    std::string* err, int* status) {
   std::unique_ptr<GpuWorkerPool> pool(new GpuWorkerPool());
   pool->device_id_ = device_id;
   pool->mode_ = mode;
-  pool->use_descriptors_ = use_descriptor_backends;
-  pool->auto_staged_min_bytes_ = auto_staged_min_bytes;
+  pool->options_ = options;
   std::promise<TaskResult> load_ready, save_ready;
   auto lf = load_ready.get_future();
   auto sf = save_ready.get_future();
@@ -305,7 +310,39 @@ std::unique_ptr<GpuWorkerPool> GpuWorkerPool::spawn(int device_id, NumaNode numa
   }
   pool->separate_worker_queues();
   pool->prime_copy_overlap();
+  // One line per pool: an operator who asked for `kernel` (the connector's
+  // default for MLA models, common.py:577-594) should see that the workers here
+  // choose the path per task in both of the reference's modes.
+  const char* mode_name = mode == TransferMode::Direct ? "direct"
+                          : mode == TransferMode::Kernel ? "kernel" : "zerocopy";
+  if (options.use_descriptor_backends) {
+    log_line(LogLevel::Info,
+             "worker pool on device %d: transfer mode '%s' -> per-fragment descriptors through the "
+             "%s backend", device_id, mode_name, mode == TransferMode::Direct ? "direct" : "kernel");
+  } else if (mode == TransferMode::ZeroCopy) {
+    log_line(LogLevel::Info,
+             "worker pool on device %d: transfer mode 'zerocopy' -> block-ID kernel over mapped "
+             "host memory for every task, no staging memory", device_id);
+  } else {
+    const uint64_t call_min = options.auto_staged_min_bytes ? options.auto_staged_min_bytes
+                                                             : kWorkerStagedCallBytes;
+    log_line(LogLevel::Info,
+             "worker pool on device %d: transfer mode '%s' -> block-ID engine, path chosen per "
+             "task (staged through device memory from %llu bytes of dense layers per task, "
+             "zero-copy kernel below); staging memory held: %llu MiB%s",
+             device_id, mode_name, static_cast<unsigned long long>(call_min),
+             static_cast<unsigned long long>(pool->staging_bytes() >> 20),
+             options.lazy_staging ? " (allocated on the first staged task)" : "");
+  }
   return pool;
+}
+
+bool GpuWorkerPool::last_load(TaskResult* out, std::chrono::steady_clock::time_point* when) {
+  std::lock_guard<std::mutex> lock(last_load_mu_);
+  if (!has_last_load_) return false;
+  *out = last_load_;
+  *when = last_load_when_;
+  return true;
 }
 
 // Worker streams must not share a hardware queue: a zero-copy save and a
@@ -502,6 +539,7 @@ std::future<TaskResult> GpuWorkerPool::push(Worker* w, std::unique_ptr<Task> t) 
       t->reply.set_value(r);
       return fut;
     }
+    t->submitted = std::chrono::steady_clock::now();
     w->queue.push_back(std::move(t));
   }
   w->cv.notify_one();
@@ -544,7 +582,7 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
                    ": " + last_error();
   } else {
     backend = build_backend(mode_);
-    if (!use_descriptors_) {
+    if (!options_.use_descriptor_backends) {
       // The pool always has a second engine (load next to save), so each
       // worker keeps to one stream: with a side stream per engine the link
       // copies of the two directions were seen on one hardware queue (a
@@ -562,13 +600,25 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
       // the layers are staged and 0.21 (4 MiB layers), 0.36 (1 MiB), 0.58
       // (256 KiB), 0.84 (64 KiB) beside the resident kernel; staging costs
       // such a call 50-70 us, the length of a 3-4 MiB transfer.
-      constexpr uint64_t kWorkerStagedCallBytes = 8ull << 20;
-      cfg.auto_staged_min_call_bytes =
-          auto_staged_min_bytes_ != 0 ? auto_staged_min_bytes_ : kWorkerStagedCallBytes;
+      cfg.auto_staged_min_call_bytes = options_.auto_staged_min_bytes != 0
+                                           ? options_.auto_staged_min_bytes
+                                           : kWorkerStagedCallBytes;
+      cfg.staging_slot_bytes = options_.staging_slot_bytes;
       xfer = Xfer::create(&cfg);
-      if (!xfer) {
+      // Everything a worker needs exists before its first task (init_worker,
+      // gpu_worker.rs:278-298): the staging slots too, unless the pool was
+      // asked to leave them to the first staged task.  A zero-copy pool never
+      // stages.
+      int xst = xfer ? xfer->enable_profile() : PF_ERR_DEVICE_INIT;
+      if (xst == PF_OK && mode_ != TransferMode::ZeroCopy && !options_.lazy_staging) {
+        xst = xfer->reserve_staging();
+      }
+      if (xst != PF_OK) {
         init.status = PF_ERR_DEVICE_INIT;
         init.message = "transfer engine init failed: " + last_error();
+        xfer.reset();
+      } else {
+        staging_bytes_ += xfer->staging_bytes();
       }
     }
   }
@@ -597,8 +647,15 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
     // process_load_task / process_save_task, gpu_worker.rs:428-523.
     const auto t0 = std::chrono::steady_clock::now();
     TaskResult res;
+    res.queue_ms = std::chrono::duration<double, std::milli>(t0 - task->submitted).count();
+    res.resolve_ms = task->completion.resolve_ms;
     std::string err;
     int st = PF_OK;
+    const uint64_t staging_before = xfer ? xfer->staging_bytes() : 0;
+    if (xfer) xfer->reset_profile();
+    auto since = [](std::chrono::steady_clock::time_point t) {
+      return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t).count();
+    };
     // A task whose layers come as per-block handles is converted in two
     // parts: a few layers first, so that the device starts on them while the
     // (much larger) rest is still being converted.  Everything is only
@@ -637,7 +694,10 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
       if (xfer) {
         BlockForm form;
         bool failed = false;
-        if (to_block_form(task->layers, begin, end, &form, &failed, &err)) {
+        const auto t_convert = std::chrono::steady_clock::now();
+        const bool converted = to_block_form(task->layers, begin, end, &form, &failed, &err);
+        res.convert_ms += since(t_convert);
+        if (converted) {
           st = is_load ? xfer->load(form.layers.data(), form.layers.size(), path, stream)
                        : xfer->save(form.layers.data(), form.layers.size(), path, stream);
           if (st != PF_OK) err = last_error();
@@ -651,17 +711,24 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
       if (!done_fast) {
         std::vector<CopyDesc> copies;
         uint64_t total = 0;
-        if (!build_copy_descs(task->layers, &copies, &total, &err, begin, end)) {
+        const auto t_convert = std::chrono::steady_clock::now();
+        const bool built = build_copy_descs(task->layers, &copies, &total, &err, begin, end);
+        res.convert_ms += since(t_convert);
+        if (!built) {
           st = PF_ERR_STORAGE;
         } else {
+          const auto t_enqueue = std::chrono::steady_clock::now();
           st = is_load ? backend->h2d(copies.data(), copies.size(), stream)
                        : backend->d2h(copies.data(), copies.size(), stream);
+          res.enqueue_ms += since(t_enqueue);
           if (st != PF_OK) err = last_error();
           res.bytes += total;
+          res.paths |= PF_TASK_PATH_DESCRIPTORS;
         }
       }
       begin = end;
     }
+    const auto t_sync = std::chrono::steady_clock::now();
     if (st == PF_OK) {
       // One synchronisation for all layers.
       hipError_t he = hipEventRecord(done, stream);
@@ -675,10 +742,43 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
       (void)hipStreamSynchronize(stream);
       (void)hipGetLastError();
     }
+    res.sync_ms = since(t_sync);
+    if (xfer) {
+      const XferProfile prof = xfer->read_profile();
+      res.plan_ms = prof.plan_ms;
+      res.staging_alloc_ms = prof.staging_alloc_ms;
+      res.enqueue_ms += prof.enqueue_ms;
+      res.staged_groups = prof.staged_groups;
+      res.zero_copy_launches = prof.zero_copy_launches;
+      res.link_copies = prof.link_copies;
+      res.device_first_ms = prof.device_first_ms;
+      res.device_ms = prof.device_ms;
+      if (prof.staged_groups != 0) res.paths |= PF_TASK_PATH_STAGED;
+      if (prof.zero_copy_launches != 0) res.paths |= PF_TASK_PATH_ZEROCOPY;
+      const uint64_t staging_now = xfer->staging_bytes();
+      if (staging_now != staging_before) staging_bytes_ += staging_now - staging_before;
+    }
     res.status = st;
     res.message = err;
-    res.elapsed_ms =
-        std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+    res.elapsed_ms = since(t0);
+    if (log_level() == LogLevel::Debug) {
+      // gpu_worker.rs:465-474,511-520.
+      log_line(LogLevel::Debug,
+               "device %d %s task: %llu bytes in %.3f ms (%.2f GB/s), paths=%u staged_groups=%u "
+               "zero_copy_launches=%u, queue %.3f convert %.3f plan %.3f staging_alloc %.3f "
+               "enqueue %.3f sync %.3f ms, device first %.3f total %.3f ms%s%s",
+               device_id_, is_load ? "load" : "save", static_cast<unsigned long long>(res.bytes),
+               res.elapsed_ms, res.elapsed_ms > 0 ? res.bytes / res.elapsed_ms / 1e6 : 0.0,
+               res.paths, res.staged_groups, res.zero_copy_launches, res.queue_ms, res.convert_ms,
+               res.plan_ms, res.staging_alloc_ms, res.enqueue_ms, res.sync_ms,
+               res.device_first_ms, res.device_ms, st == PF_OK ? "" : ": ", err.c_str());
+    }
+    if (is_load) {
+      std::lock_guard<std::mutex> lock(last_load_mu_);
+      has_last_load_ = true;
+      last_load_ = res;
+      last_load_when_ = std::chrono::steady_clock::now();
+    }
     if (is_load && !task->completion.load_state_shm.empty()) {
       std::string aerr;
       auto ls = LoadState::attach(task->completion.load_state_shm, &aerr);

@@ -6,6 +6,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+#include <chrono>
 #include <condition_variable>
 #include <deque>
 #include <functional>
@@ -71,18 +73,42 @@ struct LayerTransferData {
   std::vector<std::shared_ptr<const void>> keep;
 };
 
-// Result of a task: status code (PF_OK or an error class) and message.
+// Result of a task: status code (PF_OK or an error class) and message, then
+// what the reference's workers log per task (bytes, duration;
+// gpu_worker.rs:458-474,505-520) and where the time went, phase by phase (the
+// fields of pf_task_result).
 struct TaskResult {
   int status = 0;
   std::string message;
   uint64_t bytes = 0;
   double elapsed_ms = 0;
+  uint32_t paths = 0;  // PF_TASK_PATH_* bits
+  uint32_t staged_groups = 0, zero_copy_launches = 0, link_copies = 0;
+  double resolve_ms = 0;  // filled by the engine for loads
+  double queue_ms = 0, convert_ms = 0, plan_ms = 0, staging_alloc_ms = 0, enqueue_ms = 0,
+         sync_ms = 0, device_first_ms = 0, device_ms = 0;
+};
+
+// What a pool's workers are given besides device, NUMA node and mode.
+struct WorkerPoolOptions {
+  bool use_descriptor_backends = false;
+  // A task whose dense layers add up to this much is staged (0 = 8 MiB).
+  uint64_t auto_staged_min_bytes = 0;
+  // Size of one staging slot; each worker of a staging pool holds two
+  // (0 = the transfer engine's default, 512 MiB).
+  uint64_t staging_slot_bytes = 0;
+  // false: both workers allocate their slots when the pool is spawned, so no
+  // task pays for it; true: a worker allocates on its first staged task.
+  bool lazy_staging = false;
 };
 
 // gpu_worker.rs:29-52: how a finished load reports back.  Shm = a LoadState
 // object the submitter polls; the future is always fulfilled as well.
 struct LoadCompletion {
   std::string load_state_shm;  // empty = none
+  // What the submitter spent turning leases into host blocks; travels with the
+  // task so that its result tells the whole load.
+  double resolve_ms = 0;
 };
 
 class Xfer;
@@ -94,8 +120,8 @@ class GpuWorkerPool {
   // backend of `mode`; otherwise they use the block-ID engine, with `mode`
   // choosing the link path (Direct = staged when possible, Kernel = zero-copy).
   static std::unique_ptr<GpuWorkerPool> spawn(int device_id, NumaNode numa_node, TransferMode mode,
-                                              bool use_descriptor_backends, std::string* err,
-                                              int* status, uint64_t auto_staged_min_bytes = 0);
+                                              const WorkerPoolOptions& options, std::string* err,
+                                              int* status);
   ~GpuWorkerPool();
   // gpu_worker.rs:204-212: fire and forget; the future (and the LoadState, if
   // named) is signalled when the task settles.
@@ -109,12 +135,18 @@ class GpuWorkerPool {
   // side when the pool was spawned: 0 = every worker stream probed has a
   // hardware queue of its own.
   size_t queue_clashes() const { return queue_clashes_; }
+  // Device memory the two workers hold for staging right now.
+  uint64_t staging_bytes() const { return staging_bytes_.load(); }
+  // The last load task this pool settled (status != 0 included) and when, on
+  // the steady clock; false when it has settled none.
+  bool last_load(TaskResult* out, std::chrono::steady_clock::time_point* when);
 
  private:
   struct Task {
     std::vector<LayerTransferData> layers;
     LoadCompletion completion;
     std::promise<TaskResult> reply;
+    std::chrono::steady_clock::time_point submitted;
   };
   struct Worker {
     std::thread thread;
@@ -134,8 +166,12 @@ class GpuWorkerPool {
 
   int device_id_ = 0;
   TransferMode mode_ = TransferMode::Direct;
-  bool use_descriptors_ = false;
-  uint64_t auto_staged_min_bytes_ = 0;  // 0 = the transfer engine's default
+  WorkerPoolOptions options_;
+  std::atomic<uint64_t> staging_bytes_{0};
+  std::mutex last_load_mu_;
+  bool has_last_load_ = false;
+  TaskResult last_load_;
+  std::chrono::steady_clock::time_point last_load_when_;
   Worker load_;
   Worker save_;
   size_t queue_clashes_ = 0;

@@ -13,6 +13,7 @@
 //               drains the slot to the host image on a side stream while the
 //               next slot is being packed (and the mirror image for loads).
 #include <algorithm>
+#include <chrono>
 #include <cstring>
 #include <memory>
 #include <string>
@@ -29,6 +30,11 @@ namespace pf {
 namespace {
 
 bool aligned16(uint64_t v) { return (v & 15ull) == 0; }
+
+using Clock = std::chrono::steady_clock;
+double ms_since(Clock::time_point t) {
+  return std::chrono::duration<double, std::milli>(Clock::now() - t).count();
+}
 
 }  // namespace
 
@@ -62,6 +68,15 @@ struct LayerPlan {
 
 int Xfer::ensure_slot(Slot& sl, uint64_t bytes) {
   if (sl.cap >= bytes) return PF_OK;
+  const Clock::time_point t0 = Clock::now();
+  struct Account {
+    XferProfile& prof;
+    Clock::time_point t0;
+    ~Account() {
+      prof.staging_alloc_ms += ms_since(t0);
+      ++prof.staging_allocs;
+    }
+  } account{prof_, t0};
   if (sl.buf) {
     // Grow-only: the old buffer may still be in flight.
     if (sl.used) PF_HIP(hipEventSynchronize(sl.freed));
@@ -74,6 +89,41 @@ int Xfer::ensure_slot(Slot& sl, uint64_t bytes) {
   PF_HIP(hipMalloc(&sl.buf, cap));
   sl.cap = cap;
   return PF_OK;
+}
+
+int Xfer::reserve_staging() {
+  for (auto& sl : slots_) {
+    const int st = ensure_slot(sl, slot_bytes_);
+    if (st != PF_OK) return st;
+  }
+  SlabPool::Slab* slab = nullptr;
+  const int st = slabs_.acquire(64 * 1024, &slab);  // stays in the pool, not in flight
+  prof_ = XferProfile();  // what was allocated here belongs to no call
+  return st;
+}
+
+int Xfer::enable_profile() {
+  if (profiling_) return PF_OK;
+  PF_HIP(hipEventCreate(&prof_begin_));
+  PF_HIP(hipEventCreate(&prof_first_));
+  PF_HIP(hipEventCreate(&prof_end_));
+  profiling_ = true;
+  return PF_OK;
+}
+
+XferProfile Xfer::read_profile() {
+  XferProfile out = prof_;
+  float ms = 0.f;
+  if (prof_begin_set_ && prof_end_set_ &&
+      hipEventElapsedTime(&ms, prof_begin_, prof_end_) == hipSuccess) {
+    out.device_ms = ms;
+  }
+  if (prof_begin_set_ && prof_first_set_ &&
+      hipEventElapsedTime(&ms, prof_begin_, prof_first_) == hipSuccess) {
+    out.device_first_ms = ms;
+  }
+  (void)hipGetLastError();
+  return out;
 }
 
 // The side stream carries the link copies next to the gather / scatter kernels
@@ -490,6 +540,8 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
     if (side_status != PF_OK) return side_status;
   }
   began_ = true;
+  const Clock::time_point t_enqueue = Clock::now();
+  prof_mark_begin(s);
   PF_HIP(hipMemcpyAsync(slab->dev, slab->host, slab_bytes, hipMemcpyHostToDevice, s));
   hipStream_t side = use_side_stream(chunks.size()) ? side_ : s;
   if (side != s) {
@@ -517,16 +569,20 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
       PF_HIP(hipStreamWaitEvent(side, sl.ready, 0));
       PF_HIP(hipMemcpyAsync(host_ptr, sl.buf, bytes, hipMemcpyDeviceToHost, side));
       PF_HIP(hipEventRecord(sl.freed, side));
+      prof_mark_first(side);
     } else {
       if (sl.used) PF_HIP(hipStreamWaitEvent(side, sl.freed, 0));
       PF_HIP(hipMemcpyAsync(sl.buf, host_ptr, bytes, hipMemcpyHostToDevice, side));
       PF_HIP(hipEventRecord(sl.ready, side));
+      prof_mark_first(side);
       PF_HIP(hipStreamWaitEvent(s, sl.ready, 0));
       st = launch(false);
       if (st != PF_OK) return st;
       PF_HIP(hipEventRecord(sl.freed, s));
     }
     sl.used = true;
+    ++prof_.staged_groups;
+    ++prof_.link_copies;
   }
   if (save && side != s) {
     PF_HIP(hipEventRecord(join_, side));
@@ -536,6 +592,8 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
   if (!layer_events_.empty()) {
     for (uint64_t li = 0; li < n_layers; ++li) PF_HIP(hipEventRecord(layer_events_[li], s));
   }
+  prof_mark_end(s);
+  prof_.enqueue_ms += ms_since(t_enqueue);
   return slabs_.release_after(slab, s);
 }
 
@@ -561,6 +619,8 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
   if (!timing_in_place_) timing_used_ = 0;
   if (n_layers == 0) return PF_OK;
   if (!layers) return fail(PF_ERR_INVALID_ARGUMENT, "layers must not be null");
+  const Clock::time_point t_call = Clock::now();
+  const double alloc_before = prof_.staging_alloc_ms;
   if (!layer_events_.empty() && layer_events_.size() < n_layers) {
     return fail(PF_ERR_INVALID_ARGUMENT, "%zu layer events set, call has %llu layers",
                 layer_events_.size(), static_cast<unsigned long long>(n_layers));
@@ -604,6 +664,7 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
       for (const LayerPlan& p : plans) total += p.layer_bytes;
       if (path == PF_PATH_STAGED || total >= auto_min_) {
         last_path_ = PF_PATH_STAGED;
+        prof_.plan_ms += ms_since(t_call);
         return run_page_pack(plans, pack, n_layers, save, s);
       }
     } else if (path == PF_PATH_STAGED) {
@@ -859,6 +920,9 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     if (side_status != PF_OK) return side_status;
   }
   began_ = true;
+  prof_.plan_ms += ms_since(t_call) - (prof_.staging_alloc_ms - alloc_before);
+  const Clock::time_point t_enqueue = Clock::now();
+  prof_mark_begin(s);
   if (!in_args) {
     PF_HIP(hipMemcpyAsync(slab->dev, slab->host, head_bytes, hipMemcpyHostToDevice, s));
   }
@@ -927,6 +991,8 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
                             save, s);
       }
       if (st != PF_OK) return st;
+      ++prof_.zero_copy_launches;
+      prof_mark_first(s);
       st = fire_events_through(plans[unit_refs[uj - 1].plan].src_index, s);
       if (st != PF_OK) return st;
       ui = uj;
@@ -1006,6 +1072,7 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
       st = link_copies(true);
       if (st != PF_OK) return st;
       PF_HIP(hipEventRecord(sl.freed, side));
+      prof_mark_first(side);
       sl.used = true;
       if (fire_through != UINT64_MAX) {
         st = fire_events_through(fire_through, side);
@@ -1016,6 +1083,7 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
       st = link_copies(false);
       if (st != PF_OK) return st;
       PF_HIP(hipEventRecord(sl.ready, side));
+      prof_mark_first(side);
       st = upload_orders();
       if (st != PF_OK) return st;
       PF_HIP(hipStreamWaitEvent(s, sl.ready, 0));
@@ -1028,6 +1096,8 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
         if (st != PF_OK) return st;
       }
     }
+    ++prof_.staged_groups;
+    prof_.link_copies += static_cast<uint32_t>(group_copies.size());
     ui = ue;
   }
   if (side_used && save) {
@@ -1041,6 +1111,8 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     st = fire_events_through(n_layers - 1, s);
     if (st != PF_OK) return st;
   }
+  prof_mark_end(s);
+  prof_.enqueue_ms += ms_since(t_enqueue);
   return in_args ? PF_OK : slabs_.release_after(slab, s);
 }
 

@@ -78,6 +78,21 @@ constexpr int kDefaultUnroll = 4;
 constexpr uint32_t kZeroCopyWorkgroupsFullTiles = 16;
 constexpr uint32_t kZeroCopyWorkgroupsMax = 64;
 
+// Where the time of the calls since reset_profile() went, and which way their
+// bytes crossed the link.  The device figures need enable_profile() and are
+// filled by read_profile() once the stream has been synchronised.
+struct XferProfile {
+  double plan_ms = 0;           // validation, unit and slab layout
+  double staging_alloc_ms = 0;  // hipMalloc / hipFree of staging slots inside a call
+  double enqueue_ms = 0;        // issuing copies and launches (row-order sort included)
+  uint32_t staged_groups = 0;
+  uint32_t zero_copy_launches = 0;
+  uint32_t link_copies = 0;
+  uint32_t staging_allocs = 0;
+  double device_first_ms = 0;   // first command -> first slot filled / drained (or first kernel)
+  double device_ms = 0;         // first command -> last command
+};
+
 class Xfer {
  public:
   explicit Xfer(const pf_xfer_config* cfg) {
@@ -107,6 +122,9 @@ class Xfer {
     for (auto& p : timing_pool_) {
       (void)hipEventDestroy(p.first);
       (void)hipEventDestroy(p.second);
+    }
+    for (hipEvent_t e : {prof_begin_, prof_first_, prof_end_}) {
+      if (e) (void)hipEventDestroy(e);
     }
     (void)hipGetLastError();
   }
@@ -170,6 +188,25 @@ class Xfer {
     timing_used_ = 0;
   }
   int last_kernel_ms(float* out_ms, uint32_t* out_launches);
+
+  // Allocate every staging slot at its configured size now (and one table
+  // slab), so that no call pays for it: hipMalloc of a slot inside a task
+  // lengthens that task.  The worker pools call this when they are spawned.
+  int reserve_staging();
+  uint64_t staging_bytes() const {
+    uint64_t total = 0;
+    for (const auto& sl : slots_) total += sl.cap;
+    return total;
+  }
+  // Three timing events bracket the device side of the calls of a profile
+  // window (begin, first slot ready, end); off unless enabled.
+  int enable_profile();
+  void reset_profile() {
+    prof_ = XferProfile();
+    prof_begin_set_ = prof_first_set_ = prof_end_set_ = false;
+  }
+  // Call after the stream of the profiled calls has been synchronised.
+  XferProfile read_profile();
 
  private:
   struct Slot {
@@ -245,6 +282,20 @@ class Xfer {
   }
   std::vector<std::pair<hipEvent_t, hipEvent_t>> timing_pool_;
   size_t timing_used_ = 0;
+
+  XferProfile prof_;
+  bool profiling_ = false;
+  hipEvent_t prof_begin_ = nullptr, prof_first_ = nullptr, prof_end_ = nullptr;
+  bool prof_begin_set_ = false, prof_first_set_ = false, prof_end_set_ = false;
+  void prof_mark_begin(hipStream_t s) {
+    if (profiling_ && !prof_begin_set_) prof_begin_set_ = hipEventRecord(prof_begin_, s) == hipSuccess;
+  }
+  void prof_mark_first(hipStream_t s) {
+    if (profiling_ && !prof_first_set_) prof_first_set_ = hipEventRecord(prof_first_, s) == hipSuccess;
+  }
+  void prof_mark_end(hipStream_t s) {
+    if (profiling_) prof_end_set_ = hipEventRecord(prof_end_, s) == hipSuccess;
+  }
 };
 
 

@@ -58,11 +58,33 @@ class LoadState:
             pass
 
 
+TASK_PATH_NAMES = ((_lib.PF_TASK_PATH_STAGED, "staged"), (_lib.PF_TASK_PATH_ZEROCOPY, "zerocopy"),
+                   (_lib.PF_TASK_PATH_DESCRIPTORS, "descriptors"))
+
+
 @dataclass
 class TaskResult:
+    """What a settled task reports: bytes and duration (what the reference's
+    workers log per task, gpu_worker.rs:458-474,505-520), which way the bytes
+    crossed the link, and the task's phases in milliseconds."""
     done: bool
     bytes: int
     elapsed_ms: float
+    paths: tuple = ()              # of "staged", "zerocopy", "descriptors"
+    staged_groups: int = 0
+    zero_copy_launches: int = 0
+    link_copies: int = 0
+    phases_ms: dict | None = None  # resolve, queue, convert, plan, staging_alloc, enqueue, sync,
+                                   # device_first, device
+
+    @classmethod
+    def from_c(cls, r) -> "TaskResult":
+        phases = {k[:-3]: getattr(r, k) for k in (
+            "resolve_ms", "queue_ms", "convert_ms", "plan_ms", "staging_alloc_ms", "enqueue_ms",
+            "sync_ms", "device_first_ms", "device_ms")}
+        return cls(bool(r.done), r.bytes, r.elapsed_ms,
+                   tuple(name for bit, name in TASK_PATH_NAMES if r.paths & bit),
+                   r.staged_groups, r.zero_copy_launches, r.link_copies, phases)
 
 
 class Task:
@@ -76,7 +98,7 @@ class Task:
     def wait(self, timeout_ms: int = -1) -> TaskResult:
         r = _lib.PfTaskResult()
         check(self._lib.pf_task_wait(self.handle, timeout_ms, C.byref(r)))
-        return TaskResult(bool(r.done), r.bytes, r.elapsed_ms)
+        return TaskResult.from_c(r)
 
     def close(self) -> None:
         if self.handle is not None:
@@ -122,12 +144,24 @@ class GpuWorkerPool:
     stream; tasks run serially per thread with one synchronisation each."""
 
     def __init__(self, device_id: int, numa_node: int = -1, transfer_mode: int = TransferMode.DIRECT,
-                 use_descriptor_backends: bool = False):
+                 use_descriptor_backends: bool = False, staging_slot_bytes: int = 0,
+                 auto_staged_min_bytes: int = 0, lazy_staging: bool = False):
+        """A staging pool (block-ID engine, mode direct or kernel) holds
+        2 workers x 2 slots of ``staging_slot_bytes`` (0 = 512 MiB) of device
+        memory from here on, unless ``lazy_staging`` leaves the allocation to the
+        first staged task of each worker."""
         self._lib = _lib.load()
         h = C.c_void_p()
-        check(self._lib.pf_worker_pool_spawn(device_id, numa_node, transfer_mode,
-                                             1 if use_descriptor_backends else 0, C.byref(h)))
+        cfg = _lib.PfWorkerPoolConfig(device_id, numa_node, transfer_mode,
+                                      1 if use_descriptor_backends else 0, staging_slot_bytes,
+                                      auto_staged_min_bytes, 1 if lazy_staging else 0, 0)
+        check(self._lib.pf_worker_pool_spawn_ex(C.byref(cfg), C.byref(h)))
         self.handle = h
+
+    @property
+    def staging_bytes(self) -> int:
+        """Device memory the two workers hold for staging right now."""
+        return self._lib.pf_worker_pool_staging_bytes(self.handle)
 
     @property
     def queue_clashes(self) -> int:
@@ -233,19 +267,28 @@ class PegaEngine:
     def __init__(self, pool_size: int, use_hugepages: bool = False, numa_aware: bool = False,
                  pool_shards: int = 1, blockwise_alloc: bool = False, ssd_enabled: bool = False,
                  use_descriptor_backends: bool = False, unit_size_hint: int = 0,
-                 lease_ttl_ms: int = 0, auto_staged_min_bytes: int = 0):
+                 lease_ttl_ms: int = 0, auto_staged_min_bytes: int = 0,
+                 staging_slot_bytes: int = 0, lazy_staging: bool = False,
+                 kernel_mode_zerocopy: bool = False):
         """``lease_ttl_ms``: how long an unconsumed query lease pins its blocks
         (0 = the reference's 600 s, lease.rs:11).  ``auto_staged_min_bytes``: a
         task whose dense layers add up to this much is staged through device
         memory by the workers instead of moved with the resident zero-copy
         kernel (0 = 8 MiB; layers of 16 MiB and more are staged in any case);
         1 = stage whatever can be staged, for servers that would rather
-        lengthen small loads than disturb the model's kernels."""
+        lengthen small loads than disturb the model's kernels.
+        ``staging_slot_bytes``: upper bound of a worker's staging slot (0 =
+        512 MiB); every registered context holds 2 workers x 2 slots of
+        min(this, what its layers can fill) in device memory from registration
+        on, unless ``lazy_staging``.  ``kernel_mode_zerocopy``: registrations
+        with TransferMode.KERNEL get zero-copy workers, the reference's meaning
+        of that mode, instead of the per-task choice."""
         self._lib = _lib.load()
         cfg = _lib.PfEngineConfig(pool_size, int(use_hugepages), int(numa_aware), pool_shards,
                                   int(blockwise_alloc), int(ssd_enabled),
                                   int(use_descriptor_backends), unit_size_hint, lease_ttl_ms,
-                                  auto_staged_min_bytes)
+                                  auto_staged_min_bytes, staging_slot_bytes, int(lazy_staging),
+                                  int(kernel_mode_zerocopy))
         h = C.c_void_p()
         check(self._lib.pf_engine_create(C.byref(cfg), C.byref(h)))
         self.handle = h
@@ -395,6 +438,18 @@ class PegaEngine:
         p = _lib.PfSaveProfile()
         check(self._lib.pf_engine_last_save_profile(self.handle, C.byref(p)))
         return {name: getattr(p, name) for name, _ in p._fields_}
+
+    def last_load_profile(self) -> TaskResult | None:
+        """The load task that settled last on this engine (None before any)."""
+        r = _lib.PfTaskResult()
+        if self._lib.pf_engine_last_load_profile(self.handle, C.byref(r)) != _lib.PF_OK:
+            return None
+        return TaskResult.from_c(r)
+
+    @property
+    def staging_bytes(self) -> int:
+        """Device memory the worker pools of all registered contexts hold for staging."""
+        return self._lib.pf_engine_staging_bytes(self.handle)
 
     def pool_usage(self) -> tuple[int, int]:
         used, total = C.c_uint64(), C.c_uint64()
