@@ -130,10 +130,12 @@ def parse_args():
     ap.add_argument("--ref-fragments", type=int, default=0,
                     help="ref_transfer_bench: only this fragment count (default: 1024..65536)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--settle-max", type=int, default=8,
+                    help="upper bound on the untimed passes run after the warmup until two agree")
     ap.add_argument("--no-extra-workloads", action="store_true",
                     help="default run only: skip the configs[3] and configs[4] workloads that "
                          "follow the headline one (the `workloads` key)")
-    ap.add_argument("--free-gib", type=int, default=40,
+    ap.add_argument("--free-gib", type=int, nargs="+", default=[10, 20, 40],
                     help="link_after_free: GiB of device memory to allocate, touch and free")
     return ap.parse_args()
 
@@ -206,112 +208,154 @@ def main():
     default_run = (args.workload == "llama8b" and args.path == "auto" and not args.layers
                    and not args.no_extra_workloads)
     if default_run:
-        keys = ("value", "save_gbps", "load_gbps", "ms_per_step", "step_save_load_ms", "config",
-                "roofline", "link", "link_settle", "byte_checks", "verified")
+        keys = ("value", "save_gbps", "load_gbps", "ms_per_step", "step_save_load_ms",
+                "settle_steps", "config", "roofline", "link", "byte_checks", "verified")
         workloads = {"llama8b": {k: result[k] for k in keys}}
+        freed = result["device_bytes_released"]
         for name in ("llama70b_fp8", "dsv3_mla"):
+            pause = pause_after_free(runtime, freed)
             extra = run_workload(args, name, set(), torch, np)
             workloads[name] = {k: extra[k] for k in keys}
+            workloads[name]["pause_after_previous_workload"] = pause
+            freed = extra["device_bytes_released"]
         result["workloads"] = workloads
     print(json.dumps(result))
 
 
-_SETTLE = {}
+_LINK_CHECK = {}
+# The driver clears freed device memory at 28.5 GiB/s on MI355X (`--workload
+# link_after_free`: 10 / 20 / 40 / 80 GiB freed -> copies of the affected stream
+# slow for 0.34 / 0.70 / 1.40 / 2.82 s); the pause allows 45 ms per GiB.
+CLEARING_S_PER_GIB = 0.045
 
 
-def wait_for_link(runtime, limit_s=20.0):
-    """Wait until host -> device copies run at the link's rate again.
-
-    Freeing device memory is followed by a stretch during which the runtime's
-    host -> device copies run at half their rate while device -> host copies
-    and kernels that read host memory are unaffected (`--workload
-    link_after_free` shows it: about 50 ms per GiB freed, in the freeing process
-    and in any other).  A process that starts right after another one released
-    tens of GiB -- this bench's own engine child, or the bench after a test run
-    -- would otherwise time that aftermath.  Copies of 256 MiB each way until
-    three host -> device copies in a row reach 0.95 of the device -> host rate;
-    no workload bytes move.  Returns what it saw."""
+def link_check(runtime):
+    """Rates of one 256 MiB copy each way on a fresh pair of streams set up the
+    way a worker pool sets up its pair (the first host -> device copy of one
+    stream issued while device -> host copies of the other are in flight): that
+    second stream is the one whose copies share a DMA engine with the driver's
+    clearing of freed device memory."""
     from pegaflow_amd.runtime import DeviceBuffer, Event, PinnedMemory, Stream
     size = 256 << 20
-    if not _SETTLE:   # kept for the life of the process: freeing them would restart the effect
-        _SETTLE.update(pin=PinnedMemory(2 * size), dev=DeviceBuffer(2 * size), stream=Stream(),
-                       ev=[Event(timing=True), Event(timing=True), Event(timing=True)])
-    pin, dev, stream, ev = _SETTLE["pin"], _SETTLE["dev"], _SETTLE["stream"], _SETTLE["ev"]
-    t0 = time.perf_counter()
-    first = None
-    good = samples = 0
-    while True:
-        ev[0].record(stream)
-        runtime.memcpy_d2h_async(pin.host_ptr, dev.ptr, size, stream)
-        ev[1].record(stream)
-        runtime.memcpy_h2d_async(dev.ptr + size, pin.host_ptr + size, size, stream)
-        ev[2].record(stream)
-        ev[2].synchronize()
-        d2h = size / ev[0].elapsed_ms(ev[1]) / 1e6
-        h2d = size / ev[1].elapsed_ms(ev[2]) / 1e6
-        samples += 1
-        if samples == 1:
-            continue   # the first copy of a stream carries its set-up
-        if first is None:
-            first = h2d
-        good = good + 1 if h2d >= 0.95 * d2h else 0
-        waited = time.perf_counter() - t0
-        if good >= 3 or waited > limit_s:
-            return {"waited_ms": round(waited * 1e3, 1), "copies": samples,
-                    "first_h2d_gbps": round(first, 2), "last_h2d_gbps": round(h2d, 2),
-                    "d2h_gbps": round(d2h, 2), "settled": good >= 3}
-
-
-def run_link_after_free(runtime, gib):
-    """Allocate, touch and free `gib` GiB of device memory, then time 327 MB
-    copies each way, one at a time, for a few seconds: how long and how much the
-    copies that follow a large hipFree are slowed."""
-    from pegaflow_amd.runtime import DeviceBuffer, Event, PinnedMemory, Stream
-    piece = 327_680_000
-    pin, dev = PinnedMemory(2 * piece), DeviceBuffer(2 * piece)
+    if not _LINK_CHECK:   # kept for the life of the process: freeing them is a free, too
+        _LINK_CHECK.update(pin=PinnedMemory(2 * size), dev=DeviceBuffer(2 * size),
+                           ev=[Event(timing=True) for _ in range(4)])
+    pin, dev, ev = _LINK_CHECK["pin"], _LINK_CHECK["dev"], _LINK_CHECK["ev"]
     sa, sb = Stream(), Stream()
-    ev = [Event(timing=True) for _ in range(4)]
+    for _ in range(6):
+        runtime.memcpy_d2h_async(pin.host_ptr, dev.ptr, 32 << 20, sa)
+    for _ in range(3):
+        runtime.memcpy_h2d_async(dev.ptr + size, pin.host_ptr + size, 32 << 20, sb)
+    sa.synchronize()
+    sb.synchronize()
+    ev[0].record(sa)
+    runtime.memcpy_d2h_async(pin.host_ptr, dev.ptr, size, sa)
+    ev[1].record(sa)
+    ev[1].synchronize()
+    ev[2].record(sb)
+    runtime.memcpy_h2d_async(dev.ptr + size, pin.host_ptr + size, size, sb)
+    ev[3].record(sb)
+    ev[3].synchronize()
+    out = {"d2h_gbps": round(size / ev[0].elapsed_ms(ev[1]) / 1e6, 2),
+           "h2d_gbps": round(size / ev[2].elapsed_ms(ev[3]) / 1e6, 2)}
+    sa.close()
+    sb.close()
+    return out
 
-    def sample(seconds):
+
+def pause_after_free(runtime, freed_bytes):
+    """Let the driver finish clearing the device memory this process just freed
+    before anything is timed: until then, copies of streams that share the
+    clearing's DMA engine (a worker pool's load stream does) run at half rate,
+    which says nothing about the transfer path.  Sleeps for the time the
+    clearing takes at its measured rate, then checks the link with a fresh
+    stream pair (and sleeps on, bounded, if that still reads slow).  No
+    workload bytes move."""
+    gib = freed_bytes / 2 ** 30
+    t0 = time.perf_counter()
+    time.sleep(CLEARING_S_PER_GIB * gib)
+    check = link_check(runtime)
+    while check["h2d_gbps"] < 0.9 * check["d2h_gbps"] and time.perf_counter() - t0 < 15.0:
+        time.sleep(0.1)
+        check = link_check(runtime)
+    return {"freed_gib": round(gib, 1), "paused_ms": round((time.perf_counter() - t0) * 1e3, 1),
+            "link_after_pause": check}
+
+
+def run_link_after_free(runtime, gib_list):
+    """What a large hipFree does to the link copies that follow it.  For each
+    size: allocate, touch and free that many GiB of device memory, then create
+    six fresh streams and time 64 MiB copies each way on every one of them in
+    turn (one copy in flight at a time) for a few seconds.  The driver clears
+    freed device memory with a DMA engine; a stream whose copies the runtime
+    placed on that engine runs at half rate until the clearing is done, the
+    others are not affected.  Reports, per size, which streams and directions
+    were slowed and until when: freed bytes / that time is the clearing rate."""
+    from pegaflow_amd.runtime import DeviceBuffer, Event, PinnedMemory, Stream
+    piece = 64 << 20
+    n_streams = 6
+    pin, dev = PinnedMemory(2 * piece), DeviceBuffer(2 * piece)
+    ev = [Event(timing=True) for _ in range(3)]
+
+    def sample(streams, seconds):
         rows, t0 = [], time.perf_counter()
         while time.perf_counter() - t0 < seconds:
-            ev[0].record(sa)
-            runtime.memcpy_d2h_async(pin.host_ptr, dev.ptr, piece, sa)
-            ev[1].record(sa)
-            ev[1].synchronize()
-            ev[2].record(sb)
-            runtime.memcpy_h2d_async(dev.ptr + piece, pin.host_ptr + piece, piece, sb)
-            ev[3].record(sb)
-            ev[3].synchronize()
-            rows.append((time.perf_counter() - t0, ev[0].elapsed_ms(ev[1]), ev[2].elapsed_ms(ev[3])))
+            for i, st in enumerate(streams):
+                ev[0].record(st)
+                runtime.memcpy_d2h_async(pin.host_ptr, dev.ptr, piece, st)
+                ev[1].record(st)
+                runtime.memcpy_h2d_async(dev.ptr + piece, pin.host_ptr + piece, piece, st)
+                ev[2].record(st)
+                ev[2].synchronize()
+                rows.append((time.perf_counter() - t0, i, ev[0].elapsed_ms(ev[1]),
+                             ev[1].elapsed_ms(ev[2])))
         return rows
 
-    sample(0.2)
-    before = sample(0.5)
-    bufs = []
-    for i in range(gib):
-        b = DeviceBuffer(1 << 30)
-        b.fill(i + 1)
-        bufs.append(b)
-    runtime.device_synchronize()
-    t0 = time.perf_counter()
-    for b in bufs:
-        b.close()
-    free_s = time.perf_counter() - t0
-    after = sample(max(3.0, 0.12 * gib))
-    norm_h2d = sorted(r[2] for r in before)[len(before) // 2]
-    norm_d2h = sorted(r[1] for r in before)[len(before) // 2]
-    slow = [r for r in after if r[2] > 1.2 * norm_h2d]
-    return {"metric": "link copies after hipFree", "unit": "ms per 327.68 MB copy",
+    warm = [Stream() for _ in range(2)]
+    sample(warm, 0.2)
+    base = sample(warm, 0.3)
+    norm_d2h = sorted(r[2] for r in base)[len(base) // 2]
+    norm_h2d = sorted(r[3] for r in base)[len(base) // 2]
+    out_rows = []
+    for gib in gib_list:
+        bufs = []
+        for i in range(gib):
+            b = DeviceBuffer(1 << 30)
+            b.fill(i + 1)
+            bufs.append(b)
+        runtime.device_synchronize()
+        t0 = time.perf_counter()
+        for b in bufs:
+            b.close()
+        free_s = time.perf_counter() - t0
+        streams = [Stream() for _ in range(n_streams)]
+        # the first two as a worker pool primes its pair: the first host -> device
+        # copy of one stream issued while device -> host copies of the other run
+        for _ in range(6):
+            runtime.memcpy_d2h_async(pin.host_ptr, dev.ptr, piece // 2, streams[0])
+        for _ in range(3):
+            runtime.memcpy_h2d_async(dev.ptr + piece, pin.host_ptr + piece, piece // 2, streams[1])
+        streams[0].synchronize()
+        streams[1].synchronize()
+        rows = sample(streams, max(2.0, 0.1 * gib))
+        slow_h2d = [r for r in rows if r[3] > 1.3 * norm_h2d]
+        slow_d2h = [r for r in rows if r[2] > 1.3 * norm_d2h]
+        last = max([r[0] for r in slow_h2d + slow_d2h], default=0.0)
+        out_rows.append({
             "freed_gib": gib, "free_call_s": round(free_s, 3),
-            "before": {"h2d_ms": round(norm_h2d, 2), "d2h_ms": round(norm_d2h, 2)},
-            "after": {"h2d_ms_max": round(max(r[2] for r in after), 2),
-                      "d2h_ms_max": round(max(r[1] for r in after), 2),
-                      "slow_h2d_copies": len(slow),
-                      "last_slow_h2d_at_s": round(slow[-1][0], 2) if slow else 0.0,
-                      "slow_h2d_ms_median": round(sorted(r[2] for r in slow)[len(slow) // 2], 2)
-                      if slow else None},
-            "device": runtime.device_name(0)}
+            "streams_with_slow_h2d": sorted({r[1] for r in slow_h2d}),
+            "streams_with_slow_d2h": sorted({r[1] for r in slow_d2h}),
+            "slow_copy_ms_median": round(sorted([r[3] for r in slow_h2d] + [r[2] for r in slow_d2h])
+                                         [(len(slow_h2d) + len(slow_d2h)) // 2], 2)
+            if slow_h2d or slow_d2h else None,
+            "last_slow_copy_at_s": round(last, 2),
+            "clearing_gib_per_s": round(gib / last, 1) if last > 0 else None})
+        for st in streams:
+            st.close()
+        time.sleep(1.0)
+    return {"metric": "link copies after hipFree", "unit": "ms per 64 MiB copy",
+            "normal": {"h2d_ms": round(norm_h2d, 3), "d2h_ms": round(norm_d2h, 3)},
+            "rows": out_rows, "device": runtime.device_name(0)}
 
 
 def run_workload(args, workload, sections, torch, np):
@@ -368,7 +412,6 @@ def run_workload(args, workload, sections, torch, np):
     pool = PinnedMemory(payload)
     pool_alloc_s = time.time() - t0
     torch.cuda.synchronize()
-    link_settle = wait_for_link(runtime)
 
     def layouts_for(caches):
         kv = nb * seg if w["split"] else 0
@@ -434,6 +477,19 @@ def run_workload(args, workload, sections, torch, np):
 
     for _ in range(args.warmup):
         one_step()
+    # A process that starts right after another one released tens of GiB of
+    # device memory (a test run, an earlier bench) can see the driver's clearing
+    # of that memory as a second or two of slower passes: the clearing shares a
+    # DMA engine with some streams' copies (`--workload link_after_free`).  How
+    # much was freed before this process started is not known here, so untimed
+    # passes run until two in a row agree (bounded); the count is reported.
+    settle_steps, prev = 0, None
+    while settle_steps < args.settle_max:
+        cur = sum(one_step())
+        settle_steps += 1
+        if prev is not None and abs(cur - prev) <= 0.015 * min(cur, prev):
+            break
+        prev = cur
     torch.cuda.synchronize()
     stream.synchronize()
     save_ms = load_ms = 0.0
@@ -629,8 +685,11 @@ def run_workload(args, workload, sections, torch, np):
     del src_cache, dst_cache, save_layers, load_layers, scratch, scratch2
     gc.collect()
     torch.cuda.empty_cache()
+    # caches, the two 1 GiB yardstick buffers, staging and what the checker held
+    released = 2 * n_layers * layer_bytes + 2 * link_bytes + (2 << 30)
     if "engine" in sections:
         import subprocess
+        engine_pause = pause_after_free(runtime, released)
         def engine_run(mode):
             cmd = [sys.executable, os.path.abspath(__file__), "--engine-child", "--workload",
                    workload, "--seed", str(args.seed), "--engine-mode", mode]
@@ -647,11 +706,16 @@ def run_workload(args, workload, sections, torch, np):
                 sys.exit(1)
             return json.loads(lines[-1])
         engine = engine_run(args.engine_mode)
+        engine["pause_before"] = engine_pause
+        # the first child released its own caches and staging when it ended
+        other_pause = pause_after_free(runtime, released + (4 << 30))
         # the other transfer mode, for comparison (instances choose one at registration)
         # the zero-copy worker mode, for comparison (instances choose a mode at registration;
         # "direct" and "kernel" both let the engine pick the path per call)
         other = "zerocopy" if args.engine_mode != "zerocopy" else "direct"
         engine["other_mode"] = engine_run(other)
+        engine["other_mode"]["pause_before"] = other_pause
+        released += 4 << 30
 
     # ---- CPU baseline: the oracle's memcpy executor on the host cores -----
     cpu = None
@@ -680,7 +744,7 @@ def run_workload(args, workload, sections, torch, np):
                    "copy_stream": args.copy_stream},
         "save_gbps": round(save_gbps, 3),
         "step_save_load_ms": step_times[:16],
-        "link_settle": link_settle,
+        "settle_steps": settle_steps,
         "load_gbps": round(load_gbps, 3),
         "roofline": roofline,
         "link": link,
@@ -690,6 +754,7 @@ def run_workload(args, workload, sections, torch, np):
         "engine": engine,
         "byte_checks": byte_checks,
         "verified": True,   # a failed byte check ends the run with exit status 1
+        "device_bytes_released": released,
         "pool_alloc_s": round(pool_alloc_s, 2),
         "device": runtime.device_name(0),
     }
@@ -1092,10 +1157,8 @@ def run_engine(torch, np, runtime, w, names, src_cache, dst_cache, save_ids, loa
     for t in dst_cache:
         t.zero_()
     torch.cuda.synchronize()
-    # This process starts right after the parent released its caches.
-    link_settle = wait_for_link(runtime)
     out = {"transfer_mode": mode_name, "worker_form": "descriptors" if descriptors else "block ids",
-           "link_settle": link_settle,
+           "link_before_first_task": link_check(runtime),
            "staging_mib_after_registration": eng.staging_bytes >> 20,
            "lazy_staging": bool(lazy_staging)}
     reps = 5
