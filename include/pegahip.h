@@ -237,20 +237,23 @@ const char* pf_backend_name(pf_backend_t b);
  *    buffer.  A handle still belongs to one thread at a time. */
 int pf_backend_h2d(pf_backend_t b, const pf_copy_desc* copies, uint64_t n, pf_stream_t s);
 int pf_backend_d2h(pf_backend_t b, const pf_copy_desc* copies, uint64_t n, pf_stream_t s);
-/* The copy of PF_MODE_KERNEL for callers that cannot allocate: code under HIP
- * graph capture, tight serving loops, harnesses that forbid hipMalloc.  No
- * counterpart in the reference (its KernelBackend reallocates its device table
- * whenever a batch outgrows it, transfer/kernel.rs:102-111).  Same bytes as
- * pf_backend_h2d (host_is_src != 0) / pf_backend_d2h (host_is_src == 0) of a
- * kernel backend, enqueue only, but the device-side descriptor table lives in
- * a fixed 1.5 MiB array inside the library's device image and the call makes
- * no hipMalloc / hipFree / hipHostMalloc, on any call including the first.
+/* The copy of PF_MODE_KERNEL for callers that cannot allocate: tight serving
+ * loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its
+ * KernelBackend reallocates its device table whenever a batch outgrows it,
+ * transfer/kernel.rs:102-111).  Same bytes as pf_backend_h2d (host_is_src != 0)
+ * / pf_backend_d2h (host_is_src == 0) of a kernel backend, enqueue only, but the
+ * device-side descriptor table lives in a fixed 1.5 MiB array inside the
+ * library's device image and the call allocates no device or pinned memory
+ * (no hipMalloc / hipFree / hipHostMalloc), on any call including the first.
  * Limits: n <= pf_desc_copy_noalloc_max() (32768), more is refused with
  * PF_ERR_INVALID_ARGUMENT; `copies` is read by the upload that the call
  * enqueues, so it stays alive and unchanged until the stream has been
- * synchronised (the usual descriptor rule); every call on one GPU shares the
- * one table, so calls on different streams of that GPU need an order between
- * them (calls on one stream are ordered by the stream). */
+ * synchronised (the usual descriptor rule), and it should sit in pinned memory
+ * for that upload to be asynchronous (from pageable memory the runtime stages
+ * it before the call returns); every call on one GPU shares the one table, so
+ * the library orders them: a call waits, on the device, for the kernel of the
+ * call before it, whatever streams the two use (calls on different streams of
+ * one GPU do not overlap).  Not tested under HIP graph capture. */
 int pf_desc_copy_noalloc(const pf_copy_desc* copies, uint64_t n, int host_is_src, pf_stream_t s);
 uint64_t pf_desc_copy_noalloc_max(void);
 /* TransferMode from the connector's string ("direct" | "kernel"),
@@ -746,6 +749,16 @@ int pf_engine_query_group_membership(pf_engine_t e, const char* instance_id, uin
 int pf_engine_create_group_lease(pf_engine_t e, const char* instance_id, uint32_t group,
                                  const uint8_t* const* hashes, const uint32_t* hash_lens,
                                  uint64_t n, uint64_t* out_lease);
+/* The two calls above as one step under one lock, which is what the membership
+ * branch of the reference's QueryPrefetch handler amounts to (service.rs:606-636
+ * leases the very block handles the membership query returned, so no eviction
+ * can come between): out_present as pf_engine_query_group_membership, and
+ * *out_lease = a lease over exactly the present blocks in list order, or 0 when
+ * none is present, or when require_all != 0 and one is missing. */
+int pf_engine_query_group_lease(pf_engine_t e, const char* instance_id, uint32_t group,
+                                const uint8_t* const* hashes, const uint32_t* hash_lens,
+                                uint64_t n, int require_all, uint8_t* out_present,
+                                uint64_t* out_lease);
 int pf_engine_pool_usage(pf_engine_t e, uint64_t* out_used, uint64_t* out_total);
 uint64_t pf_engine_cached_blocks(pf_engine_t e);
 /* Blocks that hold some but not all of their slots (saves of the remaining

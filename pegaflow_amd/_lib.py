@@ -309,6 +309,10 @@ PROTOTYPES = {
     "pf_engine_create_group_lease": (C.c_int, [vp, C.c_char_p, u32,
                                                C.POINTER(C.POINTER(C.c_uint8)), C.POINTER(u32),
                                                u64, C.POINTER(u64)]),
+    "pf_engine_query_group_lease": (C.c_int, [vp, C.c_char_p, u32,
+                                              C.POINTER(C.POINTER(C.c_uint8)), C.POINTER(u32),
+                                              u64, C.c_int, C.POINTER(C.c_uint8),
+                                              C.POINTER(u64)]),
     "pf_engine_pool_usage": (C.c_int, [vp, C.POINTER(u64), C.POINTER(u64)]),
     "pf_engine_cached_blocks": (u64, [vp]),
     "pf_engine_inflight_blocks": (u64, [vp]),

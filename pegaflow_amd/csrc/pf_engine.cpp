@@ -868,6 +868,40 @@ int Engine::query_group_membership(const std::string& instance_id, uint32_t grou
   return PF_OK;
 }
 
+int Engine::query_group_lease(const std::string& instance_id, uint32_t group,
+                              const std::vector<std::string_view>& hashes, bool require_all,
+                              std::vector<uint8_t>* present, uint64_t* out_lease,
+                              std::string* err) {
+  auto instance = get_instance(instance_id, err);
+  if (!instance) return PF_ERR_INSTANCE_MISSING;
+  auto topo = instance->sealed_topology(err);
+  if (!topo) return PF_ERR_INVALID_ARGUMENT;
+  size_t slots = 0;
+  std::string cause;
+  if (!topo->group_total_slots(group, &slots, &cause)) return bad(err, PF_ERR_INVALID_ARGUMENT, cause);
+  present->assign(hashes.size(), 0);
+  *out_lease = 0;
+  // Membership and lease under one lock: the blocks that are reported present
+  // are the blocks the lease pins (service.rs:606-636 leases the handles the
+  // membership query returned; nothing can evict one in between).
+  std::lock_guard<std::mutex> lock(mu_);
+  sweep_expired_locked();
+  Lease lease;
+  lease.instance_id = instance_id;
+  lease.remaining_consumers = std::max<size_t>(instance->world_size(), 1);
+  lease.expires_at = lease_deadline();
+  for (size_t i = 0; i < hashes.size(); ++i) {
+    SealedEntry* hit = find_sealed(instance->ns_id(), hashes[i], group);
+    if (hit == nullptr) continue;
+    (*present)[i] = 1;
+    lease.blocks.push_back(hit->block);
+  }
+  if (lease.blocks.empty() || (require_all && lease.blocks.size() != hashes.size())) return PF_OK;
+  *out_lease = next_lease_++;
+  leases_[*out_lease] = std::move(lease);
+  return PF_OK;
+}
+
 int Engine::create_group_lease(const std::string& instance_id, uint32_t group,
                                const std::vector<std::string_view>& hashes, uint64_t* out_lease,
                                std::string* err) {

@@ -155,6 +155,13 @@ class Engine {
   int create_group_lease(const std::string& instance_id, uint32_t group,
                          const std::vector<std::string_view>& hashes, uint64_t* out_lease,
                          std::string* err);
+  // The two above in one step, under one lock (service.rs:606-636): which of
+  // `hashes` are sealed in `group`, and a lease over exactly those blocks in
+  // that order (*out_lease = 0 when none is, or when `require_all` and one is
+  // missing).
+  int query_group_lease(const std::string& instance_id, uint32_t group,
+                        const std::vector<std::string_view>& hashes, bool require_all,
+                        std::vector<uint8_t>* present, uint64_t* out_lease, std::string* err);
   bool release_query_lease(uint64_t lease);
   // The periodic sweep of the reference's lease manager (lease.rs:66-80), for
   // the embedder's timer: drops expired leases, returns how many.

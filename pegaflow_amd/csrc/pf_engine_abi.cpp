@@ -581,6 +581,36 @@ int pf_engine_create_group_lease(pf_engine_t e, const char* instance_id, uint32_
   return st;
 }
 
+int pf_engine_query_group_lease(pf_engine_t e, const char* instance_id, uint32_t group,
+                                const uint8_t* const* hashes, const uint32_t* hash_lens,
+                                uint64_t n, int require_all, uint8_t* out_present,
+                                uint64_t* out_lease) {
+  PF_REQUIRE_PTR(e);
+  PF_REQUIRE_PTR(instance_id);
+  PF_REQUIRE_PTR(out_lease);
+  if (n != 0) {
+    PF_REQUIRE_PTR(hashes);
+    PF_REQUIRE_PTR(hash_lens);
+    PF_REQUIRE_PTR(out_present);
+  }
+  std::vector<std::string_view> h;
+  h.reserve(n);
+  for (uint64_t i = 0; i < n; ++i) {
+    h.emplace_back(reinterpret_cast<const char*>(hashes[i]), hash_lens[i]);
+  }
+  std::vector<uint8_t> present;
+  std::string err;
+  int st = reinterpret_cast<pf::Engine*>(e)->query_group_lease(instance_id, group, h,
+                                                               require_all != 0, &present,
+                                                               out_lease, &err);
+  if (st != PF_OK) {
+    pf::last_error() = err;
+    return st;
+  }
+  for (uint64_t i = 0; i < n; ++i) out_present[i] = present[i];
+  return PF_OK;
+}
+
 int pf_engine_pool_usage(pf_engine_t e, uint64_t* out_used, uint64_t* out_total) {
   PF_REQUIRE_PTR(e);
   PF_REQUIRE_PTR(out_used);

@@ -741,10 +741,14 @@ int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipSt
 // (and grows) on demand.  Callers that must not allocate get the same copy with
 // the table in a fixed array that is part of the library's device image.  Every
 // GPU the library runs on holds its own copy of the array, at its own address,
-// until the process ends; every call on a GPU shares it, so calls that overlap
-// on one GPU (different streams, no ordering between them) race on the table.
-// Nothing in it has to start at zero: a call overwrites rows [0, n) before its
-// kernel reads exactly those rows.
+// until the process ends, and every call on a GPU shares it.  Nothing in it has
+// to start at zero: a call overwrites rows [0, n) before its kernel reads
+// exactly those rows.  Calls are ordered among themselves: the upload and the
+// launch of a call are issued under one lock, and the upload waits (on the
+// device) for an event recorded behind the previous call's kernel, whichever
+// stream that ran on, so a call never overwrites rows a kernel is still
+// reading.  Calls on different streams of one GPU therefore run one after the
+// other; that is the price of the single table.
 
 // Most descriptors one call takes: 32768 x 48 bytes = 1.5 MiB per GPU.
 #define PF_NOALLOC_MAX_DESCS 32768u
@@ -764,29 +768,40 @@ uint32_t noalloc_workgroups(uint64_t total_bytes, uint64_t n) {
   return static_cast<uint32_t>(scaled < 64 ? scaled : 64);
 }
 
+// Per device: the table's address, the event behind the last call's kernel, and
+// whether there has been a call.  Set up on a device's first call (address and
+// event are host-side objects: no device or pinned memory is allocated).
+struct NoAllocDevice {
+  void* table = nullptr;
+  hipEvent_t last_done = nullptr;
+  bool used = false;
+};
 std::mutex g_scratch_mu;
-void* g_scratch_ptr[kNoAllocMaxDevices] = {};
+NoAllocDevice g_noalloc[kNoAllocMaxDevices];
 
 // Device address of `scratch` on the current device.  The array's name is only
 // a host-side handle for the symbol; the address comes from the runtime, once
-// per device, and is what every later use takes.
-int scratch_on_current_device(void** out) {
+// per device, and is what every later use takes.  g_scratch_mu held.
+int noalloc_on_current_device(NoAllocDevice** out) {
   int device = -1;
   PF_HIP(hipGetDevice(&device));
   if (device < 0 || device >= kNoAllocMaxDevices) {
     return pf::fail(PF_ERR_INVALID_ARGUMENT, "device %d is beyond the %d this call supports",
                     device, kNoAllocMaxDevices);
   }
-  std::lock_guard<std::mutex> lock(g_scratch_mu);
-  if (g_scratch_ptr[device] == nullptr) {
+  NoAllocDevice& d = g_noalloc[device];
+  if (d.table == nullptr) {
     void* ptr = nullptr;
     PF_HIP(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)));
     if (ptr == nullptr) {
       return pf::fail(PF_ERR_DEVICE_INIT, "hipGetSymbolAddress(scratch) returned a null address");
     }
-    g_scratch_ptr[device] = ptr;
+    hipEvent_t done = nullptr;
+    PF_HIP(hipEventCreateWithFlags(&done, hipEventDisableTiming));
+    d.last_done = done;
+    d.table = ptr;
   }
-  *out = g_scratch_ptr[device];
+  *out = &d;
   return PF_OK;
 }
 
@@ -816,15 +831,20 @@ extern "C" int pf_desc_copy_noalloc(const pf_copy_desc* copies, uint64_t n, int 
     if (c.size > max_size) max_size = c.size;
   }
   if (max_size == 0) return PF_OK;
-  void* table = nullptr;
-  int st = scratch_on_current_device(&table);
+  // Upload and launch under one lock: two threads cannot interleave their rows.
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  NoAllocDevice* dev = nullptr;
+  int st = noalloc_on_current_device(&dev);
   if (st != PF_OK) return st;
   hipStream_t stream = pf::native(s);
-  // The caller's array is the table: one copy, in stream order behind the
-  // previous call's kernel on this stream.
-  PF_HIP(hipMemcpyAsync(table, copies, n * sizeof(pf_copy_desc), hipMemcpyHostToDevice, stream));
+  // The previous call's kernel may still be reading the table, on this stream
+  // or another: this call's upload waits for it on the device.
+  if (dev->used) PF_HIP(hipStreamWaitEvent(stream, dev->last_done, 0));
+  // The caller's array is the table: one copy.  From pinned memory it is
+  // asynchronous; from pageable memory the runtime stages it before returning.
+  PF_HIP(hipMemcpyAsync(dev->table, copies, n * sizeof(pf_copy_desc), hipMemcpyHostToDevice, stream));
   const dim3 grid = pf::desc_copy_grid(n, max_size, noalloc_workgroups(total_size, n)), block(pf::kLanes, 1, 1);
-  const pf_copy_desc* rows = static_cast<const pf_copy_desc*>(table);
+  const pf_copy_desc* rows = static_cast<const pf_copy_desc*>(dev->table);
   if (host_is_src) {
     hipLaunchKernelGGL((pf::desc48_copy_kernel<pf::kDescUnroll, true>), grid, block, 0, stream, rows,
                        static_cast<uint32_t>(n));
@@ -834,6 +854,8 @@ extern "C" int pf_desc_copy_noalloc(const pf_copy_desc* copies, uint64_t n, int 
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return pf::fail_hip(e, "desc48_copy_kernel launch");
+  PF_HIP(hipEventRecord(dev->last_done, stream));
+  dev->used = true;
   return PF_OK;
 }
 

@@ -391,6 +391,19 @@ class PegaEngine:
                                                      ptrs, lens, len(hashes), C.byref(lease)))
         return lease.value
 
+    def query_group_lease(self, instance_id: str, group: int, hashes: Sequence[bytes],
+                          require_all: bool = False) -> tuple[list[bool], int]:
+        """Membership and lease in one step under the engine's lock: which of
+        ``hashes`` are sealed in ``group`` and a lease over exactly those blocks
+        (0 when none is, or when ``require_all`` and one is missing)."""
+        ptrs, lens, _bufs = _pack_hashes(hashes)
+        out = (C.c_uint8 * max(len(hashes), 1))()
+        lease = C.c_uint64()
+        check(self._lib.pf_engine_query_group_lease(self.handle, instance_id.encode(), group, ptrs,
+                                                    lens, len(hashes), 1 if require_all else 0,
+                                                    out, C.byref(lease)))
+        return [bool(out[i]) for i in range(len(hashes))], lease.value
+
     def batch_load_multi(self, instance_id: str, tp_rank: int, device_id: int,
                          layer_groups: Sequence[Sequence[str]],
                          loads: Sequence[tuple[int, Sequence[Sequence[int | None]]]],

@@ -17,11 +17,19 @@ Differences from the reference, on purpose:
   * ``wrapper_bytes`` carries ``HipIPCWrapper.to_bytes()`` records, not pickles;
   * a lease travels as 16 bytes (the reference's size) whose first 8 are this
     engine's 64-bit lease id;
-  * RDMA / MetaServer RPCs are not served (UNIMPLEMENTED).
+  * RDMA / MetaServer RPCs are not served (UNIMPLEMENTED);
+  * ``transfer_mode`` KERNEL (what the connector sends for MLA models,
+    python/pegaflow/connector/common.py:577-594) registers workers that choose
+    the way across the link per task, like DIRECT; an engine created with
+    ``kernel_mode_zerocopy=True`` gives such registrations the reference's
+    kernel mode (one copy kernel over mapped host memory).  The worker pool
+    logs its choice when it is spawned and every settled load is logged here at
+    debug level with the path it took.
 """
 
 from __future__ import annotations
 
+import logging
 import threading
 from concurrent import futures
 from typing import Sequence
@@ -36,6 +44,8 @@ from .transfer import TransferMode
 
 # The reference release whose client this server accepts
 # (service.rs:118-130: client and server versions must match).
+log = logging.getLogger(__name__)
+
 PROTOCOL_VERSION = "0.23.12"
 DEFAULT_ENDPOINT = "127.0.0.1:50055"
 
@@ -222,7 +232,16 @@ class EngineService:
         keep = []
         for task in tasks:
             try:
-                if wait or task.wait(0).done:
+                result = task.wait(-1 if wait else 0)
+                if result.done:
+                    # which way the bytes went and how long it took (the reference's
+                    # worker logs the same per load, gpu_worker.rs:465-474)
+                    if log.isEnabledFor(logging.DEBUG):
+                        log.debug("load settled: %d bytes in %.3f ms, paths=%s staged_groups=%d "
+                                  "zero_copy_launches=%d phases_ms=%s", result.bytes,
+                                  result.elapsed_ms, ",".join(result.paths) or "-",
+                                  result.staged_groups, result.zero_copy_launches,
+                                  result.phases_ms)
                     task.close()
                 else:
                     keep.append(task)
@@ -331,17 +350,17 @@ class EngineService:
         hashes = list(req.block_hashes)
         try:
             if req.group_id > 0:
-                present = self.engine.query_group_membership(req.instance_id, req.group_id, hashes)
+                # membership and lease in one step: what is reported present is
+                # what the lease pins (service.rs:606-636)
+                present, lease_id = self.engine.query_group_lease(
+                    req.instance_id, req.group_id, hashes, require_all=req.wait_for_full_prefix)
                 positions = [i for i, hit in enumerate(present) if hit]
                 if req.wait_for_full_prefix and len(positions) != len(hashes):
                     # all-or-nothing want-set: a short answer carries no lease
                     ready = QueryReadyMsg(num_hit_blocks=len(positions), lease=b"",
                                        hit_positions=list(range(len(positions))))
                     return QueryResponse(ready=ready)
-                lease = b""
-                if positions:
-                    lease = lease_to_bytes(self.engine.create_group_lease(
-                        req.instance_id, req.group_id, [hashes[i] for i in positions]))
+                lease = lease_to_bytes(lease_id) if positions else b""
                 return QueryResponse(ready=QueryReadyMsg(num_hit_blocks=len(positions), lease=lease,
                                                       hit_positions=positions))
             hits, lease = self.engine.query_prefix(req.instance_id, hashes)

@@ -70,6 +70,7 @@ def main():
             t0 = time.perf_counter()
             eng.batch_save_kv_blocks("src", 0, 0, 0, packed_b)
             times["save"] = time.perf_counter() - t0
+            times["save_span"] = (t0, time.perf_counter())
 
         def do_load():
             t0 = time.perf_counter()
@@ -77,6 +78,7 @@ def main():
                                                         [load_ids.tolist()])
             task.wait()
             times["load"] = time.perf_counter() - t0
+            times["load_span"] = (t0, time.perf_counter())
             task.close()
 
         threads = [threading.Thread(target=do_save), threading.Thread(target=do_load)]
@@ -86,7 +88,9 @@ def main():
         for t in threads:
             t.join()
         span = time.perf_counter() - t0
-        rates.append({"save_gbps": round(payload / times["save"] / 1e9, 2),
+        (s0, s1), (l0, l1) = times["save_span"], times["load_span"]
+        rates.append({"in_flight_together": bool(s0 < l1 and l0 < s1),
+                      "save_gbps": round(payload / times["save"] / 1e9, 2),
                       "load_gbps": round(payload / times["load"] / 1e9, 2),
                       "aggregate_gbps": round(2 * payload / span / 1e9, 2)})
         # drop batch B so the next repetition stores it again

@@ -32,10 +32,67 @@ def test_python_prototypes_cover_the_header():
     assert sorted(_lib.PROTOTYPES) == declared_functions()
 
 
-def test_struct_sizes_match_the_header():
-    assert C.sizeof(_lib.PfCopyDesc) == 48
-    assert C.sizeof(_lib.PfKvLayout) == 72
-    assert C.sizeof(_lib.PfHostMem) == 32
+def header_structs():
+    """{struct name: [field names]} of every `typedef struct pf_x { ... } pf_x;`."""
+    text = open(os.path.join(ROOT, "include", "pegahip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    out = {}
+    for name, body in re.findall(r"typedef struct (pf_\w+) \{(.*?)\} \1;", text, flags=re.S):
+        fields = []
+        for decl in body.split(";"):
+            decl = decl.strip()
+            if not decl:
+                continue
+            # `a, b, c` after one type (pf_save_profile) or a single declarator
+            for part in decl.split(","):
+                fields.append(re.findall(r"(\w+)\s*(?:\[\d+\])?\s*$", part.strip())[0])
+        out[name] = fields
+    return out
+
+
+@pytest.fixture(scope="module")
+def c_layout(tmp_path_factory):
+    """Sizes and field offsets as a C compiler lays the header out: the output of
+    tests/native/abi_layout.c, which also pins every number with _Static_assert."""
+    import json
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("gcc not installed")
+    exe = tmp_path_factory.mktemp("abi") / "abi_layout"
+    proc = subprocess.run(["gcc", "-std=c11", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", ROOT,
+                           os.path.join(ROOT, "tests", "native", "abi_layout.c"), "-o", str(exe)],
+                          capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr
+    return json.loads(subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout)
+
+
+def test_c_layout_covers_every_struct_and_field_of_the_header(c_layout):
+    structs = header_structs()
+    assert len(structs) >= 20
+    assert sorted(c_layout) == sorted(structs)
+    for name, fields in structs.items():
+        assert list(c_layout[name]["fields"]) == fields, name
+
+
+def test_ctypes_mirrors_match_the_c_layout(c_layout):
+    """Every struct of the header has a ctypes mirror with the same size, the same
+    fields in the same order and every field at the same offset (a swapped pair
+    of equally sized fields changes the names at the offsets)."""
+    for name, layout in c_layout.items():
+        mirror = getattr(_lib, "".join(part.capitalize() for part in name.split("_")), None)
+        assert mirror is not None, f"pegaflow_amd/_lib.py has no mirror of {name}"
+        assert C.sizeof(mirror) == layout["size"], name
+        assert [f[0] for f in mirror._fields_] == list(layout["fields"]), name
+        for field, offset in layout["fields"].items():
+            assert getattr(mirror, field).offset == offset, f"{name}.{field}"
+
+
+def test_copy_desc_is_the_reference_field_order(c_layout):
+    # transfer/mod.rs:36-44: device, host, host_device, size, device_allocation, host_allocation
+    assert list(c_layout["pf_copy_desc"]["fields"]) == [
+        "device", "host", "host_device", "size", "device_allocation", "host_allocation"]
+    assert c_layout["pf_copy_desc"]["size"] == 48
 
 
 def test_no_device_is_an_error_not_a_fallback():

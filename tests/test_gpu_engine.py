@@ -640,6 +640,14 @@ def test_recurrent_group_seals_final_block_save(engine):
         engine.create_group_lease("hybrid-hma", 1, [])
     with pytest.raises(_lib.StorageError, match="not resident"):
         engine.create_group_lease("hybrid-hma", 1, [hashes[0]])
+    # membership and lease in one step (what the QueryPrefetch handler uses)
+    present, both = engine.query_group_lease("hybrid-hma", 1, prefix)
+    assert present == [False, False, True] and both != 0
+    engine.release_query_lease(both)
+    present, none = engine.query_group_lease("hybrid-hma", 1, prefix, require_all=True)
+    assert present == [False, False, True] and none == 0
+    present, none = engine.query_group_lease("hybrid-hma", 1, prefix[:2])
+    assert present == [False, False] and none == 0
     for l in layers:
         l.zero_gpu()
     state = LoadState()
@@ -859,3 +867,118 @@ def test_lower_staging_threshold_moves_the_same_bytes(gpu):
         view[:, dest] = src[:, ids]
         l.assert_gpu_matches(want)
     e.close()
+
+
+@pytest.mark.parametrize("mode,use_desc,small_paths,large_paths", [
+    (TransferMode.DIRECT, False, ("zerocopy",), ("staged",)),
+    (TransferMode.KERNEL, False, ("zerocopy",), ("staged",)),
+    (TransferMode.ZEROCOPY, False, ("zerocopy",), ("zerocopy",)),
+    (TransferMode.DIRECT, True, ("descriptors",), ("descriptors",)),
+    (TransferMode.KERNEL, True, ("descriptors",), ("descriptors",)),
+], ids=["direct", "kernel", "zerocopy", "direct-descriptors", "kernel-descriptors"])
+def test_task_result_reports_the_path_taken(gpu, mode, use_desc, small_paths, large_paths):
+    """pf_task_result.paths: a 4 MiB task and a 300 MiB task through the workers
+    of each mode.  `direct` and `kernel` pools choose per task (zero-copy kernel
+    below 8 MiB of dense layers, staged above), a `zerocopy` pool never stages,
+    descriptor pools go through the backends; the bytes are checked each time."""
+    rng = np.random.default_rng(77)
+    seg, nb = 32768, 5120                      # one K/V-split layer of 320 MiB
+    cache0 = random_bytes(rng, 2 * nb * seg)
+    dev = DeviceBuffer(cache0.nbytes)
+    dev.copy_from_host(cache0)
+    layout = KVCacheLayout(dev.ptr, cache0.nbytes, nb, seg, nb * seg, 2)
+    kv = cache0.reshape(2, nb, seg)
+    pool = GpuWorkerPool(0, -1, mode, use_descriptor_backends=use_desc)
+    expected_staging = 0 if (use_desc or mode == TransferMode.ZEROCOPY) else 4 * (512 << 20)
+    assert pool.staging_bytes == expected_staging
+    for n, paths in ((64, small_paths), (4800, large_paths)):   # 4 MiB, 300 MiB
+        host = PinnedMemory(2 * n * seg)
+        host.as_numpy()[:] = 0
+        ids = rng.choice(nb, n, replace=False)
+        blocks = [HostBlock((host.host_ptr + i * seg, host.host_ptr + (n + i) * seg),
+                            (host.device_ptr + i * seg, host.device_ptr + (n + i) * seg), (1, 2),
+                            (seg, seg)) for i in range(n)]
+        res = pool.batch_save([LayerTransferData("kv", layout, ids, blocks)]).wait()
+        assert res.paths == paths, (n, res)
+        assert res.bytes == 2 * n * seg
+        if "staged" in paths:
+            assert res.staged_groups >= 1 and res.link_copies >= 1 and res.zero_copy_launches == 0
+        if paths == ("zerocopy",):
+            assert res.zero_copy_launches >= 1 and res.staged_groups == 0
+        # nothing is allocated inside a task: the slots exist since the pool was spawned
+        assert res.phases_ms["staging_alloc"] == 0.0
+        assert res.phases_ms["sync"] > 0.0 and res.elapsed_ms >= res.phases_ms["sync"]
+        img = host.as_numpy().reshape(2, n, seg)
+        assert np.array_equal(img[0], kv[0, ids]) and np.array_equal(img[1], kv[1, ids])
+        dest = rng.choice(nb, n, replace=False)
+        dev.fill(0)
+        res = pool.submit_load([LayerTransferData("kv", layout, dest, blocks)], None).wait()
+        assert res.paths == paths, (n, res)
+        got = dev.copy_to_host().reshape(2, nb, seg)
+        assert np.array_equal(got[:, dest], kv[:, ids])
+        rest = np.ones(nb, dtype=bool)
+        rest[dest] = False
+        assert not got[:, rest].any()
+        dev.copy_from_host(cache0)
+        host.close()
+    assert pool.staging_bytes == expected_staging
+    pool.close()
+    dev.close()
+
+
+def test_lazy_staging_allocates_on_the_first_staged_task(gpu):
+    """pf_worker_pool_config.lazy_staging / staging_slot_bytes: nothing is held
+    until a worker stages, then two slots of the configured size per worker."""
+    rng = np.random.default_rng(78)
+    seg, nb, n = 32768, 1024, 512               # 32 MiB task
+    cache0 = random_bytes(rng, 2 * nb * seg)
+    dev = DeviceBuffer(cache0.nbytes)
+    dev.copy_from_host(cache0)
+    layout = KVCacheLayout(dev.ptr, cache0.nbytes, nb, seg, nb * seg, 2)
+    pool = GpuWorkerPool(0, -1, TransferMode.DIRECT, staging_slot_bytes=48 << 20, lazy_staging=True)
+    assert pool.staging_bytes == 0
+    host = PinnedMemory(2 * n * seg)
+    ids = rng.choice(nb, n, replace=False)
+    blocks = [HostBlock((host.host_ptr + i * seg, host.host_ptr + (n + i) * seg),
+                        (host.device_ptr + i * seg, host.device_ptr + (n + i) * seg), (1, 2),
+                        (seg, seg)) for i in range(n)]
+    res = pool.batch_save([LayerTransferData("kv", layout, ids, blocks)]).wait()
+    assert res.paths == ("staged",) and res.phases_ms["staging_alloc"] > 0.0
+    assert pool.staging_bytes == 2 * (48 << 20)          # the save worker's two slots
+    img = host.as_numpy().reshape(2, n, seg)
+    kv = cache0.reshape(2, nb, seg)
+    assert np.array_equal(img[0], kv[0, ids]) and np.array_equal(img[1], kv[1, ids])
+    res = pool.batch_save([LayerTransferData("kv", layout, ids, blocks)]).wait()
+    assert res.phases_ms["staging_alloc"] == 0.0
+    pool.close()
+    host.close()
+    dev.close()
+
+
+def test_engine_load_profile_and_staging_report(gpu):
+    """pf_engine_last_load_profile mirrors the task's own result; a context's
+    staging is sized by what its layers can fill, not by the 512 MiB default;
+    kernel_mode_zerocopy gives KERNEL registrations the reference's kernel mode."""
+    e = PegaEngine(pool_size=64 << 20)
+    assert e.last_load_profile() is None
+    layers = [Layer(f"layer_{i}", 64, 16384, split_kv_stride=64 * 16384) for i in range(3)]
+    register(e, "profile", layers)
+    # 2 MiB layers: slots at the 32 MiB floor, 2 workers x 2 slots
+    assert e.staging_bytes == 4 * (32 << 20)
+    hashes = make_block_hashes(48, 5)
+    ids = list(range(8, 56))
+    e.batch_save_kv_blocks("profile", 0, 0, 0, [LayerSave(l.name, ids, hashes) for l in layers])
+    _hits, lease = e.query_prefix("profile", hashes)
+    res = e.batch_load_kv_blocks_multi_layer("profile", 0, 0, [[l.name for l in layers]], lease,
+                                             [ids]).wait()
+    assert res.paths == ("zerocopy",)            # 4.5 MiB of dense layers: below the 8 MiB rule
+    last = e.last_load_profile()
+    assert last.bytes == res.bytes == 3 * 48 * 2 * 16384
+    assert last.paths == res.paths and last.phases_ms == res.phases_ms
+    assert res.phases_ms["resolve"] > 0.0
+    e.close()
+    z = PegaEngine(pool_size=64 << 20, kernel_mode_zerocopy=True)
+    zlayers = [Layer(f"layer_{i}", 64, 16384, split_kv_stride=64 * 16384) for i in range(2)]
+    register(z, "kernel-as-reference", zlayers, mode=TransferMode.KERNEL)
+    assert z.staging_bytes == 0
+    z.close()

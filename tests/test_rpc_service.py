@@ -21,9 +21,8 @@ class FakeTask:
         self.closed = False
 
     def wait(self, _timeout):
-        class R:
-            done = True
-        return R()
+        from pegaflow_amd.engine import TaskResult
+        return TaskResult(True, 0, 0.0)
 
     def close(self):
         self.closed = True
@@ -66,6 +65,13 @@ class FakeEngine:
         self.next_lease += 1
         self.leases[self.next_lease] = list(hashes)
         return self.next_lease
+
+    def query_group_lease(self, instance, group, hashes, require_all=False):
+        present = [h in self.sealed for h in hashes]
+        hit = [h for h in hashes if h in self.sealed]
+        if not hit or (require_all and len(hit) != len(hashes)):
+            return present, 0
+        return present, self.create_group_lease(instance, group, hit)
 
     def release_query_lease(self, lease):
         if lease not in self.leases:

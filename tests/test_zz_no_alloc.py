@@ -103,6 +103,42 @@ def test_noalloc_two_calls_without_a_synchronise_between(gpu):
     host.close()
 
 
+def test_noalloc_calls_on_two_streams_share_the_table_safely(gpu):
+    """A long call on one stream, then a short one on another stream with no
+    host synchronise between them: the second call's upload overwrites the rows
+    the first call's kernel reads, so the library makes it wait on the device
+    for that kernel.  Both results must be whole."""
+    rng = np.random.default_rng(11)
+    slot, n = 4096, 24576
+    src = random_bytes(rng, n * slot)
+    sa, sb = Stream(), Stream()
+    host = PinnedMemory(n * slot)
+    host2 = PinnedMemory(64 * slot)
+    dev = DeviceBuffer(n * slot)
+    dev.copy_from_host(src)
+    host.as_numpy()[:] = 0
+    host2.as_numpy()[:] = 0
+    perm = rng.permutation(n).astype(np.uint64)
+    first = desc_array(dev.ptr + np.arange(n, dtype=np.uint64) * slot,
+                       host.host_ptr + perm * slot, host.device_ptr + perm * slot, slot)
+    pick = rng.permutation(n)[:64].astype(np.uint64)
+    second = desc_array(dev.ptr + pick * slot,
+                        host2.host_ptr + np.arange(64, dtype=np.uint64) * slot,
+                        host2.device_ptr + np.arange(64, dtype=np.uint64) * slot, slot)
+    for _ in range(3):
+        keep = [desc_copy_noalloc(first, sa, False), desc_copy_noalloc(second, sb, False)]
+        sa.synchronize()
+        sb.synchronize()
+        del keep
+        srcv = src.reshape(n, slot)
+        assert np.array_equal(host.as_numpy().reshape(n, slot)[perm.astype(np.int64)], srcv)
+        assert np.array_equal(host2.as_numpy().reshape(64, slot), srcv[pick.astype(np.int64)])
+        host.as_numpy()[:] = 0
+        host2.as_numpy()[:] = 0
+    for o in (sa, sb, dev, host, host2):
+        o.close()
+
+
 def test_noalloc_refusals(gpu):
     stream = Stream()
     host = PinnedMemory(4096)
