@@ -104,6 +104,9 @@ def parse_args():
     ap.add_argument("--layers", type=int, default=0, help="override the layer count")
     ap.add_argument("--slot-mb", type=int, default=0)
     ap.add_argument("--slots", type=int, default=0)
+    ap.add_argument("--group-mb", type=int, default=0,
+                    help="staged layers that follow one another share a slot and a launch up to "
+                         "this size (pf_xfer_config.staged_group_bytes; default: the slot size)")
     ap.add_argument("--unroll", type=int, default=0)
     ap.add_argument("--zc-max-wg", type=int, default=0)
     ap.add_argument("--copy-stream", type=int, default=0, choices=[0, 1, 2],
@@ -412,6 +415,10 @@ def run_workload(args, workload, sections, torch, np):
     pool = PinnedMemory(payload)
     pool_alloc_s = time.time() - t0
     torch.cuda.synchronize()
+    # Whatever ran on this GPU before this process may have freed device memory a
+    # moment ago: check the link with a fresh stream pair and wait (bounded) while
+    # the driver's clearing of that memory still slows it.
+    link_at_start = pause_after_free(runtime, 0)
 
     def layouts_for(caches):
         kv = nb * seg if w["split"] else 0
@@ -453,7 +460,7 @@ def run_workload(args, workload, sections, torch, np):
     load_layers = layers_for(dst_cache, load_ids)
     xfer = BlockTransfer(staging_slot_bytes=args.slot_mb << 20, staging_slots=args.slots,
                          tile_unroll=args.unroll, zerocopy_max_workgroups=args.zc_max_wg,
-                         copy_stream=args.copy_stream)
+                         copy_stream=args.copy_stream, staged_group_bytes=args.group_mb << 20)
     stream = Stream()
     ev = [Event(timing=True) for _ in range(4)]
 
@@ -745,6 +752,7 @@ def run_workload(args, workload, sections, torch, np):
         "save_gbps": round(save_gbps, 3),
         "step_save_load_ms": step_times[:16],
         "settle_steps": settle_steps,
+        "link_at_start": link_at_start,
         "load_gbps": round(load_gbps, 3),
         "roofline": roofline,
         "link": link,

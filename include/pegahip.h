@@ -341,6 +341,12 @@ typedef struct pf_xfer_config {
                                        0 = off.  For engines that move KV beside running kernels:
                                        the resident zero-copy kernel costs those for as long as
                                        the call lasts. */
+  uint64_t staged_group_bytes;      /* staged layers that follow one another share one staging
+                                       slot, and one gather / scatter launch, while together
+                                       they stay below this size (and the slot's); a group's
+                                       layers complete together.  0 = default: as many whole
+                                       layers as fit the slot, or 32 MiB while per-layer
+                                       events are set (pf_xfer_set_layer_events). */
 } pf_xfer_config;
 
 typedef struct pf_xfer_s* pf_xfer_t;
@@ -658,9 +664,9 @@ typedef struct pf_engine_config {
                                         can be staged, UINT64_MAX = only the large layers. */
   uint64_t staging_slot_bytes;       /* upper bound of a worker's staging slot; 0 = default
                                         (512 MiB).  Every registered context (instance, GPU)
-                                        holds 2 workers x 2 slots of min(this, what its layers
-                                        can fill: the largest layer, or a block's page for
-                                        page-first instances) in device memory from registration
+                                        holds 2 workers x 2 slots of min(this, the bytes of all
+                                        its registered layers, at least 32 MiB) in device memory
+                                        from registration
                                         on -- memory the serving framework's own budget does not
                                         know about. */
   uint32_t lazy_staging;             /* 1 = workers allocate their slots on the first staged

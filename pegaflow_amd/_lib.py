@@ -94,7 +94,7 @@ class PfXferConfig(C.Structure):
     _fields_ = [("staging_slot_bytes", u64), ("staging_slots", u32),
                 ("zerocopy_max_workgroups", u32), ("auto_staged_min_bytes", u64),
                 ("tile_unroll", u32), ("copy_stream", u32),
-                ("auto_staged_min_call_bytes", u64)]
+                ("auto_staged_min_call_bytes", u64), ("staged_group_bytes", u64)]
 
 
 class PfAllocRegion(C.Structure):

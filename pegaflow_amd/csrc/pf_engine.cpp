@@ -299,16 +299,13 @@ int Engine::register_context_layer_batch_strided(
   options.use_descriptor_backends = cfg_.use_descriptor_backends;
   options.auto_staged_min_bytes = cfg_.auto_staged_min_bytes;
   options.lazy_staging = cfg_.lazy_staging;
-  // A staging slot never holds more than one layer's blocks (layer-first) or
-  // the pages of one call (page-first: every layer's slice of a block), so a
-  // context of small layers gets small slots.  Small layers that follow one
-  // another share up to 32 MiB of a slot: that is the floor.
+  // A staging slot is filled with as many whole layers of a task as fit, so it
+  // never needs to be larger than everything the context registered: a context
+  // of small layers gets small slots.  Small layers that follow one another
+  // share up to 32 MiB of a slot even with per-layer events: that is the floor.
   {
     uint64_t fill = 0;
-    for (const auto& kv : ctx->reg.kv_caches) {
-      const uint64_t bytes = kv.second.block_bytes() * kv.second.num_blocks();
-      fill = page_first ? fill + bytes : std::max(fill, bytes);
-    }
+    for (const auto& kv : ctx->reg.kv_caches) fill += kv.second.block_bytes() * kv.second.num_blocks();
     constexpr uint64_t kSlotFloor = 32ull << 20, kSlotDefault = 512ull << 20;
     const uint64_t cap = cfg_.staging_slot_bytes ? cfg_.staging_slot_bytes : kSlotDefault;
     fill = (std::max(fill, kSlotFloor) + 0xFFFFFull) & ~0xFFFFFull;

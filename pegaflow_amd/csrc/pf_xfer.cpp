@@ -835,7 +835,9 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
   std::vector<size_t> group_end(unit_refs.size(), 0);
   std::vector<uint64_t> unit_slot_off(unit_refs.size(), 0);
   {
-    const uint64_t group_cap = std::min<uint64_t>(kStagedGroupBytes, slot_bytes_);
+    const uint64_t group_wish =
+        group_bytes_ != 0 ? group_bytes_ : (want_events ? kStagedGroupBytes : slot_bytes_);
+    const uint64_t group_cap = std::min<uint64_t>(group_wish, slot_bytes_);
     size_t ui = 0;
     while (ui < unit_refs.size()) {
       if (!plans[unit_refs[ui].plan].staged) {

@@ -45,9 +45,14 @@ constexpr uint32_t kDefaultSlots = 2;
 // tenth of its rate by staging.
 constexpr uint64_t kDefaultAutoStagedMin = 16ull << 20;
 // Staged units that follow one another share a staging slot, and one gather or
-// scatter launch, while together they stay below this size and count: the
-// copies of a group still take well under a millisecond, so the pipeline
-// keeps its grain.
+// scatter launch, while together they fit the slot (at most kStagedGroupUnits
+// of them): a launch pays ~6 us of ramp and tail whatever its size, so fewer,
+// larger launches move more bytes per microsecond (fp8 shape, 256 MiB layers:
+// one layer per launch 5.93 TB/s, two 6.12, four 6.18; Llama shape with 1 GiB
+// slots, three layers per launch: 6.1-6.28 against 5.97), and the layers of a
+// group complete together.  A caller that asked for a completion event per
+// layer wants them apart: then only small layers are grouped, up to
+// kStagedGroupBytes, whose copies still take well under a millisecond.
 // Layers below this size stay with the zero-copy kernel even in a call that
 // is staged for its total size.
 constexpr uint64_t kMinStagedLayerBytes = 32ull << 10;
@@ -104,6 +109,7 @@ class Xfer {
       call_min_ = cfg->auto_staged_min_call_bytes;
       if (cfg->tile_unroll) unroll_ = static_cast<int>(cfg->tile_unroll);
       if (cfg->copy_stream) copy_stream_ = cfg->copy_stream;
+      if (cfg->staged_group_bytes) group_bytes_ = cfg->staged_group_bytes;
     }
   }
 
@@ -255,6 +261,7 @@ class Xfer {
   uint64_t auto_min_ = kDefaultAutoStagedMin;
   uint64_t call_min_ = 0;  // PF_PATH_AUTO: stage every dense layer of a call that moves this much (0 = off)
   int unroll_ = kDefaultUnroll;
+  uint64_t group_bytes_ = 0;  // 0 = fill the slot (kStagedGroupBytes while layer events are set)
 
   hipStream_t side_ = nullptr;
   hipEvent_t fork_ = nullptr;

@@ -239,11 +239,11 @@ class BlockTransfer:
     def __init__(self, staging_slot_bytes: int = 0, staging_slots: int = 0,
                  zerocopy_max_workgroups: int = 0, auto_staged_min_bytes: int = 0,
                  tile_unroll: int = 0, copy_stream: int = 0,
-                 auto_staged_min_call_bytes: int = 0):
+                 auto_staged_min_call_bytes: int = 0, staged_group_bytes: int = 0):
         self._lib = _lib.load()
         cfg = _lib.PfXferConfig(staging_slot_bytes, staging_slots, zerocopy_max_workgroups,
                                 auto_staged_min_bytes, tile_unroll, copy_stream,
-                                auto_staged_min_call_bytes)
+                                auto_staged_min_call_bytes, staged_group_bytes)
         h = C.c_void_p()
         check(self._lib.pf_xfer_create(C.byref(cfg), C.byref(h)))
         self.handle = h

@@ -107,7 +107,7 @@ int main(void) {
   FIELD(pf_layer_blocks, page_len, 176);
   END();
 
-  BEGIN(pf_xfer_config, 40);
+  BEGIN(pf_xfer_config, 48);
   FIELD(pf_xfer_config, staging_slot_bytes, 0);
   FIELD(pf_xfer_config, staging_slots, 8);
   FIELD(pf_xfer_config, zerocopy_max_workgroups, 12);
@@ -115,6 +115,7 @@ int main(void) {
   FIELD(pf_xfer_config, tile_unroll, 24);
   FIELD(pf_xfer_config, copy_stream, 28);
   FIELD(pf_xfer_config, auto_staged_min_call_bytes, 32);
+  FIELD(pf_xfer_config, staged_group_bytes, 40);
   END();
 
   BEGIN(pf_alloc_region, 24);
