@@ -92,14 +92,15 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload",
                     choices=sorted(WORKLOADS) + ["ref_transfer_bench", "ref_cpu_path",
-                                                 "link_after_free"],
+                                                 "link_after_free", "launch_fit"],
                     default="llama8b",
                     help="ref_transfer_bench = the shapes of the reference's own "
                          "benches/transfer_h2d.rs through the descriptor backends; "
                          "ref_cpu_path = the engine-level groups of its benches/cpu_path.rs "
                          "(long lists of 1 KiB blocks through save / query / load); "
                          "link_after_free = what a large hipFree does to the link copies that "
-                         "follow it")
+                         "follow it; launch_fit = duration of one staged gather / scatter launch "
+                         "against its bytes: the fixed cost of a launch and the steady rate")
     ap.add_argument("--path", choices=["auto", "staged", "zerocopy"], default="auto")
     ap.add_argument("--layers", type=int, default=0, help="override the layer count")
     ap.add_argument("--slot-mb", type=int, default=0)
@@ -192,6 +193,9 @@ def main():
         return
     if args.workload == "link_after_free":
         print(json.dumps(run_link_after_free(runtime, args.free_gib)))
+        return
+    if args.workload == "launch_fit":
+        print(json.dumps(run_launch_fit(torch, np, runtime)))
         return
     if args.engine_child:
         print(json.dumps(run_workload(args, args.workload, {"engine_child"}, torch, np)))
@@ -359,6 +363,72 @@ def run_link_after_free(runtime, gib_list):
     return {"metric": "link copies after hipFree", "unit": "ms per 64 MiB copy",
             "normal": {"h2d_ms": round(norm_h2d, 3), "d2h_ms": round(norm_d2h, 3)},
             "rows": out_rows, "device": runtime.device_name(0)}
+
+
+def run_launch_fit(torch, np, runtime):
+    """Duration of one staged gather and one staged scatter launch against the
+    bytes it moves: Llama-shaped layers ([2, 8192, 32 KiB]), 512 to 8192 shuffled
+    blocks per launch, every launch running alone (link copies in order on the
+    kernels' stream) and bracketed by HIP events; the rotation over eight caches
+    keeps a launch from finding the previous one's lines.  A straight line through
+    the points gives the fixed cost of a launch (ramp, tail and the event
+    bracket, whose own reading is reported) and the steady rate."""
+    from pegaflow_amd.layout import KVCacheLayout
+    from pegaflow_amd.runtime import Event, PinnedMemory, Stream
+    from pegaflow_amd.transfer import BlockTransfer, LayerBlocks, TransferPath
+    dev = torch.device("cuda:0")
+    nb, seg, n_caches = 8192, 32768, 8
+    caches = [torch.empty(2 * nb * seg, device=dev, dtype=torch.uint8).random_(0, 256)
+              for _ in range(n_caches)]
+    pool = PinnedMemory(2 * nb * seg)
+    stream = Stream()
+    xfer = BlockTransfer(copy_stream=2)
+    xfer.set_kernel_timing(1)
+    rng = np.random.default_rng(0)
+    rows = []
+    for n in (512, 1024, 2048, 4096, 6144, 8192):
+        ids = rng.permutation(nb)[:n].astype(np.uint32)
+        per = {"save": [], "load": []}
+        for rep in range(2 + 2 * n_caches):
+            cache = caches[rep % n_caches]
+            layer = [LayerBlocks(layout=KVCacheLayout(cache.data_ptr(), 2 * nb * seg, nb, seg, nb * seg, 2),
+                                 block_ids=ids, host=(pool.host_ptr, pool.host_ptr + n * seg),
+                                 host_device=(pool.device_ptr, pool.device_ptr + n * seg),
+                                 host_len=(n * seg, n * seg), host_stride=seg)]
+            for name, fn in (("save", xfer.save), ("load", xfer.load)):
+                fn(layer, stream, TransferPath.STAGED)
+                stream.synchronize()
+                ms, launches = xfer.last_kernel_ms()
+                assert launches == 1
+                if rep >= 2:
+                    per[name].append(ms * 1e3)
+        med = {k: sorted(v)[len(v) // 2] for k, v in per.items()}
+        rows.append({"blocks": n, "alg_bytes": 4 * n * seg, "gather_us": round(med["save"], 2),
+                     "scatter_us": round(med["load"], 2),
+                     "gather_gbps": round(4 * n * seg / med["save"] / 1e3, 1),
+                     "scatter_gbps": round(4 * n * seg / med["load"] / 1e3, 1)})
+    pair = [Event(timing=True), Event(timing=True)]
+    empty = []
+    for _ in range(50):
+        pair[0].record(stream)
+        pair[1].record(stream)
+        pair[1].synchronize()
+        empty.append(pair[0].elapsed_ms(pair[1]) * 1e3)
+    fits = {}
+    x = np.array([r["alg_bytes"] for r in rows], dtype=np.float64)
+    for key in ("gather_us", "scatter_us"):
+        y = np.array([r[key] for r in rows])
+        slope, intercept = np.polyfit(x, y, 1)
+        fits[key[:-3]] = {"fixed_us": round(float(intercept), 2),
+                          "steady_gbps": round(1.0 / slope / 1e3, 1),
+                          "max_residual_us": round(float(np.abs(y - (slope * x + intercept)).max()), 2)}
+    xfer.close()
+    stream.close()
+    pool.close()
+    return {"metric": "staged launch duration against bytes", "unit": "us",
+            "rows": rows, "fit": fits, "empty_event_pair_us": round(sorted(empty)[len(empty) // 2], 2),
+            "note": "fixed_us includes the event bracket (empty_event_pair_us)",
+            "device": runtime.device_name(0)}
 
 
 def run_workload(args, workload, sections, torch, np):
