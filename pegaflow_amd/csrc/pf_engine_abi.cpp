@@ -279,6 +279,14 @@ int pf_task_wait(pf_task_t t, int timeout_ms, pf_task_result* out) {
       }
       return PF_OK;
     }
+    if (timeout_ms < 0) {
+      // Short tasks settle within tens of microseconds: poll for that long
+      // before parking the thread on the future (whose wake-up costs as much).
+      const auto spin_until = std::chrono::steady_clock::now() + std::chrono::microseconds(100);
+      while (h->fut.wait_for(std::chrono::seconds(0)) != std::future_status::ready &&
+             std::chrono::steady_clock::now() < spin_until) {
+      }
+    }
     h->result = h->fut.get();
     h->settled = true;
   }

@@ -210,20 +210,22 @@ __global__ __launch_bounds__(kLanes) void desc48_copy_kernel(
 }
 
 // Block-ID gather / scatter over mapped host memory (the zero-copy form).  The
-// grid is one row of workgroups, as many as the launch may keep on the device;
-// all of them walk the units one after the other and stride over the tiles of
-// each, so the units complete in order and the workgroup count does not grow
-// with the number of units.  Tile order inside a unit is (segment, list
-// position, tile in fragment), so at any moment the workgroups touch
-// neighbouring far-side addresses.
-// `units` may live in global memory (the uploaded slab) or in the kernel's own
-// argument segment; `bias` is added to the id-list and page-table addresses of
-// a unit (0 for absolute device addresses, the argument segment's base for
-// units that carry offsets into it).
+// grid is a few rows of workgroups, as many workgroups in all as the launch
+// may keep on the device.  Row y walks the units y, y + rows, ... one after the
+// other and its workgroups stride over the tiles of each, so the workgroup
+// count does not grow with the number of units.  With large units there is one
+// row and the units complete in order; a call of many small units (a few
+// blocks of every layer, the shape of a decode-time load) gets several rows,
+// or most workgroups would find no tile in a unit of four tiles and the rest
+// would walk all the units alone: 32 layers x 1 block loaded in 68 us with one
+// row of 16 workgroups (4 of them busy, 32 tiles each one after the other,
+// every tile a round trip over the link).  Tile order inside a unit is
+// (segment, list position, tile in fragment), so at any moment the workgroups
+// of a row touch neighbouring far-side addresses.
 template <int U, bool TO_FAR, typename UnitPtr>
 __device__ __forceinline__ void block_units_body(UnitPtr units, uint32_t n_units, uint64_t bias) {
   constexpr uint64_t kTile = static_cast<uint64_t>(U) * kLanes * 16;
-  for (uint32_t unit = 0; unit < n_units; ++unit) {
+  for (uint32_t unit = blockIdx.y; unit < n_units; unit += gridDim.y) {
     // Every field below is wave-uniform: read once into scalar registers.
     UnitPtr up = units + unit;
     const uint64_t near_base = up->near_base;
@@ -442,6 +444,24 @@ constexpr int kDescUnroll = 4;
 
 bool unroll_supported(int unroll) { return unroll == 1 || unroll == 2 || unroll == 4 || unroll == 8; }
 
+namespace {
+// Grid of a zero-copy launch: `max_workgroups` (0 = no cap) in all; x strides
+// over the tiles of a unit, y over the units.  Units as large as the cap or
+// larger leave one row.
+dim3 block_units_grid(uint32_t n_units, uint64_t max_tiles, uint32_t max_workgroups) {
+  uint64_t gx = max_tiles < kMaxGridX ? max_tiles : kMaxGridX;
+  if (max_workgroups != 0 && gx > max_workgroups) gx = max_workgroups;
+  uint64_t gy = 1;
+  if (max_workgroups != 0 && gx < max_workgroups) {
+    gy = max_workgroups / gx;
+    if (gy > n_units) gy = n_units;
+    if (gy > 65535) gy = 65535;
+    if (gy < 1) gy = 1;
+  }
+  return dim3(static_cast<uint32_t>(gx), static_cast<uint32_t>(gy), 1);
+}
+}  // namespace
+
 int launch_desc_copy(const uint64_t* table, uint64_t n, uint64_t max_size, hipStream_t s,
                      uint32_t max_workgroups);
 
@@ -452,10 +472,7 @@ int launch_block_units(const BlockUnit* units, uint32_t n_units, uint64_t max_ti
     return fail(PF_ERR_INVALID_ARGUMENT, "unit of %llu tiles exceeds the kernel limit",
                 static_cast<unsigned long long>(max_tiles));
   }
-  // One row of workgroups for the whole launch, whatever the number of units.
-  uint64_t gx = max_tiles < kMaxGridX ? max_tiles : kMaxGridX;
-  if (max_workgroups_x != 0 && gx > max_workgroups_x) gx = max_workgroups_x;
-  dim3 grid(static_cast<uint32_t>(gx), 1, 1);
+  const dim3 grid = block_units_grid(n_units, max_tiles, max_workgroups_x);
   dim3 block(kLanes, 1, 1);
 #define PF_LAUNCH_UNITS(U_)                                                                   \
   case U_:                                                                                    \
@@ -487,9 +504,7 @@ int launch_block_units_args(const ArgSlab& slab, uint32_t first_unit, uint32_t n
     return fail(PF_ERR_INVALID_ARGUMENT, "unit of %llu tiles exceeds the kernel limit",
                 static_cast<unsigned long long>(max_tiles));
   }
-  uint64_t gx = max_tiles < kMaxGridX ? max_tiles : kMaxGridX;
-  if (max_workgroups_x != 0 && gx > max_workgroups_x) gx = max_workgroups_x;
-  dim3 grid(static_cast<uint32_t>(gx), 1, 1);
+  const dim3 grid = block_units_grid(n_units, max_tiles, max_workgroups_x);
   dim3 block(kLanes, 1, 1);
 #define PF_LAUNCH_ARGS(U_)                                                                       \
   case U_:                                                                                       \

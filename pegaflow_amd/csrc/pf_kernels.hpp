@@ -42,8 +42,10 @@ bool unroll_supported(int unroll);
 
 // Launch the zero-copy block-ID kernel over the `n_units` units starting at
 // `units` (device).  `max_tiles` is the largest tile count of any of them;
-// `max_workgroups_x` (0 = no cap) is the number of workgroups of the launch:
-// all of them walk the units in order and stride over each unit's tiles.
+// `max_workgroups_x` (0 = no cap) is the number of workgroups of the launch.
+// With units of at least that many tiles there is one row of workgroups: all of
+// them walk the units in order and stride over each unit's tiles.  Smaller
+// units get several rows, each walking every rows-th unit.
 // to_far: true = gather near -> far (save), false = scatter far -> near (load).
 int launch_block_units(const BlockUnit* units, uint32_t n_units, uint64_t max_tiles, bool to_far,
                        int unroll, uint32_t max_workgroups_x, hipStream_t s);

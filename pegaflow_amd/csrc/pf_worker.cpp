@@ -732,7 +732,20 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
     if (st == PF_OK) {
       // One synchronisation for all layers.
       hipError_t he = hipEventRecord(done, stream);
-      if (he == hipSuccess) he = hipEventSynchronize(done);
+      if (he == hipSuccess) {
+        // A blocking wait costs its wake-up (10-15 us measured here, a fifth of
+        // a 2 MiB task): poll for the length of a short task first.
+        const auto spin_until = std::chrono::steady_clock::now() + std::chrono::microseconds(150);
+        he = hipErrorNotReady;
+        while (std::chrono::steady_clock::now() < spin_until) {
+          he = hipEventQuery(done);
+          if (he != hipErrorNotReady) break;
+        }
+        if (he == hipErrorNotReady) {
+          (void)hipGetLastError();
+          he = hipEventSynchronize(done);
+        }
+      }
       if (he != hipSuccess) {
         st = fail_hip(he, "Failed to synchronize");
         err = last_error();
