@@ -41,8 +41,8 @@ HBM_PEAK_GBPS = 8000.0      # MI355X published HBM3E bandwidth
 # launches it was measured on; `roofline.traffic` is read from there and only
 # reported when this run's launches have that same algorithmic size.
 TRAFFIC_PROFILES = {
-    "llama8b": "block_tiles_kernel_llama8b_save_load.md",
-    "llama70b_fp8": "block_tiles_kernel_llama70b_fp8_save_load.md",
+    "llama8b": "block_tiles_rows_kernel_llama8b_save_load.md",
+    "llama70b_fp8": "block_tiles_rows_kernel_llama70b_fp8_save_load.md",
     "dsv3_mla": "block_tiles_kernel_dsv3_mla_page_first_save_load.md",
 }
 
@@ -692,7 +692,7 @@ def run_workload(args, workload, sections, torch, np):
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                 "traffic": traffic, "traffic_source": traffic_source,
-                "kernel": ("block_tiles_kernel (staged gather/scatter)" if staged_path
+                "kernel": ("block_tiles_rows_kernel / block_tiles_kernel (staged gather/scatter)" if staged_path
                            else "block_units_kernel (zero-copy, host-link bound)"),
                 "measured": f"HIP events around each of the {live['launches']} launches of the "
                             f"{args.steps} timed steps",

@@ -78,6 +78,14 @@ constexpr uint32_t kMaxTileUnits = 32767;
 int launch_block_tiles(const BlockUnit* units, uint32_t n_units, uint32_t max_blocks,
                        uint64_t max_frag_bytes, uint32_t max_seg, bool to_far, hipStream_t s);
 
+// Up to eight units of any lengths in one launch with no idle workgroups: the
+// rows of all units laid end to end along grid.y (`host_units` is the host
+// copy of `units`, read for the row counts).  *launched = false when the launch
+// does not fit this form (more units, or more than kMaxTileBlocks rows in all):
+// nothing was enqueued and the caller uses launch_block_tiles.
+int launch_block_tiles_rows(const BlockUnit* units, const BlockUnit* host_units, uint32_t n_units,
+                            bool to_far, hipStream_t s, bool* launched);
+
 // The same for a single unit, handed over by value (its `ids` / `order` are
 // device addresses as usual).
 int launch_block_tiles_one(const BlockUnit& unit, bool to_far, hipStream_t s);

@@ -57,7 +57,7 @@ struct LayerPlan {
   uint64_t ids_slab_off = 0;    // byte offset of the id list inside the slab
   uint64_t table_slab_off = 0;  // byte offset of the page table inside the slab
   uint64_t order_slab_off = 0;  // byte offset of the row order inside the slab (staged loads)
-  uint64_t per_unit = 0;        // list positions per staged unit
+  std::vector<std::pair<uint64_t, uint64_t>> units;  // (first position, count) of each staged unit
   bool ordered = false;
   bool order_owner = false;     // this plan fills the order region
   bool order_shared = false;    // another plan's order region serves this one
@@ -692,21 +692,80 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
   };
   std::vector<UnitRef> unit_refs;
   uint64_t max_unit_bytes = 0;
-  for (size_t pi = 0; pi < plans.size(); ++pi) {
-    LayerPlan& p = plans[pi];
-    if (!p.staged) {
-      unit_refs.push_back({pi, 0, p.n_blocks});
-      continue;
+  // Staged layers are cut into units and the units packed into staging-slot
+  // fills ("groups": one gather or scatter launch and its link copies each) in
+  // one pass.  A fill takes whole layers while they fit and then the head of
+  // the next one, whose tail opens the following fill, so that every launch but
+  // the last moves a slot's worth of bytes whatever the size of a layer (a
+  // launch costs ~6 us beyond its bytes; Llama shape, 327 MB layers in 512 MiB
+  // slots: 537 MB per launch instead of 327).  A piece of a layer is at least
+  // kMinSplitBytes, or the layer is left whole for the next fill.  While the
+  // caller wants a completion event per layer only small layers share a fill
+  // (group_cap) and none is split.  group_end[ui] is one past the last unit of
+  // the group that starts at unit ui (0 for units inside a group and for
+  // zero-copy units); unit_slot_off[ui] is the unit's offset in its slot.
+  std::vector<size_t> group_end;
+  std::vector<uint64_t> unit_slot_off;
+  {
+    constexpr uint64_t kMinSplitBytes = 16ull << 20;
+    const uint64_t group_wish =
+        group_bytes_ != 0 ? group_bytes_ : (want_events ? kStagedGroupBytes : slot_bytes_);
+    const uint64_t group_cap = std::min<uint64_t>(group_wish, slot_bytes_);
+    const bool may_split = !want_events && group_bytes_ == 0;
+    constexpr size_t kNone = static_cast<size_t>(-1);
+    size_t group_start = kNone;
+    uint64_t used = 0;
+    auto close_group = [&]() {
+      if (group_start == kNone) return;
+      group_end[group_start] = unit_refs.size();
+      max_unit_bytes = std::max(max_unit_bytes, used);
+      group_start = kNone;
+      used = 0;
+    };
+    for (size_t pi = 0; pi < plans.size(); ++pi) {
+      LayerPlan& p = plans[pi];
+      if (!p.staged) {
+        close_group();
+        unit_refs.push_back({pi, 0, p.n_blocks});
+        group_end.push_back(0);
+        unit_slot_off.push_back(0);
+        continue;
+      }
+      const uint64_t block_bytes = p.frag_bytes * p.n_seg;
+      const uint64_t slot_blocks =
+          std::min<uint64_t>(std::max<uint64_t>(slot_bytes_ / block_bytes, 1), kMaxTileBlocks);
+      uint64_t pos = 0;
+      while (pos < p.n_blocks) {
+        const uint64_t remaining = p.n_blocks - pos;
+        uint64_t take = 0;
+        if (group_start == kNone) {
+          // A fresh fill takes up to a whole slot of this layer.
+          take = std::min(remaining, slot_blocks);
+        } else {
+          const uint64_t room = group_cap > used ? (group_cap - used) / block_bytes : 0;
+          const bool full = unit_refs.size() - group_start >= kStagedGroupUnits;
+          if (!full && room >= remaining) {
+            take = remaining;  // the rest of the layer fits
+          } else if (!full && may_split && room * block_bytes >= kMinSplitBytes &&
+                     (remaining - room) * block_bytes >= kMinSplitBytes) {
+            take = room;       // its head fills the slot, its tail opens the next fill
+          } else {
+            close_group();
+            continue;
+          }
+        }
+        if (group_start == kNone) {
+          group_start = unit_refs.size();
+        }
+        unit_slot_off.push_back(used);
+        unit_refs.push_back({pi, pos, take});
+        group_end.push_back(0);
+        p.units.emplace_back(pos, take);
+        used += (take * block_bytes + 255) & ~255ull;
+        pos += take;
+      }
     }
-    const uint64_t block_bytes = p.frag_bytes * p.n_seg;
-    uint64_t per_unit = std::max<uint64_t>(slot_bytes_ / block_bytes, 1);
-    per_unit = std::min<uint64_t>(per_unit, kMaxTileBlocks);
-    p.per_unit = per_unit;
-    for (uint64_t first = 0; first < p.n_blocks; first += per_unit) {
-      uint64_t count = std::min(per_unit, p.n_blocks - first);
-      unit_refs.push_back({pi, first, count});
-      max_unit_bytes = std::max(max_unit_bytes, count * block_bytes);
-    }
+    close_group();
   }
   // The visiting orders of staged loads sit behind everything else in the slab
   // and are uploaded on their own, after the first link copy is under way:
@@ -748,7 +807,7 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
         p.ordered = true;
         for (size_t pj = 0; pj < pi; ++pj) {
           if (plans[pj].ordered && plans[pj].ids_slab_off == p.ids_slab_off &&
-              plans[pj].per_unit == p.per_unit) {
+              plans[pj].units == p.units) {
             p.order_slab_off = plans[pj].order_slab_off;
             p.order_shared = true;
             break;
@@ -827,43 +886,10 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
   BlockUnit* units_host = reinterpret_cast<BlockUnit*>(slab_host);
   const BlockUnit* units_dev = reinterpret_cast<const BlockUnit*>(slab_dev);
   uint32_t slot_cursor = next_slot_;
-  // Small staged units that follow one another share a slot: one gather (or
-  // scatter) launch serves the whole group, which saves a launch and its
-  // hand-offs per layer (~12 of the ~30 us a staged layer costs beyond its
-  // bytes).  group_end[ui] is one past the last unit of the group that starts
-  // at ui (0 for units inside a group and for zero-copy units).
-  std::vector<size_t> group_end(unit_refs.size(), 0);
-  std::vector<uint64_t> unit_slot_off(unit_refs.size(), 0);
-  {
-    const uint64_t group_wish =
-        group_bytes_ != 0 ? group_bytes_ : (want_events ? kStagedGroupBytes : slot_bytes_);
-    const uint64_t group_cap = std::min<uint64_t>(group_wish, slot_bytes_);
-    size_t ui = 0;
-    while (ui < unit_refs.size()) {
-      if (!plans[unit_refs[ui].plan].staged) {
-        ++ui;
-        continue;
-      }
-      uint64_t used = 0;
-      size_t ue = ui;
-      while (ue < unit_refs.size() && plans[unit_refs[ue].plan].staged &&
-             ue - ui < kStagedGroupUnits) {
-        const LayerPlan& q = plans[unit_refs[ue].plan];
-        const uint64_t bytes = (unit_refs[ue].count * q.frag_bytes * q.n_seg + 255) & ~255ull;
-        if (ue > ui && used + bytes > group_cap) break;
-        unit_slot_off[ue] = used;
-        used += bytes;
-        ++ue;
-      }
-      group_end[ui] = ue;
-      max_unit_bytes = std::max(max_unit_bytes, used);
-      ui = ue;
-    }
-    if (max_unit_bytes != 0) {
-      for (auto& sl : slots_) {
-        st = ensure_slot(sl, max_unit_bytes);
-        if (st != PF_OK) return st;
-      }
+  if (max_unit_bytes != 0) {
+    for (auto& sl : slots_) {
+      st = ensure_slot(sl, max_unit_bytes);
+      if (st != PF_OK) return st;
     }
   }
   uint32_t group_slot = 0;
@@ -914,8 +940,10 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
   next_slot_ = slot_cursor;
 
   // ---- 4. enqueue ---------------------------------------------------------
+  // A second stream pays off when the link copies of one fill can overlap the
+  // gather of the next: count the fills.
   size_t staged_units = 0;
-  for (const UnitRef& r : unit_refs) staged_units += plans[r.plan].staged ? 1 : 0;
+  for (size_t ge : group_end) staged_units += ge != 0 ? 1 : 0;
   // Before anything of this call is on `s`: the check wants the stream idle.
   if (use_side_stream(staged_units)) {
     const int side_status = ensure_side_stream(s);
@@ -936,8 +964,10 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     orders_pending = false;
     for (const LayerPlan& p : plans) {
       if (p.order_owner) {
-        fill_row_order(p.ids, p.n_blocks, p.per_unit,
-                       reinterpret_cast<uint32_t*>(slab_host + p.order_slab_off));
+        uint32_t* order = reinterpret_cast<uint32_t*>(slab_host + p.order_slab_off);
+        for (const auto& unit : p.units) {
+          fill_row_order(p.ids + unit.first, unit.second, unit.second, order + unit.first);
+        }
       }
     }
     PF_HIP(hipMemcpyAsync(reinterpret_cast<void*>(slab_dev + head_bytes), slab_host + head_bytes,
@@ -1055,9 +1085,15 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
       }
       int rc = timing_begin(s);
       if (rc != PF_OK) return rc;
-      rc = launch_block_tiles(units_dev + ui, static_cast<uint32_t>(ue - ui), max_blocks, max_frag,
-                              max_seg, to_far, s);
+      bool launched = false;
+      rc = launch_block_tiles_rows(units_dev + ui, units_host + ui, static_cast<uint32_t>(ue - ui),
+                                   to_far, s, &launched);
       if (rc != PF_OK) return rc;
+      if (!launched) {
+        rc = launch_block_tiles(units_dev + ui, static_cast<uint32_t>(ue - ui), max_blocks, max_frag,
+                                max_seg, to_far, s);
+        if (rc != PF_OK) return rc;
+      }
       return timing_end(s);
     };
     // The events of every layer that ends inside the group fire behind it.

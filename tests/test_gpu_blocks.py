@@ -604,6 +604,82 @@ def test_small_staged_layers_share_slots_and_launches(stream, copy_stream):
     pool.close()
 
 
+@pytest.mark.parametrize("copy_stream", [0, 2], ids=["side_stream", "in_order"])
+def test_layers_split_across_staging_slot_fills(stream, copy_stream):
+    """Without per-layer events a staging slot is filled to the brim: whole
+    layers while they fit, then the head of the next layer, whose tail opens
+    the following fill.  Five layers of 40, 40, 24, 52 and 2 MiB in 64 MiB
+    slots make three fills per direction - [L0, head of L1], [tail of L1, L2,
+    head of L3], [tail of L3, L4] - with split and contiguous layers, unlike
+    fragment sizes and unlike row counts inside one launch.  Bytes against the
+    oracle both ways, the launch count, and the same call with per-layer
+    events (no layer split, one more fill)."""
+    rng = np.random.default_rng(4242)
+    shapes = [dict(num_blocks=700, seg=32768, segments=2, n_ids=640),     # 40 MiB
+              dict(num_blocks=1400, seg=32768, segments=1, n_ids=1280),   # 40 MiB, contiguous
+              dict(num_blocks=800, seg=16384, segments=2, n_ids=768),     # 24 MiB
+              dict(num_blocks=900, seg=32768, segments=2, n_ids=832),     # 52 MiB
+              dict(num_blocks=64, seg=16400, segments=2, n_ids=61)]       # ~2 MiB, fragments with a tail
+    cases = [Case(rng, **kw) for kw in shapes]
+    hosts, layers, Ls = [], [], []
+    for c in cases:
+        L = c.product_layout()
+        Ls.append(L)
+        nseg = 2 if L.is_split else 1
+        h = PinnedMemory(nseg * len(c.ids) * L.host_stride)
+        h.as_numpy()[:] = SENT
+        hosts.append(h)
+        c.dev.copy_from_host(c.cache0)
+        layers.append(_dense_layer(c, L, h, c.ids))
+    xfer = BlockTransfer(staging_slot_bytes=64 << 20, staging_slots=2, auto_staged_min_bytes=1,
+                         copy_stream=copy_stream)
+    xfer.set_kernel_timing(1)
+    xfer.save(layers, stream, TransferPath.STAGED)
+    stream.synchronize()
+    assert xfer.last_path == ST
+    assert xfer.last_kernel_ms()[1] == 3
+    images = []
+    for c, L, h in zip(cases, Ls, hosts):
+        n, stride = len(c.ids), L.host_stride
+        oc = c.cache0.copy()
+        ok = np.full(n * stride, SENT, dtype=np.uint8)
+        ov = np.full(n * stride, SENT, dtype=np.uint8) if L.is_split else None
+        O.transfer_layer(c.oracle_layout(oc), c.ids, ok, ov, host_is_src=False)
+        hv = h.as_numpy()
+        assert np.array_equal(hv[: n * stride], ok), c.args
+        if ov is not None:
+            assert np.array_equal(hv[n * stride:], ov), c.args
+        images.append((ok, ov))
+
+    def load_and_check(want_launches):
+        for li, c in enumerate(cases):
+            c.dev.fill(SENT)
+            layers[li].block_ids = rng.choice(c.num_blocks, len(c.ids), replace=False).astype(np.uint32)
+        xfer.load(layers, stream, TransferPath.STAGED)
+        stream.synchronize()
+        assert xfer.last_kernel_ms()[1] == want_launches
+        for li, c in enumerate(cases):
+            oc = np.full_like(c.cache0, SENT)
+            ok, ov = images[li]
+            O.transfer_layer(c.oracle_layout(oc), layers[li].block_ids, ok, ov, host_is_src=True)
+            assert np.array_equal(c.dev.copy_to_host(), oc), li
+
+    load_and_check(3)
+    # Per-layer events: a layer's event fires behind the fill that completes it,
+    # so layers stay whole and small ones share fills of at most 32 MiB:
+    # [L0] [L1] [L2] [L3] [L4].
+    events = [Event() for _ in cases]
+    xfer.set_layer_events(events)
+    load_and_check(5)
+    for e in events:
+        e.synchronize()
+    xfer.set_layer_events(None)
+    xfer.close()
+    for c, h in zip(cases, hosts):
+        c.close()
+        h.close()
+
+
 def test_call_size_rule_stages_small_layers_of_a_long_call(stream):
     """auto_staged_min_call_bytes: PF_PATH_AUTO stages the dense layers of a
     call whose dense bytes reach the threshold even though no layer reaches
