@@ -754,6 +754,9 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
             continue;
           }
         }
+        // A unit is one grid.y extent at most; what is left of the layer follows
+        // as another unit, in this fill while there is room.
+        take = std::min<uint64_t>(take, kMaxTileBlocks);
         if (group_start == kNone) {
           group_start = unit_refs.size();
         }

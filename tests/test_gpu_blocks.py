@@ -680,6 +680,58 @@ def test_layers_split_across_staging_slot_fills(stream, copy_stream):
         h.close()
 
 
+def test_long_layer_of_small_blocks_behind_another_layer_in_one_fill(stream):
+    """A layer of 68 000 blocks of 1 KiB (more rows than one grid extent)
+    that fits the room a small layer left in the slot: it becomes two units
+    of the same fill, and the bytes are the oracle's both ways."""
+    rng = np.random.default_rng(515)
+    cases = [Case(rng, num_blocks=128, seg=4096, segments=2, n_ids=100),
+             Case(rng, num_blocks=70000, seg=1024, segments=1, n_ids=68000)]
+    hosts, layers, Ls = [], [], []
+    for c in cases:
+        L = c.product_layout()
+        Ls.append(L)
+        nseg = 2 if L.is_split else 1
+        h = PinnedMemory(nseg * len(c.ids) * L.host_stride)
+        h.as_numpy()[:] = SENT
+        hosts.append(h)
+        c.dev.copy_from_host(c.cache0)
+        layers.append(_dense_layer(c, L, h, c.ids))
+    xfer = BlockTransfer(staging_slot_bytes=128 << 20, staging_slots=2, auto_staged_min_bytes=1)
+    xfer.set_kernel_timing(1)
+    xfer.save(layers, stream, TransferPath.STAGED)
+    stream.synchronize()
+    assert xfer.last_path == ST
+    assert xfer.last_kernel_ms()[1] == 1
+    images = []
+    for c, L, h in zip(cases, Ls, hosts):
+        n, stride = len(c.ids), L.host_stride
+        oc = c.cache0.copy()
+        ok = np.full(n * stride, SENT, dtype=np.uint8)
+        ov = np.full(n * stride, SENT, dtype=np.uint8) if L.is_split else None
+        O.transfer_layer(c.oracle_layout(oc), c.ids, ok, ov, host_is_src=False)
+        hv = h.as_numpy()
+        assert np.array_equal(hv[: n * stride], ok), c.args
+        if ov is not None:
+            assert np.array_equal(hv[n * stride:], ov), c.args
+        images.append((ok, ov))
+    for li, c in enumerate(cases):
+        c.dev.fill(SENT)
+        layers[li].block_ids = rng.choice(c.num_blocks, len(c.ids), replace=False).astype(np.uint32)
+    xfer.load(layers, stream, TransferPath.STAGED)
+    stream.synchronize()
+    assert xfer.last_kernel_ms()[1] == 1
+    for li, c in enumerate(cases):
+        oc = np.full_like(c.cache0, SENT)
+        ok, ov = images[li]
+        O.transfer_layer(c.oracle_layout(oc), layers[li].block_ids, ok, ov, host_is_src=True)
+        assert np.array_equal(c.dev.copy_to_host(), oc), li
+    xfer.close()
+    for c, h in zip(cases, hosts):
+        c.close()
+        h.close()
+
+
 def test_call_size_rule_stages_small_layers_of_a_long_call(stream):
     """auto_staged_min_call_bytes: PF_PATH_AUTO stages the dense layers of a
     call whose dense bytes reach the threshold even though no layer reaches
