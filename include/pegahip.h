@@ -344,9 +344,10 @@ typedef struct pf_xfer_config {
   uint64_t staged_group_bytes;      /* staged layers that follow one another share one staging
                                        slot, and one gather / scatter launch, while together
                                        they stay below this size (and the slot's); a group's
-                                       layers complete together.  0 = default: as many whole
-                                       layers as fit the slot, or 32 MiB while per-layer
-                                       events are set (pf_xfer_set_layer_events). */
+                                       layers complete together.  0 = default: every slot is
+                                       filled to the brim, a layer split where the slot ends,
+                                       or whole layers up to 32 MiB while per-layer events
+                                       are set (pf_xfer_set_layer_events). */
 } pf_xfer_config;
 
 typedef struct pf_xfer_s* pf_xfer_t;
@@ -374,6 +375,30 @@ int pf_xfer_last_path(pf_xfer_t x);
  * up over calls until pf_xfer_last_kernel_ms reads (and clears) them. */
 int pf_xfer_last_kernel_ms(pf_xfer_t x, float* out_ms, uint32_t* out_launches);
 int pf_xfer_set_kernel_timing(pf_xfer_t x, int enable);
+
+/* How pf_xfer_save / pf_xfer_load cut the staged layers of one call into units
+ * (runs of list positions of one layer) and pack the units into staging-slot
+ * fills, one gather or scatter launch and its link copies per fill: the planner
+ * those calls use, as pure host arithmetic (no device needed), for callers that
+ * want to know what a call will cost and for tests.  layer_blocks[i] = list
+ * positions of layer i, block_bytes[i] = payload bytes of one position (all
+ * segments; 0 = the layer is not staged and gets one unit outside any fill).
+ * slot_bytes and group_bytes as in pf_xfer_config (0 = default);
+ * per_layer_events != 0 = as after pf_xfer_set_layer_events.  Writes at most
+ * `capacity` units to `out` (may be NULL when capacity is 0) and always the
+ * number of units and of fills.  No counterpart in the reference. */
+typedef struct pf_fill_unit {
+  uint64_t layer;       /* index into the call's layers */
+  uint64_t first;       /* first list position of the unit */
+  uint64_t count;       /* list positions */
+  uint64_t slot_offset; /* byte offset of the unit inside its fill's staging slot */
+  uint64_t fill;        /* number of the fill the unit belongs to; UINT64_MAX = not staged */
+} pf_fill_unit;
+
+int pf_plan_staged_fills(const uint64_t* layer_blocks, const uint64_t* block_bytes,
+                         uint64_t n_layers, uint64_t slot_bytes, uint64_t group_bytes,
+                         uint32_t per_layer_events, pf_fill_unit* out, uint64_t capacity,
+                         uint64_t* out_units, uint64_t* out_fills);
 
 /* Plain device-to-device copy with the same tile shape as the gather/scatter
  * kernels (pointers and size 16-byte aligned).  tile_unroll 0 = the

@@ -97,6 +97,10 @@ class PfXferConfig(C.Structure):
                 ("auto_staged_min_call_bytes", u64), ("staged_group_bytes", u64)]
 
 
+class PfFillUnit(C.Structure):
+    _fields_ = [("layer", u64), ("first", u64), ("count", u64), ("slot_offset", u64), ("fill", u64)]
+
+
 class PfAllocRegion(C.Structure):
     _fields_ = [("offset_bytes", u64), ("size_bytes", u64), ("token", u64)]
 
@@ -225,6 +229,8 @@ PROTOTYPES = {
     "pf_xfer_last_path": (C.c_int, [vp]),
     "pf_xfer_last_kernel_ms": (C.c_int, [vp, C.POINTER(C.c_float), C.POINTER(u32)]),
     "pf_xfer_set_kernel_timing": (C.c_int, [vp, C.c_int]),
+    "pf_plan_staged_fills": (C.c_int, [C.POINTER(u64), C.POINTER(u64), u64, u64, u64, u32,
+                                       C.POINTER(PfFillUnit), u64, C.POINTER(u64), C.POINTER(u64)]),
     "pf_plain_copy": (C.c_int, [u64, u64, u64, u32, vp]),
     "pf_allocator_create": (C.c_int, [u64, u64, u32, C.POINTER(vp)]),
     "pf_allocator_destroy": (C.c_int, [vp]),

@@ -614,6 +614,63 @@ int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool s
   return st;
 }
 
+FillPlan plan_staged_fills(const std::vector<FillLayer>& layers, uint64_t slot_bytes,
+                           uint64_t group_cap, bool may_split, uint64_t max_unit_blocks) {
+  FillPlan plan;
+  constexpr size_t kNone = static_cast<size_t>(-1);
+  size_t fill_start = kNone;
+  uint64_t used = 0;
+  auto close_fill = [&]() {
+    if (fill_start == kNone) return;
+    plan.units[fill_start].fill_end = plan.units.size();
+    plan.max_fill_bytes = std::max(plan.max_fill_bytes, used);
+    ++plan.fills;
+    fill_start = kNone;
+    used = 0;
+  };
+  for (size_t li = 0; li < layers.size(); ++li) {
+    const FillLayer& layer = layers[li];
+    if (layer.block_bytes == 0) {
+      close_fill();
+      plan.units.push_back({li, 0, layer.n_blocks, 0, 0});
+      continue;
+    }
+    const uint64_t block_bytes = layer.block_bytes;
+    const uint64_t slot_blocks =
+        std::min<uint64_t>(std::max<uint64_t>(slot_bytes / block_bytes, 1), max_unit_blocks);
+    uint64_t pos = 0;
+    while (pos < layer.n_blocks) {
+      const uint64_t remaining = layer.n_blocks - pos;
+      uint64_t take = 0;
+      if (fill_start == kNone) {
+        // A fresh fill takes up to a whole slot of this layer.
+        take = std::min(remaining, slot_blocks);
+      } else {
+        const uint64_t room = group_cap > used ? (group_cap - used) / block_bytes : 0;
+        const bool full = plan.units.size() - fill_start >= kStagedGroupUnits;
+        if (!full && room >= remaining) {
+          take = remaining;  // the rest of the layer fits
+        } else if (!full && may_split && room * block_bytes >= kMinSplitBytes &&
+                   (remaining - room) * block_bytes >= kMinSplitBytes) {
+          take = room;       // its head fills the slot, its tail opens the next fill
+        } else {
+          close_fill();
+          continue;
+        }
+        // A unit is one grid extent at most; what is left of the layer follows
+        // as another unit, in this fill while there is room.
+        take = std::min(take, max_unit_blocks);
+      }
+      if (fill_start == kNone) fill_start = plan.units.size();
+      plan.units.push_back({li, pos, take, used, 0});
+      used += (take * block_bytes + 255) & ~255ull;
+      pos += take;
+    }
+  }
+  close_fill();
+  return plan;
+}
+
 int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save,
                    hipStream_t s) {
   if (!timing_in_place_) timing_used_ = 0;
@@ -692,83 +749,31 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
   };
   std::vector<UnitRef> unit_refs;
   uint64_t max_unit_bytes = 0;
-  // Staged layers are cut into units and the units packed into staging-slot
-  // fills ("groups": one gather or scatter launch and its link copies each) in
-  // one pass.  A fill takes whole layers while they fit and then the head of
-  // the next one, whose tail opens the following fill, so that every launch but
-  // the last moves a slot's worth of bytes whatever the size of a layer (a
-  // launch costs ~6 us beyond its bytes; Llama shape, 327 MB layers in 512 MiB
-  // slots: 537 MB per launch instead of 327).  A piece of a layer is at least
-  // kMinSplitBytes, or the layer is left whole for the next fill.  While the
-  // caller wants a completion event per layer only small layers share a fill
-  // (group_cap) and none is split.  group_end[ui] is one past the last unit of
-  // the group that starts at unit ui (0 for units inside a group and for
-  // zero-copy units); unit_slot_off[ui] is the unit's offset in its slot.
+  // Units and staging-slot fills (plan_staged_fills).  group_end[ui] is one
+  // past the last unit of the fill that starts at unit ui (0 for units inside
+  // a fill and for zero-copy units); unit_slot_off[ui] is the unit's offset in
+  // its slot.
   std::vector<size_t> group_end;
   std::vector<uint64_t> unit_slot_off;
   {
-    constexpr uint64_t kMinSplitBytes = 16ull << 20;
+    std::vector<FillLayer> fill_layers(plans.size());
+    for (size_t pi = 0; pi < plans.size(); ++pi) {
+      const LayerPlan& p = plans[pi];
+      fill_layers[pi] = {p.n_blocks, p.staged ? p.frag_bytes * p.n_seg : 0};
+    }
     const uint64_t group_wish =
         group_bytes_ != 0 ? group_bytes_ : (want_events ? kStagedGroupBytes : slot_bytes_);
-    const uint64_t group_cap = std::min<uint64_t>(group_wish, slot_bytes_);
-    const bool may_split = !want_events && group_bytes_ == 0;
-    constexpr size_t kNone = static_cast<size_t>(-1);
-    size_t group_start = kNone;
-    uint64_t used = 0;
-    auto close_group = [&]() {
-      if (group_start == kNone) return;
-      group_end[group_start] = unit_refs.size();
-      max_unit_bytes = std::max(max_unit_bytes, used);
-      group_start = kNone;
-      used = 0;
-    };
-    for (size_t pi = 0; pi < plans.size(); ++pi) {
-      LayerPlan& p = plans[pi];
-      if (!p.staged) {
-        close_group();
-        unit_refs.push_back({pi, 0, p.n_blocks});
-        group_end.push_back(0);
-        unit_slot_off.push_back(0);
-        continue;
-      }
-      const uint64_t block_bytes = p.frag_bytes * p.n_seg;
-      const uint64_t slot_blocks =
-          std::min<uint64_t>(std::max<uint64_t>(slot_bytes_ / block_bytes, 1), kMaxTileBlocks);
-      uint64_t pos = 0;
-      while (pos < p.n_blocks) {
-        const uint64_t remaining = p.n_blocks - pos;
-        uint64_t take = 0;
-        if (group_start == kNone) {
-          // A fresh fill takes up to a whole slot of this layer.
-          take = std::min(remaining, slot_blocks);
-        } else {
-          const uint64_t room = group_cap > used ? (group_cap - used) / block_bytes : 0;
-          const bool full = unit_refs.size() - group_start >= kStagedGroupUnits;
-          if (!full && room >= remaining) {
-            take = remaining;  // the rest of the layer fits
-          } else if (!full && may_split && room * block_bytes >= kMinSplitBytes &&
-                     (remaining - room) * block_bytes >= kMinSplitBytes) {
-            take = room;       // its head fills the slot, its tail opens the next fill
-          } else {
-            close_group();
-            continue;
-          }
-        }
-        // A unit is one grid.y extent at most; what is left of the layer follows
-        // as another unit, in this fill while there is room.
-        take = std::min<uint64_t>(take, kMaxTileBlocks);
-        if (group_start == kNone) {
-          group_start = unit_refs.size();
-        }
-        unit_slot_off.push_back(used);
-        unit_refs.push_back({pi, pos, take});
-        group_end.push_back(0);
-        p.units.emplace_back(pos, take);
-        used += (take * block_bytes + 255) & ~255ull;
-        pos += take;
-      }
+    const FillPlan fp =
+        plan_staged_fills(fill_layers, slot_bytes_, std::min<uint64_t>(group_wish, slot_bytes_),
+                          !want_events && group_bytes_ == 0, kMaxTileBlocks);
+    max_unit_bytes = fp.max_fill_bytes;
+    unit_refs.reserve(fp.units.size());
+    for (const FillUnit& u : fp.units) {
+      unit_refs.push_back({u.layer, u.first, u.count});
+      group_end.push_back(u.fill_end);
+      unit_slot_off.push_back(u.slot_off);
+      if (plans[u.layer].staged) plans[u.layer].units.emplace_back(u.first, u.count);
     }
-    close_group();
   }
   // The visiting orders of staged loads sit behind everything else in the slab
   // and are uploaded on their own, after the first link copy is under way:
@@ -1200,6 +1205,45 @@ int pf_xfer_last_kernel_ms(pf_xfer_t x, float* out_ms, uint32_t* out_launches) {
   PF_REQUIRE_PTR(out_ms);
   PF_REQUIRE_PTR(out_launches);
   return reinterpret_cast<pf::Xfer*>(x)->last_kernel_ms(out_ms, out_launches);
+}
+
+int pf_plan_staged_fills(const uint64_t* layer_blocks, const uint64_t* block_bytes,
+                         uint64_t n_layers, uint64_t slot_bytes, uint64_t group_bytes,
+                         uint32_t per_layer_events, pf_fill_unit* out, uint64_t capacity,
+                         uint64_t* out_units, uint64_t* out_fills) {
+  PF_REQUIRE_PTR(out_units);
+  PF_REQUIRE_PTR(out_fills);
+  if (n_layers != 0) {
+    PF_REQUIRE_PTR(layer_blocks);
+    PF_REQUIRE_PTR(block_bytes);
+  }
+  if (capacity != 0) PF_REQUIRE_PTR(out);
+  const uint64_t slot = slot_bytes != 0 ? slot_bytes : pf::kDefaultSlotBytes;
+  std::vector<pf::FillLayer> layers(n_layers);
+  for (uint64_t i = 0; i < n_layers; ++i) layers[i] = {layer_blocks[i], block_bytes[i]};
+  const uint64_t wish =
+      group_bytes != 0 ? group_bytes : (per_layer_events ? pf::kStagedGroupBytes : slot);
+  const pf::FillPlan plan =
+      pf::plan_staged_fills(layers, slot, std::min<uint64_t>(wish, slot),
+                            !per_layer_events && group_bytes == 0, pf::kMaxTileBlocks);
+  uint64_t fill = 0;
+  size_t fill_end = 0;
+  bool in_fill = false;
+  for (size_t ui = 0; ui < plan.units.size(); ++ui) {
+    const pf::FillUnit& u = plan.units[ui];
+    if (u.fill_end != 0) {
+      if (in_fill) ++fill;
+      in_fill = true;
+      fill_end = u.fill_end;
+    }
+    const bool staged = in_fill && ui < fill_end;
+    if (ui < capacity) {
+      out[ui] = {u.layer, u.first, u.count, u.slot_off, staged ? fill : UINT64_MAX};
+    }
+  }
+  *out_units = plan.units.size();
+  *out_fills = plan.fills;
+  return PF_OK;
 }
 
 int pf_plain_copy(uint64_t dst, uint64_t src, uint64_t bytes, uint32_t tile_unroll,

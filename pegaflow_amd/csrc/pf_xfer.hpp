@@ -45,7 +45,7 @@ constexpr uint32_t kDefaultSlots = 2;
 // tenth of its rate by staging.
 constexpr uint64_t kDefaultAutoStagedMin = 16ull << 20;
 // Staged units that follow one another share a staging slot, and one gather or
-// scatter launch, while together they fit the slot (at most kStagedGroupUnits
+// scatter launch, while together they fit the slot (plan_staged_fills; at most kStagedGroupUnits
 // of them, enough for every layer of an 80-layer model: a task of 32 layers x
 // 256 KiB took 238 us in two groups of 16 and takes one gather and one link
 // copy as one group): a launch pays ~6 us of ramp and tail whatever its size, so fewer,
@@ -64,6 +64,43 @@ constexpr uint64_t kMinStagedLayerBytes = 32ull << 10;
 constexpr uint64_t kRowOrderFromBytes = 4ull << 20;
 constexpr uint64_t kStagedGroupBytes = 32ull << 20;
 constexpr size_t kStagedGroupUnits = 128;
+// A layer is split between two fills only into pieces of at least this size.
+constexpr uint64_t kMinSplitBytes = 16ull << 20;
+
+// How the layers of one call are cut into units (runs of list positions of one
+// layer) and the units packed into staging-slot fills: one gather or scatter
+// launch and its link copies per fill.  Pure arithmetic.
+//
+// A fill takes whole layers while they fit and then, when `may_split`, the
+// head of the next one, whose tail opens the following fill: every launch but
+// the last then moves a slot's worth of bytes whatever the size of a layer (a
+// launch costs ~6 us beyond its bytes; Llama shape, 327 MB layers in 512 MiB
+// slots: 537 MB per launch instead of 327).  A piece of a layer is at least
+// kMinSplitBytes, or the layer is left whole for the next fill.  Without
+// `may_split` (the caller wants a completion event per layer, or set a group
+// size) layers stay whole and share a fill up to `group_cap` bytes; a layer
+// larger than a slot always takes several fills.  No unit has more than
+// `max_unit_blocks` positions (one grid extent) and no fill more than
+// kStagedGroupUnits units.  A layer with block_bytes == 0 is not staged: it
+// closes the current fill and gets one unit of its own outside any fill.
+struct FillLayer {
+  uint64_t n_blocks;
+  uint64_t block_bytes;  // payload of one list position (all segments); 0 = not staged
+};
+struct FillUnit {
+  size_t layer;
+  uint64_t first;     // first list position
+  uint64_t count;
+  uint64_t slot_off;  // byte offset inside the fill's slot (256-byte aligned)
+  size_t fill_end;    // first unit of a fill: one past its last unit; otherwise 0
+};
+struct FillPlan {
+  std::vector<FillUnit> units;
+  uint64_t max_fill_bytes = 0;
+  size_t fills = 0;
+};
+FillPlan plan_staged_fills(const std::vector<FillLayer>& layers, uint64_t slot_bytes,
+                           uint64_t group_cap, bool may_split, uint64_t max_unit_blocks);
 constexpr int kDefaultUnroll = 4;
 // Zero-copy launches are capped to a few workgroups: the host link, not the
 // GPU, is the bound, and every workgroup that stays resident for the length of

@@ -232,6 +232,41 @@ class LayerBlocks:
     _keep: list = field(default_factory=list, repr=False)
 
 
+@dataclass(frozen=True)
+class FillUnit:
+    """One unit of a staged call: list positions ``first .. first+count`` of
+    layer ``layer``, at ``slot_offset`` of the staging slot of fill number
+    ``fill`` (None: the layer is not staged)."""
+    layer: int
+    first: int
+    count: int
+    slot_offset: int
+    fill: int | None
+
+
+def plan_staged_fills(layer_blocks: Sequence[int], block_bytes: Sequence[int],
+                      staging_slot_bytes: int = 0, staged_group_bytes: int = 0,
+                      per_layer_events: bool = False) -> tuple[list[FillUnit], int]:
+    """(units, number of fills) of a staged save or load of these layers: the
+    planner ``BlockTransfer`` uses, as host arithmetic (pf_plan_staged_fills).
+    One gather or scatter launch runs per fill."""
+    lib = _lib.load()
+    n = len(layer_blocks)
+    if len(block_bytes) != n:
+        raise ValueError("layer_blocks and block_bytes differ in length")
+    blocks = (C.c_uint64 * max(n, 1))(*layer_blocks)
+    sizes = (C.c_uint64 * max(n, 1))(*block_bytes)
+    n_units, n_fills = C.c_uint64(), C.c_uint64()
+    args = (blocks, sizes, n, staging_slot_bytes, staged_group_bytes, int(per_layer_events))
+    check(lib.pf_plan_staged_fills(*args, None, 0, C.byref(n_units), C.byref(n_fills)))
+    out = (_lib.PfFillUnit * max(n_units.value, 1))()
+    check(lib.pf_plan_staged_fills(*args, out, n_units.value, C.byref(n_units), C.byref(n_fills)))
+    none = (1 << 64) - 1
+    units = [FillUnit(int(u.layer), int(u.first), int(u.count), int(u.slot_offset),
+                      None if u.fill == none else int(u.fill)) for u in out[: n_units.value]]
+    return units, int(n_fills.value)
+
+
 class BlockTransfer:
     """Block-ID gather (save) / scatter (load) engine.  Enqueue-only; one
     instance per worker thread."""

@@ -59,6 +59,14 @@ int main(void) {
 
   /* transfer/mod.rs:36-44 of the reference: device, host, host_device, size,
    * device_allocation, host_allocation, eight bytes each. */
+  BEGIN(pf_fill_unit, 40);
+  FIELD(pf_fill_unit, layer, 0);
+  FIELD(pf_fill_unit, first, 8);
+  FIELD(pf_fill_unit, count, 16);
+  FIELD(pf_fill_unit, slot_offset, 24);
+  FIELD(pf_fill_unit, fill, 32);
+  END();
+
   BEGIN(pf_copy_desc, 48);
   FIELD(pf_copy_desc, device, 0);
   FIELD(pf_copy_desc, host, 8);

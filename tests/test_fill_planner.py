@@ -1,0 +1,158 @@
+"""The planner that cuts the staged layers of a call into units and packs them
+into staging-slot fills (pf_plan_staged_fills, the function pf_xfer_save /
+pf_xfer_load use): hand-worked plans for the benchmark shapes and for the
+shapes the GPU tests run, and its invariants on random calls.  Host arithmetic
+only - no device."""
+
+from hypothesis import given, settings, strategies as st
+
+from pegaflow_amd.transfer import plan_staged_fills
+
+MiB = 1 << 20
+KiB = 1 << 10
+MAX_UNIT_BLOCKS = 65535
+MIN_SPLIT = 16 * MiB
+MAX_FILL_UNITS = 128
+
+
+def fills_of(units):
+    """{fill: [(layer, first, count)]} in order."""
+    out = {}
+    for u in units:
+        if u.fill is not None:
+            out.setdefault(u.fill, []).append((u.layer, u.first, u.count))
+    return out
+
+
+def test_llama_shape_fills_every_slot():
+    # 32 layers x 5000 blocks x 64 KiB in 512 MiB slots: a slot holds 8192 blocks
+    units, fills = plan_staged_fills([5000] * 32, [64 * KiB] * 32)
+    assert fills == 20
+    by_fill = fills_of(units)
+    assert by_fill[0] == [(0, 0, 5000), (1, 0, 3192)]
+    assert by_fill[1] == [(1, 3192, 1808), (2, 0, 5000), (3, 0, 1384)]
+    # a fill stops short of the brim only where the next piece would be under 16 MiB (256 blocks)
+    for f in range(19):
+        assert 8192 - 256 < sum(c for _, _, c in by_fill[f]) <= 8192
+    assert sum(c for v in by_fill.values() for _, _, c in v) == 32 * 5000
+    assert [u.slot_offset for u in units[:2]] == [0, 5000 * 64 * KiB]
+
+
+def test_fp8_shape_two_layers_per_fill():
+    units, fills = plan_staged_fills([8192] * 80, [32 * KiB] * 80)
+    assert fills == 40
+    assert all(len(v) == 2 for v in fills_of(units).values())
+
+
+def test_per_layer_events_keep_layers_whole():
+    units, fills = plan_staged_fills([5000] * 32, [64 * KiB] * 32, per_layer_events=True)
+    assert fills == 32 and len(units) == 32
+    assert all(u.first == 0 and u.count == 5000 and u.slot_offset == 0 for u in units)
+    # small layers share a fill up to 32 MiB: 8 x 4 MiB each
+    units, fills = plan_staged_fills([64] * 32, [64 * KiB] * 32, per_layer_events=True)
+    assert fills == 4
+
+
+def test_small_layers_of_a_call_share_one_fill():
+    # 80 layers x 4 blocks x 64 KiB = 20 MiB: one fill; 200 layers: 128 + 72
+    _, fills = plan_staged_fills([4] * 80, [64 * KiB] * 80)
+    assert fills == 1
+    units, fills = plan_staged_fills([4] * 200, [64 * KiB] * 200)
+    assert fills == 2
+    assert [len(v) for v in fills_of(units).values()] == [128, 72]
+
+
+def test_split_pieces_are_at_least_16_mib():
+    # 40, 40, 24, 52, 2 MiB in 64 MiB slots (the GPU test's shapes)
+    blocks = [640, 1280, 768, 832, 61]
+    sizes = [64 * KiB, 32 * KiB, 32 * KiB, 64 * KiB, 32800]
+    units, fills = plan_staged_fills(blocks, sizes, staging_slot_bytes=64 * MiB)
+    assert fills == 3
+    assert fills_of(units) == {0: [(0, 0, 640), (1, 0, 768)],
+                               1: [(1, 768, 512), (2, 0, 768), (3, 0, 384)],
+                               2: [(3, 384, 448), (4, 0, 61)]}
+    # 40 + 30 MiB: the second layer would leave a 6 MiB tail -> it stays whole
+    units, fills = plan_staged_fills([640, 480], [64 * KiB] * 2, staging_slot_bytes=64 * MiB)
+    assert fills_of(units) == {0: [(0, 0, 640)], 1: [(1, 0, 480)]}
+
+
+def test_layer_larger_than_a_slot_and_unstaged_layers():
+    # 1.5 slots, an unstaged layer (block_bytes 0), then a small staged one
+    units, fills = plan_staged_fills([1536, 7, 16], [MiB, 0, MiB], staging_slot_bytes=1024 * MiB)
+    assert fills == 3
+    assert [(u.layer, u.first, u.count, u.fill) for u in units] == [
+        (0, 0, 1024, 0), (0, 1024, 512, 1), (1, 0, 7, None), (2, 0, 16, 2)]
+
+
+def test_units_never_exceed_one_grid_extent():
+    units, fills = plan_staged_fills([100, 68000], [8 * KiB, KiB], staging_slot_bytes=128 * MiB)
+    assert fills == 1
+    assert [(u.layer, u.first, u.count) for u in units] == [
+        (0, 0, 100), (1, 0, 65535), (1, 65535, 2465)]
+    units, _ = plan_staged_fills([200000], [KiB])
+    assert [u.count for u in units] == [65535, 65535, 65535, 3395]
+    assert all(u.fill == 0 for u in units)
+
+
+def test_empty_call_and_empty_layers():
+    assert plan_staged_fills([], []) == ([], 0)
+    units, fills = plan_staged_fills([0, 5, 0], [64 * KiB] * 3)
+    assert fills == 1 and [(u.layer, u.count) for u in units] == [(1, 5)]
+
+
+layer_strategy = st.tuples(st.integers(0, 70000),
+                           st.sampled_from([0, 1000, KiB, 4104, 16 * KiB, 64 * KiB, 72 * KiB, MiB]))
+
+
+@settings(max_examples=300, deadline=None)
+@given(layers=st.lists(layer_strategy, min_size=0, max_size=40),
+       slot=st.sampled_from([MiB, 32 * MiB, 64 * MiB, 512 * MiB]),
+       group=st.sampled_from([0, 0, 8 * MiB, 512 * MiB]),
+       events=st.booleans())
+def test_plan_invariants(layers, slot, group, events):
+    blocks = [b for b, _ in layers]
+    sizes = [s for _, s in layers]
+    units, fills = plan_staged_fills(blocks, sizes, staging_slot_bytes=slot,
+                                     staged_group_bytes=group, per_layer_events=events)
+    # every list position of every layer exactly once, in order, layers in order
+    covered = {}
+    last_layer = -1
+    for u in units:
+        assert u.layer >= last_layer
+        last_layer = u.layer
+        assert u.first == covered.get(u.layer, 0)
+        covered[u.layer] = u.first + u.count
+        assert u.count <= MAX_UNIT_BLOCKS or sizes[u.layer] == 0
+        assert (u.fill is None) == (sizes[u.layer] == 0)
+    for li, (b, s) in enumerate(layers):
+        if b or s == 0:
+            assert covered.get(li, 0) == b
+    # fills are numbered in order and hold their units back to back inside the slot
+    by_fill = {}
+    for u in units:
+        if u.fill is not None:
+            by_fill.setdefault(u.fill, []).append(u)
+    assert sorted(by_fill) == list(range(fills))
+    may_split = not events and group == 0
+    for f, us in by_fill.items():
+        assert len(us) <= MAX_FILL_UNITS
+        cursor = 0
+        for u in us:
+            assert u.slot_offset == cursor and cursor % 256 == 0
+            cursor += (u.count * sizes[u.layer] + 255) & ~255
+        # one block may exceed a slot (then it is alone); otherwise a fill fits its slot
+        if len(us) > 1 or us[0].count > 1:
+            assert cursor <= slot + 255 * len(us)
+    # a layer that fits a slot shares fills with others only whole, or in pieces of
+    # >= 16 MiB (a larger layer takes several fills anyway, and its tail may be short)
+    for li, (b, s) in enumerate(layers):
+        if s == 0 or b == 0 or b * s > slot:
+            continue
+        mine = [u for u in units if u.layer == li]
+        layer_fills = sorted({u.fill for u in mine})
+        if len(layer_fills) > 1:
+            for f in layer_fills:
+                shared = any(u.layer != li for u in by_fill[f])
+                piece = sum(u.count for u in mine if u.fill == f) * s
+                if shared:
+                    assert may_split and piece >= MIN_SPLIT
