@@ -461,8 +461,7 @@ __global__ __launch_bounds__(kLanes) void plain_copy_kernel(uint64_t dst, uint64
 template <int LT>
 __global__ __launch_bounds__(LT) void plain_tiles_kernel(uint64_t dst, uint64_t src,
                                                          uint64_t bytes) {
-  const uint64_t off = (static_cast<uint64_t>(blockIdx.y) * gridDim.x + blockIdx.x) * (LT * 16ull) +
-                       threadIdx.x * 16ull;
+  const uint64_t off = static_cast<uint64_t>(blockIdx.x) * (LT * 16ull) + threadIdx.x * 16ull;
   if (off < bytes) {
     const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const g_u32x4*>(src + off));
     __builtin_nontemporal_store(v, reinterpret_cast<g_u32x4*>(dst + off));
@@ -770,10 +769,11 @@ int launch_plain_copy(void* dst, const void* src, uint64_t bytes, int unroll, hi
   if (unroll == 0) {
     constexpr uint64_t kTile = kTileLanes * 16;
     const uint64_t n = (bytes + kTile - 1) / kTile;
-    const uint32_t gx = static_cast<uint32_t>(n < 65536 ? n : 65536);
-    const uint64_t gy = (n + gx - 1) / gx;
-    if (gy > 65535) return fail(PF_ERR_INVALID_ARGUMENT, "plain copy too large");
-    hipLaunchKernelGGL(plain_tiles_kernel<kTileLanes>, dim3(gx, static_cast<uint32_t>(gy), 1),
+    // Exactly one workgroup per tile, like the gather / scatter grids: a
+    // yardstick that launched idle workgroups (a 65 536-wide grid rounded up to
+    // whole rows: 18 % of them for a 327 MB copy) read 4 % low.
+    if (n > 0x7FFFFFFFull) return fail(PF_ERR_INVALID_ARGUMENT, "plain copy too large");
+    hipLaunchKernelGGL(plain_tiles_kernel<kTileLanes>, dim3(static_cast<uint32_t>(n), 1, 1),
                        dim3(kTileLanes, 1, 1), 0, s, reinterpret_cast<uint64_t>(dst),
                        reinterpret_cast<uint64_t>(src), bytes);
     hipError_t e0 = hipGetLastError();
