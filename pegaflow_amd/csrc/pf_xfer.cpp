@@ -86,7 +86,12 @@ int Xfer::ensure_slot(Slot& sl, uint64_t bytes) {
     sl.used = false;
   }
   uint64_t cap = std::max(bytes, slot_bytes_);
-  PF_HIP(hipMalloc(&sl.buf, cap));
+  const hipError_t e = hipMalloc(&sl.buf, cap);
+  if (e != hipSuccess) {
+    sl.buf = nullptr;
+    if (e == hipErrorOutOfMemory) staging_oom_ = true;  // run() may take the zero-copy path instead
+    return fail_hip(e, "hipMalloc of a staging slot");
+  }
   sl.cap = cap;
   return PF_OK;
 }
@@ -600,7 +605,24 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
 int Xfer::run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save,
               hipStream_t s) {
   began_ = false;
-  const int st = run_impl(layers, n_layers, path, save, s);
+  staging_oom_ = false;
+  int st = run_impl(layers, n_layers, path, save, s);
+  if (st != PF_OK && !began_ && staging_oom_ && path == PF_PATH_AUTO) {
+    // The device has no memory left for a staging slot (slots allocated on
+    // first use, or grown for an oversized block).  Nothing is enqueued yet,
+    // and the zero-copy path moves the same bytes without device memory: a
+    // slower neighbour for the model's kernels beats a failed transfer.  The
+    // next AUTO call tries to allocate again.
+    if (!staging_oom_logged_) {
+      staging_oom_logged_ = true;
+      log_line(LogLevel::Info,
+               "no device memory for a staging slot (%s): this transfer, and later ones while "
+               "that lasts, take the zero-copy path", last_error().c_str());
+    }
+    (void)hipGetLastError();
+    began_ = false;
+    st = run_impl(layers, n_layers, PF_PATH_ZEROCOPY, save, s);
+  }
   if (st != PF_OK && began_) {
     // Something was already enqueued, possibly on the side stream, which the
     // caller's synchronise of `s` would not cover: drain both before the

@@ -300,6 +300,8 @@ class Xfer {
   uint64_t auto_min_ = kDefaultAutoStagedMin;
   uint64_t call_min_ = 0;  // PF_PATH_AUTO: stage every dense layer of a call that moves this much (0 = off)
   int unroll_ = kDefaultUnroll;
+  bool staging_oom_ = false;         // the current call failed to allocate a staging slot
+  bool staging_oom_logged_ = false;
   uint64_t group_bytes_ = 0;  // 0 = fill the slot (kStagedGroupBytes while layer events are set)
 
   hipStream_t side_ = nullptr;

@@ -732,6 +732,46 @@ def test_long_layer_of_small_blocks_behind_another_layer_in_one_fill(stream):
         h.close()
 
 
+def test_auto_takes_zero_copy_when_no_staging_slot_can_be_allocated(stream):
+    """A staging slot the device cannot hold (1 TiB): PF_PATH_AUTO moves the
+    same bytes over the zero-copy path instead of failing; an explicit
+    PF_PATH_STAGED reports the allocation error and touches nothing."""
+    rng = np.random.default_rng(808)
+    c = Case(rng, num_blocks=256, seg=32768, segments=2, n_ids=200)
+    L = c.product_layout()
+    n, stride = len(c.ids), L.host_stride
+    h = PinnedMemory(2 * n * stride)
+    h.as_numpy()[:] = SENT
+    c.dev.copy_from_host(c.cache0)
+    layer = _dense_layer(c, L, h, c.ids)
+    xfer = BlockTransfer(staging_slot_bytes=1 << 40, auto_staged_min_bytes=1)
+    with pytest.raises(_lib.PegaHipError, match="staging slot"):
+        xfer.save([layer], stream, TransferPath.STAGED)
+    stream.synchronize()
+    assert (h.as_numpy() == SENT).all()
+    for _ in range(2):                       # the second call finds the slots still missing
+        h.as_numpy()[:] = SENT
+        xfer.save([layer], stream, TransferPath.AUTO)
+        stream.synchronize()
+        assert xfer.last_path == ZC
+        oc = c.cache0.copy()
+        ok = np.full(n * stride, SENT, dtype=np.uint8)
+        ov = np.full(n * stride, SENT, dtype=np.uint8)
+        O.transfer_layer(c.oracle_layout(oc), c.ids, ok, ov, host_is_src=False)
+        assert np.array_equal(h.as_numpy()[: n * stride], ok)
+        assert np.array_equal(h.as_numpy()[n * stride:], ov)
+    c.dev.fill(SENT)
+    xfer.load([layer], stream, TransferPath.AUTO)
+    stream.synchronize()
+    assert xfer.last_path == ZC
+    oc = np.full_like(c.cache0, SENT)
+    O.transfer_layer(c.oracle_layout(oc), c.ids, ok, ov, host_is_src=True)
+    assert np.array_equal(c.dev.copy_to_host(), oc)
+    xfer.close()
+    c.close()
+    h.close()
+
+
 def test_call_size_rule_stages_small_layers_of_a_long_call(stream):
     """auto_staged_min_call_bytes: PF_PATH_AUTO stages the dense layers of a
     call whose dense bytes reach the threshold even though no layer reaches
