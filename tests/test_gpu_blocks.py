@@ -604,8 +604,9 @@ def test_small_staged_layers_share_slots_and_launches(stream, copy_stream):
     pool.close()
 
 
+@pytest.mark.parametrize("kind", ["mixed", "contiguous"])
 @pytest.mark.parametrize("copy_stream", [0, 2], ids=["side_stream", "in_order"])
-def test_layers_split_across_staging_slot_fills(stream, copy_stream):
+def test_layers_split_across_staging_slot_fills(stream, copy_stream, kind):
     """Without per-layer events a staging slot is filled to the brim: whole
     layers while they fit, then the head of the next layer, whose tail opens
     the following fill.  Five layers of 40, 40, 24, 52 and 2 MiB in 64 MiB
@@ -620,6 +621,10 @@ def test_layers_split_across_staging_slot_fills(stream, copy_stream):
               dict(num_blocks=800, seg=16384, segments=2, n_ids=768),     # 24 MiB
               dict(num_blocks=900, seg=32768, segments=2, n_ids=832),     # 52 MiB
               dict(num_blocks=64, seg=16400, segments=2, n_ids=61)]       # ~2 MiB, fragments with a tail
+    if kind == "contiguous":
+        # the same sizes with one segment per block everywhere (MLA-like): the
+        # one-segment form of the launch
+        shapes = [dict(kw, seg=kw["seg"] * kw["segments"], segments=1) for kw in shapes]
     cases = [Case(rng, **kw) for kw in shapes]
     hosts, layers, Ls = [], [], []
     for c in cases:
