@@ -668,7 +668,11 @@ FillPlan plan_staged_fills(const std::vector<FillLayer>& layers, uint64_t slot_b
         // A fresh fill takes up to a whole slot of this layer.
         take = std::min(remaining, slot_blocks);
       } else {
-        const uint64_t room = group_cap > used ? (group_cap - used) / block_bytes : 0;
+        // A layer that opened the fill may go on to the end of the slot (it came
+        // back here only because a unit is capped at one grid extent); behind
+        // other layers the fill ends at the group size.
+        const uint64_t cap = plan.units[fill_start].layer == li ? slot_bytes : group_cap;
+        const uint64_t room = cap > used ? (cap - used) / block_bytes : 0;
         const bool full = plan.units.size() - fill_start >= kStagedGroupUnits;
         if (!full && room >= remaining) {
           take = remaining;  // the rest of the layer fits

@@ -4,7 +4,7 @@ pf_xfer_load use): hand-worked plans for the benchmark shapes and for the
 shapes the GPU tests run, and its invariants on random calls.  Host arithmetic
 only - no device."""
 
-from hypothesis import given, settings, strategies as st
+from hypothesis import example, given, settings, strategies as st
 
 from pegaflow_amd.transfer import plan_staged_fills
 
@@ -94,6 +94,16 @@ def test_units_never_exceed_one_grid_extent():
     assert all(u.fill == 0 for u in units)
 
 
+def test_long_layer_keeps_its_fill_under_per_layer_events():
+    # 65 536 rows of 1000 bytes fit a 64 MiB slot but not one grid extent: two
+    # units of one fill, although per-layer events cap shared fills at 32 MiB
+    units, fills = plan_staged_fills([65536, 1], [1000, 1000], staging_slot_bytes=64 * MiB,
+                                     per_layer_events=True)
+    assert fills == 2
+    assert [(u.layer, u.first, u.count, u.fill) for u in units] == [
+        (0, 0, 65535, 0), (0, 65535, 1, 0), (1, 0, 1, 1)]
+
+
 def test_empty_call_and_empty_layers():
     assert plan_staged_fills([], []) == ([], 0)
     units, fills = plan_staged_fills([0, 5, 0], [64 * KiB] * 3)
@@ -104,7 +114,11 @@ layer_strategy = st.tuples(st.integers(0, 70000),
                            st.sampled_from([0, 1000, KiB, 4104, 16 * KiB, 64 * KiB, 72 * KiB, MiB]))
 
 
-@settings(max_examples=300, deadline=None)
+# derandomize: the same examples on every machine and in every run
+@settings(max_examples=400, deadline=None, derandomize=True, database=None)
+@example(layers=[(65536, 1000), (1, 1000)], slot=64 * MiB, group=0, events=True)
+@example(layers=[(65, 16384), (1, 1000)], slot=MiB, group=0, events=False)
+@example(layers=[(5000, 64 * KiB)] * 32, slot=512 * MiB, group=0, events=False)
 @given(layers=st.lists(layer_strategy, min_size=0, max_size=40),
        slot=st.sampled_from([MiB, 32 * MiB, 64 * MiB, 512 * MiB]),
        group=st.sampled_from([0, 0, 8 * MiB, 512 * MiB]),
