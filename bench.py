@@ -114,6 +114,9 @@ def parse_args():
                     help="staged path: 0 default, 1 link copies on a side stream, 2 in order on "
                          "the caller's stream (kernels then never overlap a copy)")
     ap.add_argument("--no-overlap", action="store_true", help="skip the GEMM-overlap section")
+    ap.add_argument("--engine-side-streams", action="store_true",
+                    help="engine section: workers move their link copies on a second stream each "
+                         "(pf_engine_config.side_copy_streams)")
     ap.add_argument("--gemm-m", type=int, default=4096,
                     help="edge of the square bf16 GEMMs of the overlap section (BASELINE: 4096)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -480,7 +483,7 @@ def run_workload(args, workload, sections, torch, np):
         torch.cuda.synchronize()
         return run_engine(torch, np, runtime, w, names, src_cache, dst_cache, save_ids, load_ids,
                           payload, args.engine_mode, args.engine_descriptors,
-                          args.engine_lazy_staging)
+                          args.engine_lazy_staging, args.engine_side_streams)
     t0 = time.time()
     pool = PinnedMemory(payload)
     pool_alloc_s = time.time() - t0
@@ -767,9 +770,11 @@ def run_workload(args, workload, sections, torch, np):
     if "engine" in sections:
         import subprocess
         engine_pause = pause_after_free(runtime, released)
-        def engine_run(mode):
+        def engine_run(mode, side_streams=False):
             cmd = [sys.executable, os.path.abspath(__file__), "--engine-child", "--workload",
                    workload, "--seed", str(args.seed), "--engine-mode", mode]
+            if side_streams or args.engine_side_streams:
+                cmd.append("--engine-side-streams")
             if args.engine_descriptors:
                 cmd.append("--engine-descriptors")
             if args.engine_lazy_staging:
@@ -793,6 +798,17 @@ def run_workload(args, workload, sections, torch, np):
         engine["other_mode"] = engine_run(other)
         engine["other_mode"]["pause_before"] = other_pause
         released += 4 << 30
+        # The opt-in form of the staged workers: link copies on a second stream per
+        # worker (pf_engine_config.side_copy_streams), for comparison.
+        if not args.engine_side_streams and args.engine_mode != "zerocopy":
+            side_pause = pause_after_free(runtime, released)
+            side = engine_run(args.engine_mode, side_streams=True)
+            engine["side_copy_streams"] = {
+                k: side.get(k) for k in ("save_gbps", "load_gbps", "save_gbps_first",
+                                         "load_gbps_first", "save_gbps_all", "load_gbps_all",
+                                         "concurrent_save_and_load", "staging_mib")}
+            engine["side_copy_streams"]["pause_before"] = side_pause
+            released += 4 << 30
 
     # ---- CPU baseline: the oracle's memcpy executor on the host cores -----
     cpu = None
@@ -1208,7 +1224,7 @@ def run_ref_cpu_path():
 
 
 def run_engine(torch, np, runtime, w, names, src_cache, dst_cache, save_ids, load_ids, payload,
-               mode_name="direct", descriptors=False, lazy_staging=False):
+               mode_name="direct", descriptors=False, lazy_staging=False, side_copy_streams=False):
     """End to end through pf_engine_*: registration, batch_save (host image
     allocation in the pinned pool, one worker task, block bookkeeping), prefix
     query, batch_load into a second instance of the same namespace.  Times are
@@ -1222,7 +1238,8 @@ def run_engine(torch, np, runtime, w, names, src_cache, dst_cache, save_ids, loa
     nseg = 2 if w["split"] else 1
     n_layers = len(names)
     eng = PegaEngine(pool_size=int(payload * 2.3) + (256 << 20),
-                     use_descriptor_backends=descriptors, lazy_staging=lazy_staging)
+                     use_descriptor_backends=descriptors, lazy_staging=lazy_staging,
+                     side_copy_streams=side_copy_streams)
     kv = nb * seg if nseg == 2 else 0
     for inst, caches in (("bench-src", src_cache), ("bench-dst", dst_cache)):
         eng.register_context_layer_batch(
@@ -1238,7 +1255,7 @@ def run_engine(torch, np, runtime, w, names, src_cache, dst_cache, save_ids, loa
     out = {"transfer_mode": mode_name, "worker_form": "descriptors" if descriptors else "block ids",
            "link_before_first_task": link_check(runtime),
            "staging_mib_after_registration": eng.staging_bytes >> 20,
-           "lazy_staging": bool(lazy_staging)}
+           "lazy_staging": bool(lazy_staging), "side_copy_streams": bool(side_copy_streams)}
     reps = 5
     save_s, load_s, query_s, load_profiles = [], [], [], []
     for rep in range(reps):

@@ -134,7 +134,7 @@ class PfTaskResult(C.Structure):
 class PfWorkerPoolConfig(C.Structure):
     _fields_ = [("device_id", C.c_int32), ("numa_node", C.c_int32), ("transfer_mode", C.c_int32),
                 ("use_descriptor_backends", u32), ("staging_slot_bytes", u64),
-                ("auto_staged_min_bytes", u64), ("lazy_staging", u32), ("reserved", u32)]
+                ("auto_staged_min_bytes", u64), ("lazy_staging", u32), ("side_copy_streams", u32)]
 
 
 class PfEngineConfig(C.Structure):
@@ -143,7 +143,7 @@ class PfEngineConfig(C.Structure):
                 ("use_descriptor_backends", u32), ("unit_size_hint", u64),
                 ("lease_ttl_ms", u64), ("auto_staged_min_bytes", u64),
                 ("staging_slot_bytes", u64), ("lazy_staging", u32),
-                ("kernel_mode_zerocopy", u32)]
+                ("kernel_mode_zerocopy", u32), ("side_copy_streams", u32), ("reserved", u32)]
 
 
 class PfIpcTensor(C.Structure):

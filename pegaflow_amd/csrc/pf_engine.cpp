@@ -299,6 +299,7 @@ int Engine::register_context_layer_batch_strided(
   options.use_descriptor_backends = cfg_.use_descriptor_backends;
   options.auto_staged_min_bytes = cfg_.auto_staged_min_bytes;
   options.lazy_staging = cfg_.lazy_staging;
+  options.side_copy_streams = cfg_.side_copy_streams;
   // A staging slot is filled with as many whole layers of a task as fit, so it
   // never needs to be larger than everything the context registered: a context
   // of small layers gets small slots.  Small layers that follow one another

@@ -43,6 +43,7 @@ struct EngineConfig {
   uint64_t staging_slot_bytes = 0;
   // Workers allocate their staging on the first staged task, not at registration.
   bool lazy_staging = false;
+  bool side_copy_streams = false;
   // Registrations that ask for TransferMode::Kernel get zero-copy workers (the
   // reference's meaning of that mode: one copy kernel over mapped host memory,
   // gpu_worker.rs:264-276) instead of the per-task choice.

@@ -164,6 +164,7 @@ int pf_worker_pool_spawn_ex(const pf_worker_pool_config* cfg, pf_worker_pool_t* 
   options.staging_slot_bytes = cfg->staging_slot_bytes;
   options.auto_staged_min_bytes = cfg->auto_staged_min_bytes;
   options.lazy_staging = cfg->lazy_staging != 0;
+  options.side_copy_streams = cfg->side_copy_streams != 0;
   std::string err;
   int status = PF_ERR_DEVICE_INIT;
   auto pool = pf::GpuWorkerPool::spawn(cfg->device_id, pf::NumaNode::from_int(cfg->numa_node),
@@ -320,6 +321,7 @@ int pf_engine_create(const pf_engine_config* cfg, pf_engine_t* out) {
   c.auto_staged_min_bytes = cfg->auto_staged_min_bytes;
   c.staging_slot_bytes = cfg->staging_slot_bytes;
   c.lazy_staging = cfg->lazy_staging != 0;
+  c.side_copy_streams = cfg->side_copy_streams != 0;
   c.kernel_mode_zerocopy = cfg->kernel_mode_zerocopy != 0;
   std::string err;
   int status = PF_ERR_STORAGE;

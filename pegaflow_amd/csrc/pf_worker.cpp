@@ -379,6 +379,16 @@ class DeviceScope {
 
 std::mutex g_worker_streams_mu;
 std::vector<std::pair<int, hipStream_t>> g_worker_streams;  // (device, stream) of live pools
+// The same for the copy streams of pools with side_copy_streams, and which
+// direction each serves: a clash between copy streams of one direction costs
+// nothing (they share the link anyway), one across directions costs the overlap
+// of a save with a load.
+struct SideStream {
+  int device;
+  hipStream_t stream;
+  bool is_load;
+};
+std::vector<SideStream> g_side_streams;
 
 // Do kernels of `candidate` (idle by construction) and `other` run side by side?
 // `other` belongs to a live pool and may receive a task at any moment: a probe
@@ -467,10 +477,58 @@ void GpuWorkerPool::separate_worker_queues() {
     queue_clashes_ += best_clashes;
     others.push_back(best);
   }
+  // The copy streams of a pool with side_copy_streams: each on a queue that
+  // none of the pool's other streams uses, nor a worker or copy stream of
+  // another pool that serves the opposite direction (kernels and copies of one
+  // direction may queue behind one another across pools; they share the link).
+  if (options_.side_copy_streams) {
+    for (Worker* w : {&save_, &load_}) {
+      if (w->side == nullptr) continue;
+      const bool is_load = w == &load_;
+      std::vector<hipStream_t> avoid = {save_.stream, load_.stream};
+      if (is_load && save_.side != nullptr) avoid.push_back(save_.side);
+      for (const SideStream& other : g_side_streams) {
+        if (other.device == device_id_ && other.is_load != is_load && avoid.size() < 8 &&
+            hipStreamQuery(other.stream) == hipSuccess) {
+          avoid.push_back(other.stream);
+        }
+      }
+      // Worker streams are registered in pairs, save then load.
+      for (size_t i = 0; i < g_worker_streams.size(); ++i) {
+        const bool other_is_load = (i & 1) != 0;
+        if (g_worker_streams[i].first == device_id_ && other_is_load != is_load &&
+            avoid.size() < 8 && hipStreamQuery(g_worker_streams[i].second) == hipSuccess) {
+          avoid.push_back(g_worker_streams[i].second);
+        }
+      }
+      (void)hipGetLastError();
+      hipStream_t best = w->side;
+      size_t best_clashes = clashes(best, avoid);
+      for (int attempt = 0; attempt < 8 && best_clashes != 0; ++attempt) {
+        hipStream_t fresh = nullptr;
+        if (hipStreamCreateWithFlags(&fresh, hipStreamNonBlocking) != hipSuccess) break;
+        const size_t c = clashes(fresh, avoid);
+        if (c < best_clashes) {
+          rejected.push_back(best);
+          best = fresh;
+          best_clashes = c;
+        } else {
+          rejected.push_back(fresh);
+        }
+      }
+      {
+        std::lock_guard<std::mutex> lock(w->mu);
+        w->side = best;
+      }
+      queue_clashes_ += best_clashes;
+    }
+  }
   for (hipStream_t s : rejected) (void)hipStreamDestroy(s);
   (void)hipGetLastError();
   g_worker_streams.emplace_back(device_id_, save_.stream);
   g_worker_streams.emplace_back(device_id_, load_.stream);
+  if (save_.side) g_side_streams.push_back({device_id_, save_.side, false});
+  if (load_.side) g_side_streams.push_back({device_id_, load_.side, true});
 }
 
 // Measured on MI355X with this runtime: whether the link copies of the save
@@ -491,14 +549,17 @@ void GpuWorkerPool::prime_copy_overlap() {
     std::memset(prime_host_, 0, 2 * chunk);
     uint8_t* h = static_cast<uint8_t*>(prime_host_);
     uint8_t* d = static_cast<uint8_t*>(prime_dev_);
+    // On the streams that will carry the copies.
+    hipStream_t save_copies = save_.side ? save_.side : save_.stream;
+    hipStream_t load_copies = load_.side ? load_.side : load_.stream;
     for (int i = 0; i < 6; ++i) {
-      (void)hipMemcpyAsync(h, d, chunk, hipMemcpyDeviceToHost, save_.stream);
+      (void)hipMemcpyAsync(h, d, chunk, hipMemcpyDeviceToHost, save_copies);
     }
     for (int i = 0; i < 3; ++i) {
-      (void)hipMemcpyAsync(d + chunk, h + chunk, chunk, hipMemcpyHostToDevice, load_.stream);
+      (void)hipMemcpyAsync(d + chunk, h + chunk, chunk, hipMemcpyHostToDevice, load_copies);
     }
-    (void)hipStreamSynchronize(save_.stream);
-    (void)hipStreamSynchronize(load_.stream);
+    (void)hipStreamSynchronize(save_copies);
+    (void)hipStreamSynchronize(load_copies);
   }
   (void)hipGetLastError();
 }
@@ -510,6 +571,10 @@ GpuWorkerPool::~GpuWorkerPool() {
     for (auto it = g_worker_streams.begin(); it != g_worker_streams.end();) {
       const bool mine = it->second == save_.stream || it->second == load_.stream;
       it = mine ? g_worker_streams.erase(it) : it + 1;
+    }
+    for (auto it = g_side_streams.begin(); it != g_side_streams.end();) {
+      const bool mine = it->stream == save_.side || it->stream == load_.side;
+      it = mine ? g_side_streams.erase(it) : it + 1;
     }
   }
   for (Worker* w : {&load_, &save_}) {
@@ -572,8 +637,13 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
   hipEvent_t done = nullptr;
   std::unique_ptr<TransferBackend> backend;
   std::unique_ptr<Xfer> xfer;
+  hipStream_t side = nullptr;
   hipError_t e = hipSetDevice(device_id_);
   if (e == hipSuccess) e = hipStreamCreateWithFlags(&stream, hipStreamNonBlocking);
+  if (e == hipSuccess && options_.side_copy_streams && !options_.use_descriptor_backends &&
+      mode_ != TransferMode::ZeroCopy) {
+    e = hipStreamCreateWithFlags(&side, hipStreamNonBlocking);
+  }
   if (e == hipSuccess) e = hipEventCreateWithFlags(&done, hipEventDisableTiming);
   if (e != hipSuccess) {
     fail_hip(e, "worker init");
@@ -591,7 +661,10 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
       // active alone (see also prime_copy_overlap).
       pf_xfer_config cfg;
       std::memset(&cfg, 0, sizeof(cfg));
-      cfg.copy_stream = 2;
+      // With side_copy_streams the pool gives each worker a second stream for
+      // the link copies, placed and primed like the worker streams (see
+      // separate_worker_queues, prime_copy_overlap).
+      cfg.copy_stream = side != nullptr ? 1 : 2;
       // The workers move KV beside a running model, so they also stage tasks
       // of small layers once the task is long enough for the resident
       // zero-copy kernel to matter to the kernels beside it.  A stream of
@@ -623,9 +696,11 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
     }
   }
   w->stream = stream;
+  w->side = side;
   ready->set_value(init);
   if (init.status != PF_OK) {
     if (done) (void)hipEventDestroy(done);
+    if (side) (void)hipStreamDestroy(side);
     if (stream) (void)hipStreamDestroy(stream);
     return;
   }
@@ -643,7 +718,9 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
       task = std::move(w->queue.front());
       w->queue.pop_front();
       stream = w->stream;  // the pool may have replaced it before the first task
+      side = w->side;
     }
+    if (xfer && side != nullptr) xfer->set_side_stream(side);
     // process_load_task / process_save_task, gpu_worker.rs:428-523.
     const auto t0 = std::chrono::steady_clock::now();
     TaskResult res;
@@ -813,6 +890,11 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
   {
     std::lock_guard<std::mutex> lock(w->mu);
     stream = w->stream;
+    side = w->side;
+  }
+  if (side) {
+    (void)hipStreamSynchronize(side);
+    (void)hipStreamDestroy(side);
   }
   (void)hipStreamDestroy(stream);
 }

@@ -100,6 +100,7 @@ struct WorkerPoolOptions {
   // false: both workers allocate their slots when the pool is spawned, so no
   // task pays for it; true: a worker allocates on its first staged task.
   bool lazy_staging = false;
+  bool side_copy_streams = false;  // link copies on a second stream per worker instead of in order
 };
 
 // gpu_worker.rs:29-52: how a finished load reports back.  Shm = a LoadState
@@ -155,6 +156,7 @@ class GpuWorkerPool {
     std::deque<std::unique_ptr<Task>> queue;
     bool stop = false;
     hipStream_t stream = nullptr;  // set by the worker before it reports ready
+    hipStream_t side = nullptr;    // link copies, with WorkerPoolOptions::side_copy_streams
   };
   // One large copy in each direction, in flight together, before the first task.
   void prime_copy_overlap();

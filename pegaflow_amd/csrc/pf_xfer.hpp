@@ -153,7 +153,7 @@ class Xfer {
   }
 
   ~Xfer() {
-    if (side_) {
+    if (side_ && side_owned_) {
       (void)hipStreamSynchronize(side_);
       (void)hipStreamDestroy(side_);
     }
@@ -206,6 +206,21 @@ class Xfer {
     return x;
   }
   int ensure_side_stream(hipStream_t s);
+
+  // The stream the link copies of the staged path run on when they do not run
+  // on the caller's (copy_stream 0 / 1): a stream of the caller's, which stays
+  // the caller's to destroy, instead of one this engine creates and places on
+  // first use.  Not while a call is in flight.
+  void set_side_stream(hipStream_t side) {
+    if (side == side_) return;
+    if (side_ && side_owned_) {
+      (void)hipStreamSynchronize(side_);
+      (void)hipStreamDestroy(side_);
+    }
+    side_ = side;
+    side_owned_ = side == nullptr;
+  }
+
   int run(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save, hipStream_t s);
   int run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, bool save,
                hipStream_t s);
@@ -305,6 +320,7 @@ class Xfer {
   uint64_t group_bytes_ = 0;  // 0 = fill the slot (kStagedGroupBytes while layer events are set)
 
   hipStream_t side_ = nullptr;
+  bool side_owned_ = true;  // created by ensure_side_stream, destroyed with the engine
   hipEvent_t fork_ = nullptr;
   hipEvent_t join_ = nullptr;
   std::vector<Slot> slots_;

@@ -145,16 +145,18 @@ class GpuWorkerPool:
 
     def __init__(self, device_id: int, numa_node: int = -1, transfer_mode: int = TransferMode.DIRECT,
                  use_descriptor_backends: bool = False, staging_slot_bytes: int = 0,
-                 auto_staged_min_bytes: int = 0, lazy_staging: bool = False):
+                 auto_staged_min_bytes: int = 0, lazy_staging: bool = False,
+                 side_copy_streams: bool = False):
         """A staging pool (block-ID engine, mode direct or kernel) holds
         2 workers x 2 slots of ``staging_slot_bytes`` (0 = 512 MiB) of device
         memory from here on, unless ``lazy_staging`` leaves the allocation to the
-        first staged task of each worker."""
+        first staged task of each worker.  ``side_copy_streams``: see PegaEngine."""
         self._lib = _lib.load()
         h = C.c_void_p()
         cfg = _lib.PfWorkerPoolConfig(device_id, numa_node, transfer_mode,
                                       1 if use_descriptor_backends else 0, staging_slot_bytes,
-                                      auto_staged_min_bytes, 1 if lazy_staging else 0, 0)
+                                      auto_staged_min_bytes, 1 if lazy_staging else 0,
+                                      1 if side_copy_streams else 0)
         check(self._lib.pf_worker_pool_spawn_ex(C.byref(cfg), C.byref(h)))
         self.handle = h
 
@@ -269,7 +271,7 @@ class PegaEngine:
                  use_descriptor_backends: bool = False, unit_size_hint: int = 0,
                  lease_ttl_ms: int = 0, auto_staged_min_bytes: int = 0,
                  staging_slot_bytes: int = 0, lazy_staging: bool = False,
-                 kernel_mode_zerocopy: bool = False):
+                 kernel_mode_zerocopy: bool = False, side_copy_streams: bool = False):
         """``lease_ttl_ms``: how long an unconsumed query lease pins its blocks
         (0 = the reference's 600 s, lease.rs:11).  ``auto_staged_min_bytes``: a
         task whose dense layers add up to this much is staged through device
@@ -282,13 +284,17 @@ class PegaEngine:
         min(this, what its layers can fill) in device memory from registration
         on, unless ``lazy_staging``.  ``kernel_mode_zerocopy``: registrations
         with TransferMode.KERNEL get zero-copy workers, the reference's meaning
-        of that mode, instead of the per-task choice."""
+        of that mode, instead of the per-task choice.  ``side_copy_streams``:
+        every worker moves its link copies on a second stream of its own (they
+        then overlap its gather / scatter kernels: 1-2 % for a direction running
+        alone) instead of in order on its one stream; four streams per context,
+        for processes with one context per GPU (pf_engine_config)."""
         self._lib = _lib.load()
         cfg = _lib.PfEngineConfig(pool_size, int(use_hugepages), int(numa_aware), pool_shards,
                                   int(blockwise_alloc), int(ssd_enabled),
                                   int(use_descriptor_backends), unit_size_hint, lease_ttl_ms,
                                   auto_staged_min_bytes, staging_slot_bytes, int(lazy_staging),
-                                  int(kernel_mode_zerocopy))
+                                  int(kernel_mode_zerocopy), int(side_copy_streams), 0)
         h = C.c_void_p()
         check(self._lib.pf_engine_create(C.byref(cfg), C.byref(h)))
         self.handle = h

@@ -21,6 +21,7 @@ sys.path.insert(0, ROOT)
 
 def main():
     layers = int(sys.argv[1]) if len(sys.argv) > 1 else 32
+    side_copy_streams = len(sys.argv) > 2 and sys.argv[2] == "side"
     import numpy as np
     from pegaflow_amd import runtime
     from pegaflow_amd.engine import LayerSave, PackedSaves, PegaEngine, worker_stream_report
@@ -39,7 +40,8 @@ def main():
         s_.copy_from_host(base)
         d_.fill(0)
     names = [f"model.layers.{i}.self_attn.attn" for i in range(layers)]
-    eng = PegaEngine(pool_size=int(payload * 2.3) + (256 << 20))
+    eng = PegaEngine(pool_size=int(payload * 2.3) + (256 << 20),
+                     side_copy_streams=side_copy_streams)
     out = {}
 
     def register(inst, caches):

@@ -187,10 +187,10 @@ int main(void) {
   FIELD(pf_worker_pool_config, staging_slot_bytes, 16);
   FIELD(pf_worker_pool_config, auto_staged_min_bytes, 24);
   FIELD(pf_worker_pool_config, lazy_staging, 32);
-  FIELD(pf_worker_pool_config, reserved, 36);
+  FIELD(pf_worker_pool_config, side_copy_streams, 36);
   END();
 
-  BEGIN(pf_engine_config, 72);
+  BEGIN(pf_engine_config, 80);
   FIELD(pf_engine_config, pool_size, 0);
   FIELD(pf_engine_config, use_hugepages, 8);
   FIELD(pf_engine_config, numa_aware, 12);
@@ -204,6 +204,8 @@ int main(void) {
   FIELD(pf_engine_config, staging_slot_bytes, 56);
   FIELD(pf_engine_config, lazy_staging, 64);
   FIELD(pf_engine_config, kernel_mode_zerocopy, 68);
+  FIELD(pf_engine_config, side_copy_streams, 72);
+  FIELD(pf_engine_config, reserved, 76);
   END();
 
   BEGIN(pf_layer_save, 40);

@@ -21,9 +21,13 @@ pytestmark = pytest.mark.gpu
 CHILD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "duplex_child.py")
 
 
-def test_two_pools_overlap_and_move_both_directions_at_once(gpu):
-    proc = subprocess.run([sys.executable, "-u", CHILD, "32"], capture_output=True, text=True,
-                          timeout=170)
+@pytest.mark.parametrize("copies", ["in_order", "side"])
+def test_two_pools_overlap_and_move_both_directions_at_once(gpu, copies):
+    """`side`: the same with pf_engine_config.side_copy_streams, a second
+    stream per worker for the link copies (worker_stream_report counts the
+    worker streams in both forms)."""
+    proc = subprocess.run([sys.executable, "-u", CHILD, "32", copies], capture_output=True,
+                          text=True, timeout=170)
     assert proc.returncode == 0, proc.stderr[-3000:]
     out = json.loads([ln for ln in proc.stdout.splitlines() if ln.startswith("{")][-1])
     print(json.dumps(out))

@@ -955,6 +955,55 @@ def test_lazy_staging_allocates_on_the_first_staged_task(gpu):
     dev.close()
 
 
+def test_side_copy_streams_move_the_same_bytes(gpu):
+    """pf_worker_pool_config.side_copy_streams: the workers' link copies on a
+    second stream each.  Four layers of 24 MiB in 32 MiB slots (several fills per
+    task, so copies and kernels do overlap), saved and loaded back into other
+    blocks; bytes as without the knob."""
+    rng = np.random.default_rng(79)
+    seg, nb, n, n_layers = 32768, 512, 384, 4
+    caches0 = [random_bytes(rng, 2 * nb * seg) for _ in range(n_layers)]
+    devs = [DeviceBuffer(c.nbytes) for c in caches0]
+    for d, c in zip(devs, caches0):
+        d.copy_from_host(c)
+    layouts = [KVCacheLayout(d.ptr, c.nbytes, nb, seg, nb * seg, 2) for d, c in zip(devs, caches0)]
+    pool = GpuWorkerPool(0, -1, TransferMode.DIRECT, staging_slot_bytes=32 << 20,
+                         side_copy_streams=True)
+    hosts = [PinnedMemory(2 * n * seg) for _ in range(n_layers)]
+    ids = rng.choice(nb, n, replace=False)
+
+    def blocks_of(host):
+        return [HostBlock((host.host_ptr + i * seg, host.host_ptr + (n + i) * seg),
+                          (host.device_ptr + i * seg, host.device_ptr + (n + i) * seg), (1, 2),
+                          (seg, seg)) for i in range(n)]
+
+    res = pool.batch_save([LayerTransferData(f"kv{li}", layouts[li], ids, blocks_of(hosts[li]))
+                           for li in range(n_layers)]).wait()
+    assert res.paths == ("staged",) and res.staged_groups >= 3
+    for li in range(n_layers):
+        img = hosts[li].as_numpy().reshape(2, n, seg)
+        kv = caches0[li].reshape(2, nb, seg)
+        assert np.array_equal(img[0], kv[0, ids]) and np.array_equal(img[1], kv[1, ids]), li
+    dest = rng.choice(nb, n, replace=False)
+    for d in devs:
+        d.fill(0)
+    res = pool.submit_load([LayerTransferData(f"kv{li}", layouts[li], dest, blocks_of(hosts[li]))
+                           for li in range(n_layers)]).wait()
+    assert res.paths == ("staged",) and res.staged_groups >= 3
+    rest = np.ones(nb, dtype=bool)
+    rest[dest] = False
+    for li in range(n_layers):
+        got = devs[li].copy_to_host().reshape(2, nb, seg)
+        kv = caches0[li].reshape(2, nb, seg)
+        assert np.array_equal(got[:, dest], kv[:, ids]), li
+        assert not got[:, rest].any(), li
+    pool.close()
+    for h in hosts:
+        h.close()
+    for d in devs:
+        d.close()
+
+
 def test_engine_load_profile_and_staging_report(gpu):
     """pf_engine_last_load_profile mirrors the task's own result; a context's
     staging is sized by what its layers can fill, not by the 512 MiB default;
