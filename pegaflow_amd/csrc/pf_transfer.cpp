@@ -237,9 +237,32 @@ int MemcpyBackend::submit(const CopyDesc* copies, uint64_t n, bool host_is_src, 
   return drained(submit_impl(copies, n, host_is_src, s), s);
 }
 
+// A long list that does not merge costs the submitting thread 6-7 ns per
+// descriptor (merging, sorting into runs, writing the table) before anything is
+// enqueued: 0.4 ms for 65 536 fragments of 4 KiB, a twelfth of their transfer.
+// Such a list goes piece by piece, everything in order on the stream, so that
+// the device works on one piece while the next is prepared (65 536 shuffled
+// 4 KiB fragments: 48.2 -> 49.3 GiB/s).  A list whose first piece merges into
+// few ranges is handed over whole: cutting it would only cut its large copies.
 int MemcpyBackend::submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_src,
                                hipStream_t s) {
+  constexpr uint64_t kPiece = 16384;
+  uint64_t done = 0;
+  while (n - done > kPiece + kPiece / 2) {
+    uint64_t ranges = 0;
+    const int st = submit_piece(copies + done, kPiece, host_is_src, s, &ranges);
+    if (st != PF_OK) return st;
+    done += kPiece;
+    if (ranges * 16 <= kPiece) break;
+  }
+  uint64_t ranges = 0;
+  return done < n ? submit_piece(copies + done, n - done, host_is_src, s, &ranges) : PF_OK;
+}
+
+int MemcpyBackend::submit_piece(const CopyDesc* copies, uint64_t n, bool host_is_src,
+                                hipStream_t s, uint64_t* out_ranges) {
   const std::vector<Range> ranges = merge_ranges(copies, n);
+  *out_ranges = ranges.size();
   const char* what = host_is_src ? "hipMemcpyHtoDAsync" : "hipMemcpyDtoHAsync";
   if (ranges.size() <= kFewRanges) {
     for (const Range& r : ranges) {

@@ -92,6 +92,9 @@ class MemcpyBackend : public TransferBackend {
  private:
   int submit(const CopyDesc* copies, uint64_t n, bool host_is_src, hipStream_t s);
   int submit_impl(const CopyDesc* copies, uint64_t n, bool host_is_src, hipStream_t s);
+  // One piece of a batch; *out_ranges = merged ranges it came to.
+  int submit_piece(const CopyDesc* copies, uint64_t n, bool host_is_src, hipStream_t s,
+                   uint64_t* out_ranges);
   SlabPool slabs_;
   // One staging buffer serves every batch.  Batches on one stream are ordered
   // by the stream; a batch on another stream first waits for `staging_done_`,

@@ -115,12 +115,14 @@ def test_unaligned_and_odd_sizes_match_oracle(backends, stream, direction):
     host.close()
 
 
-@pytest.mark.parametrize("n", [4096, 16385])
+@pytest.mark.parametrize("n", [4096, 16385, 40001])
 def test_shuffled_4k_fragments(backends, stream, n):
     """Shape of the reference's transfer bench (benches/transfer_h2d.rs):
     4096-byte fragments in a seeded shuffled order, device strided by two.
     The larger, odd count makes the direct backend's packing launch take two
-    fragments per workgroup with one left over."""
+    fragments per workgroup with one left over; the largest goes through the
+    direct backend in pieces (lists that do not merge are submitted 16 384
+    descriptors at a time)."""
     seg = 4096
     perm = xorshift_shuffle(n)
     assert sorted(perm) == list(range(n))
@@ -263,12 +265,15 @@ def _run_both_directions(backend, stream, descs_fn, dev_bytes, host_bytes, rows,
         host.close()
 
 
-def test_direct_backend_packs_host_dense_runs(stream, gpu):
+@pytest.mark.parametrize("n", [3000, 21000])
+def test_direct_backend_packs_host_dense_runs(stream, gpu, n):
     """Many small ranges whose host sides follow one another (the batch image
     of a save): the direct backend stages them instead of one copy each.  K/V
-    style interleave over two host allocations, device side shuffled."""
+    style interleave over two host allocations, device side shuffled.  The
+    larger list (42 000 descriptors) is submitted in pieces, each with its own
+    runs through the one staging buffer."""
     from pegaflow_amd.transfer import desc_array
-    seg, n = 4096, 3000
+    seg = 4096
     perm = np.array(xorshift_shuffle(n), dtype=np.uint64)
     k_dev = perm * 2 * seg                       # K region: every other slot
     v_dev = (2 * n + perm * 2) * seg             # V region behind it
