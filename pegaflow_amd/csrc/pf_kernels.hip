@@ -401,16 +401,20 @@ struct RowEnds {
 template <int LT, bool TO_FAR, int SEGS>
 __global__ __launch_bounds__(LT) void block_tiles_rows_kernel(const BlockUnit* __restrict__ units,
                                                               RowEnds ends) {
+  // More rows than one grid extent are folded over grid.z: z = chunk * SEGS + segment.
+  const uint32_t chunk = SEGS == 2 ? blockIdx.z >> 1 : blockIdx.z;
+  const uint32_t seg = SEGS == 2 ? blockIdx.z & 1u : 0u;
+  const uint32_t row = chunk * gridDim.y + blockIdx.y;
   uint32_t unit = 0, first = 0;
 #pragma unroll
   for (uint32_t k = 0; k + 1 < kMaxRowUnits; ++k) {
-    if (blockIdx.y >= ends.end[k]) {
+    if (row >= ends.end[k]) {
       unit = k + 1;
       first = ends.end[k];
     }
   }
-  const uint32_t seg = SEGS == 2 ? blockIdx.z : 0u;
-  block_tiles_copy<LT, TO_FAR, const BlockUnit*>(units + unit, blockIdx.y - first, seg);
+  // (A row past the last unit's end, in the last chunk, finds no block there.)
+  block_tiles_copy<LT, TO_FAR, const BlockUnit*>(units + unit, row - first, seg);
 }
 
 // One unit, passed by value: its fields arrive with the kernel's arguments
@@ -616,8 +620,14 @@ int launch_block_tiles_rows(const BlockUnit* units, const BlockUnit* host_units,
     *launched = true;
     return PF_OK;
   }
-  if (rows > kMaxTileBlocks || gx > 0x7FFFFFFFull) return PF_OK;  // the caller takes another form
-  dim3 grid(static_cast<uint32_t>(gx), static_cast<uint32_t>(rows), max_seg);
+  // Rows beyond one grid extent go into further chunks of equal length along grid.z.
+  const uint64_t chunks = (rows + kMaxTileBlocks - 1) / kMaxTileBlocks;
+  const uint64_t gy = (rows + chunks - 1) / chunks;
+  if (chunks * max_seg > kMaxTileBlocks || rows >= 0xFFFFFFFFull || gx > 0x7FFFFFFFull) {
+    return PF_OK;  // the caller takes another form
+  }
+  dim3 grid(static_cast<uint32_t>(gx), static_cast<uint32_t>(gy),
+            static_cast<uint32_t>(chunks * max_seg));
   dim3 block(kTileLanes, 1, 1);
   if (max_seg == 2) {
     if (to_far) {

@@ -81,7 +81,7 @@ int launch_block_tiles(const BlockUnit* units, uint32_t n_units, uint32_t max_bl
 // Up to eight units of any lengths in one launch with no idle workgroups: the
 // rows of all units laid end to end along grid.y (`host_units` is the host
 // copy of `units`, read for the row counts).  *launched = false when the launch
-// does not fit this form (more units, or more than kMaxTileBlocks rows in all):
+// does not fit this form (more than eight units):
 // nothing was enqueued and the caller uses launch_block_tiles.
 int launch_block_tiles_rows(const BlockUnit* units, const BlockUnit* host_units, uint32_t n_units,
                             bool to_far, hipStream_t s, bool* launched);
