@@ -92,7 +92,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload",
                     choices=sorted(WORKLOADS) + ["ref_transfer_bench", "ref_cpu_path",
-                                                 "link_after_free", "launch_fit"],
+                                                 "link_after_free", "launch_fit",
+                                                 "fragment_sweep"],
                     default="llama8b",
                     help="ref_transfer_bench = the shapes of the reference's own "
                          "benches/transfer_h2d.rs through the descriptor backends; "
@@ -100,7 +101,9 @@ def parse_args():
                          "(long lists of 1 KiB blocks through save / query / load); "
                          "link_after_free = what a large hipFree does to the link copies that "
                          "follow it; launch_fit = duration of one staged gather / scatter launch "
-                         "against its bytes: the fixed cost of a launch and the steady rate")
+                         "against its bytes: the fixed cost of a launch and the steady rate; "
+                         "fragment_sweep = rate of the staged gather / scatter launches against "
+                         "the fragment size, 1 KiB to 256 KiB")
     ap.add_argument("--path", choices=["auto", "staged", "zerocopy"], default="auto")
     ap.add_argument("--layers", type=int, default=0, help="override the layer count")
     ap.add_argument("--slot-mb", type=int, default=0)
@@ -199,6 +202,9 @@ def main():
         return
     if args.workload == "launch_fit":
         print(json.dumps(run_launch_fit(torch, np, runtime)))
+        return
+    if args.workload == "fragment_sweep":
+        print(json.dumps(run_fragment_sweep(torch, np, runtime)))
         return
     if args.engine_child:
         print(json.dumps(run_workload(args, args.workload, {"engine_child"}, torch, np)))
@@ -432,6 +438,73 @@ def run_launch_fit(torch, np, runtime):
             "rows": rows, "fit": fits, "empty_event_pair_us": round(sorted(empty)[len(empty) // 2], 2),
             "note": "fixed_us includes the event bracket (empty_event_pair_us)",
             "device": runtime.device_name(0)}
+
+
+def run_fragment_sweep(torch, np, runtime):
+    """HBM rate of the staged gather / scatter launches against the fragment
+    size: eight K/V-split layers of 320 MiB payload per call (512 MiB staging
+    fills, five launches per direction), shuffled ids, every launch running alone
+    and bracketed by HIP events (the launch gap is inside the figure); one layer
+    of every size is checked block by block."""
+    from pegaflow_amd.layout import KVCacheLayout
+    from pegaflow_amd.runtime import PinnedMemory, Stream
+    from pegaflow_amd.transfer import BlockTransfer, LayerBlocks, TransferPath
+    dev = torch.device("cuda:0")
+    n_layers, target = 8, 320 << 20
+    pool = PinnedMemory(n_layers * target)
+    stream = Stream()
+    xfer = BlockTransfer()
+    xfer.set_kernel_timing(1)
+    rng = np.random.default_rng(0)
+    rows = []
+    for seg in (1024, 2048, 4096, 8192, 16384, 32768, 65536, 131072, 262144):
+        n = target // (2 * seg)
+        nb = int(n * 1.6)
+        src = [torch.empty(2 * nb * seg, device=dev, dtype=torch.uint8).random_(0, 256)
+               for _ in range(n_layers)]
+        dst = [torch.zeros(2 * nb * seg, device=dev, dtype=torch.uint8) for _ in range(n_layers)]
+        torch.cuda.synchronize()
+        save_ids = rng.permutation(nb)[:n].astype(np.uint32)
+        load_ids = rng.permutation(nb)[:n].astype(np.uint32)
+
+        def layers(caches, ids):
+            out = []
+            for li, t in enumerate(caches):
+                off = li * 2 * n * seg
+                out.append(LayerBlocks(
+                    layout=KVCacheLayout(t.data_ptr(), 2 * nb * seg, nb, seg, nb * seg, 2),
+                    block_ids=ids, host=(pool.host_ptr + off, pool.host_ptr + off + n * seg),
+                    host_device=(pool.device_ptr + off, pool.device_ptr + off + n * seg),
+                    host_len=(n * seg, n * seg), host_stride=seg, layer_name=f"l{li}"))
+            return out
+
+        sv, ld = layers(src, save_ids), layers(dst, load_ids)
+        for _rep in range(3):
+            xfer.save(sv, stream, TransferPath.STAGED)
+            stream.synchronize()
+            save_ms, save_launches = xfer.last_kernel_ms()
+            xfer.load(ld, stream, TransferPath.STAGED)
+            stream.synchronize()
+            load_ms, load_launches = xfer.last_kernel_ms()
+        got = dst[3].cpu().numpy().reshape(2, nb, seg)
+        want = src[3].cpu().numpy().reshape(2, nb, seg)
+        if not np.array_equal(got[:, load_ids], want[:, save_ids]):
+            print(f"bench.py: fragment sweep, {seg}-byte fragments: bytes differ", file=sys.stderr)
+            sys.exit(1)
+        alg = 2.0 * n_layers * 2 * n * seg
+        rows.append({"fragment_bytes": seg, "blocks_per_layer": n,
+                     "launches": [save_launches, load_launches],
+                     "gather_gbps": round(alg / save_ms / 1e6, 1),
+                     "scatter_gbps": round(alg / load_ms / 1e6, 1),
+                     "gather_frac_of_hbm_peak": round(alg / save_ms / 1e6 / HBM_PEAK_GBPS, 3),
+                     "scatter_frac_of_hbm_peak": round(alg / load_ms / 1e6 / HBM_PEAK_GBPS, 3)})
+        del src, dst, sv, ld
+        torch.cuda.empty_cache()
+    xfer.close()
+    stream.close()
+    pool.close()
+    return {"metric": "staged gather / scatter rate against the fragment size", "unit": "GB/s",
+            "rows": rows, "verified": True, "device": runtime.device_name(0)}
 
 
 def run_workload(args, workload, sections, torch, np):
