@@ -664,11 +664,12 @@ int launch_block_tiles(const BlockUnit* units, uint32_t n_units, uint32_t max_bl
   // page and every cache in ascending position order.  Measured on the
   // DeepSeek-V3 page-first shape (61 units x 119 pages per launch): gather
   // 5.3 -> 5.9 TB/s, scatter 5.5 -> 6.2 TB/s against positions-inner.
-  // A few large units (whole layers that share a staging slot) keep the order
-  // of a single unit, one (unit, segment) after the other: with 2-4 units per
-  // launch that form measured 1-2 % faster than units-inner (Llama shape,
-  // three layers per launch: 6.10 against 6.04 TB/s; fp8 shape, four: 6.18
-  // against 6.10).
+  // A few units of equal length (page packing of a model with few layers) keep
+  // the order of a single unit, one (unit, segment) after the other: with 2-4
+  // units per launch that form measured 1-2 % faster than units-inner (Llama
+  // shape, three layers per launch: 6.10 against 6.04 TB/s; fp8 shape, four:
+  // 6.18 against 6.10).  Staging fills of up to eight units of unlike lengths
+  // do not come here: launch_block_tiles_rows.
   constexpr uint32_t kUnitsInnerFrom = 9;
   const bool units_inner = n_units >= kUnitsInnerFrom;
   const uint32_t unit_segs = max_seg * n_units;
