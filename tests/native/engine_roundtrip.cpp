@@ -23,7 +23,7 @@ int run(bool page_first,int mode,bool desc,bool blockwise,int nseg,int L,uint64_
   const uint64_t layer_bytes=nseg*nb*seg;
   std::vector<void*> src(L),dst(L); std::vector<std::vector<uint8_t>> host(L);
   std::mt19937_64 rng(7);
-  for(int l=0;l<L;l++){ if(hipMalloc(&src[l],layer_bytes)||hipMalloc(&dst[l],layer_bytes)) return 2; host[l].resize(layer_bytes); for(auto& b:host[l]) b=(uint8_t)rng(); (void)hipMemcpy(src[l],host[l].data(),layer_bytes,hipMemcpyHostToDevice); (void)hipMemset(dst[l],0,layer_bytes);} 
+  for(int l=0;l<L;l++){ if(hipMalloc(&src[l],layer_bytes)||hipMalloc(&dst[l],layer_bytes)) return 2; host[l].resize(layer_bytes); { uint64_t* w8=reinterpret_cast<uint64_t*>(host[l].data()); for(uint64_t k=0;k<layer_bytes/8;k++) w8[k]=rng(); for(uint64_t k=layer_bytes&~7ull;k<layer_bytes;k++) host[l][k]=(uint8_t)rng(); } (void)hipMemcpy(src[l],host[l].data(),layer_bytes,hipMemcpyHostToDevice); (void)hipMemset(dst[l],0,layer_bytes);} 
   std::vector<std::string> names(L); std::vector<const char*> cn(L); for(int l=0;l<L;l++){ names[l]="model.layers."+std::to_string(l)+".attn"; cn[l]=names[l].c_str(); }
   std::vector<uint64_t> sz(L,layer_bytes),nbs(L,nb),bpb(L,seg),kvs(L,nseg==2?nb*seg:0),sg(L,nseg);
   for(int which=0;which<2;which++){
