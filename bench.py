@@ -784,6 +784,11 @@ def run_workload(args, workload, sections, torch, np):
     if staged_path:
         roofline["plain_copy_over_layers_gbps"] = {"from_caches": round(plain_gather_form, 1),
                                                    "into_caches": round(plain_scatter_form, 1)}
+        # the launches that ran alone against the id-less copy of the same memory
+        alone = roofline["launches_alone"]
+        roofline["frac_of_plain_copy_over_layers"] = {
+            "gather": round(alone["save_kernel_gbps"] / plain_gather_form, 3),
+            "scatter": round(alone["load_kernel_gbps"] / plain_scatter_form, 3)}
 
     link = {"bound": "pcie_gen5_x16", "theoretical_gbps": PCIE_GEN5_X16_GBPS,
             "measured_d2h_gbps": round(d2h_peak, 2), "measured_h2d_gbps": round(h2d_peak, 2),
