@@ -300,8 +300,8 @@ int Engine::register_context_layer_batch_strided(
   options.auto_staged_min_bytes = cfg_.auto_staged_min_bytes;
   options.lazy_staging = cfg_.lazy_staging;
   options.side_copy_streams = cfg_.side_copy_streams;
-  // A staging slot is filled with as many whole layers of a task as fit, so it
-  // never needs to be larger than everything the context registered: a context
+  // A staging slot is filled with the layers of a task one behind the other, so
+  // it never needs to be larger than everything the context registered: a context
   // of small layers gets small slots.  Small layers that follow one another
   // share up to 32 MiB of a slot even with per-layer events: that is the floor.
   {
