@@ -705,27 +705,36 @@ def run_workload(args, workload, sections, torch, np):
                                      stream.handle))
     hbm_copy_gbps = 2 * time_copy(plain, reps=20)
 
-    # The same yardstick over the memory the gather and the scatter touch: one
-    # plain copy of a layer's payload from the head of each layer's cache into
-    # a staging-sized buffer, and back into each destination cache -- what the
-    # kernels would do if the block ids were 0..n-1 and the layout one segment.
-    # Copying one buffer pair over and over (above) is placement-dependent and
-    # comes out 5-10 % faster than a walk over 32 different caches.
+    # The same yardstick over the memory the gather and the scatter touch: plain
+    # copies from the head of each layer's cache into a staging-sized buffer, and
+    # back into each destination cache -- what the kernels would do if the block
+    # ids were 0..n-1 and the layout one segment.  Measured the way the kernels'
+    # `launches_alone` are: every launch between a pair of events of its own (so
+    # the bracket is inside both figures), and of the size of a mean staged launch
+    # of this workload (a layer's cache at most).  Copying one buffer pair over
+    # and over (above) is placement-dependent and comes out faster than a walk
+    # over 32 different caches.
+    staged_launches_per_direction = max(live_launches_per_step // 2, 1)
+    plain_launch_bytes = min(payload // staged_launches_per_direction, layer_bytes, link_bytes) & ~15
+    plain_pairs = [(Event(timing=True), Event(timing=True)) for _ in range(3 * n_layers)]
+
     def plain_over_layers(to_cache):
-        def once():
+        def once(pairs):
             for li in range(n_layers):
                 cache = (dst_cache if to_cache else src_cache)[li].data_ptr()
                 a, b = (cache, scratch.data_ptr()) if to_cache else (scratch.data_ptr(), cache)
-                _lib.check(lib.pf_plain_copy(a, b, payload_per_layer, 0, stream.handle))
-        once()
+                if pairs:
+                    pairs[li][0].record(stream)
+                _lib.check(lib.pf_plain_copy(a, b, plain_launch_bytes, 0, stream.handle))
+                if pairs:
+                    pairs[li][1].record(stream)
+        once(None)
         stream.synchronize()
-        ev[0].record(stream)
-        for _ in range(3):
-            once()
-        ev[1].record(stream)
-        ev[1].synchronize()
-        return 2 * payload * 3 / (ev[0].elapsed_ms(ev[1]) / 1e3) / 1e9
-    assert payload_per_layer <= link_bytes
+        for rep in range(3):
+            once(plain_pairs[rep * n_layers: (rep + 1) * n_layers])
+        stream.synchronize()
+        total_ms = sum(a.elapsed_ms(b) for a, b in plain_pairs)
+        return 2 * plain_launch_bytes * len(plain_pairs) / (total_ms / 1e3) / 1e9
     plain_gather_form = plain_over_layers(False)
     plain_scatter_form = plain_over_layers(True)
 
@@ -783,7 +792,8 @@ def run_workload(args, workload, sections, torch, np):
                 "plain_copy_same_tile_gbps": round(hbm_copy_gbps, 1)}
     if staged_path:
         roofline["plain_copy_over_layers_gbps"] = {"from_caches": round(plain_gather_form, 1),
-                                                   "into_caches": round(plain_scatter_form, 1)}
+                                                   "into_caches": round(plain_scatter_form, 1),
+                                                   "bytes_per_launch": 2 * plain_launch_bytes}
         # the launches that ran alone against the id-less copy of the same memory
         alone = roofline["launches_alone"]
         roofline["frac_of_plain_copy_over_layers"] = {
