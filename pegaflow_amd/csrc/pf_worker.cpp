@@ -685,6 +685,16 @@ void GpuWorkerPool::run(Worker* w, bool is_load, NumaNode numa, std::promise<Tas
       int xst = xfer ? xfer->enable_profile() : PF_ERR_DEVICE_INIT;
       if (xst == PF_OK && mode_ != TransferMode::ZeroCopy && !options_.lazy_staging) {
         xst = xfer->reserve_staging();
+        if (xst != PF_OK && xfer->staging_out_of_memory()) {
+          // Not fatal: every task can cross the link with the zero-copy kernel,
+          // and each staged task tries the allocation again (Xfer::run).
+          log_line(LogLevel::Info,
+                   "worker pool on device %d: no device memory for the %s worker's staging slots "
+                   "(%s); its tasks take the zero-copy path until the slots can be allocated",
+                   device_id_, is_load ? "load" : "save", last_error().c_str());
+          (void)hipGetLastError();
+          xst = PF_OK;
+        }
       }
       if (xst != PF_OK) {
         init.status = PF_ERR_DEVICE_INIT;

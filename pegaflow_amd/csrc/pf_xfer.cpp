@@ -97,6 +97,7 @@ int Xfer::ensure_slot(Slot& sl, uint64_t bytes) {
 }
 
 int Xfer::reserve_staging() {
+  staging_oom_ = false;
   for (auto& sl : slots_) {
     const int st = ensure_slot(sl, slot_bytes_);
     if (st != PF_OK) return st;

@@ -206,6 +206,8 @@ class Xfer {
     return x;
   }
   int ensure_side_stream(hipStream_t s);
+  // Whether the last reserve_staging() or call failed for want of device memory.
+  bool staging_out_of_memory() const { return staging_oom_; }
 
   // The stream the link copies of the staged path run on when they do not run
   // on the caller's (copy_stream 0 / 1): a stream of the caller's, which stays

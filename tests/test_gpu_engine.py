@@ -955,6 +955,39 @@ def test_lazy_staging_allocates_on_the_first_staged_task(gpu):
     dev.close()
 
 
+def test_pool_without_room_for_staging_still_moves_tasks(gpu):
+    """A pool whose staging slots cannot be allocated (1 TiB each) is spawned
+    all the same, holds no staging memory, and moves a 32 MiB task - which it
+    would stage - over the zero-copy path, bytes as ever."""
+    rng = np.random.default_rng(80)
+    seg, nb, n = 32768, 1024, 512
+    cache0 = random_bytes(rng, 2 * nb * seg)
+    dev = DeviceBuffer(cache0.nbytes)
+    dev.copy_from_host(cache0)
+    layout = KVCacheLayout(dev.ptr, cache0.nbytes, nb, seg, nb * seg, 2)
+    pool = GpuWorkerPool(0, -1, TransferMode.DIRECT, staging_slot_bytes=1 << 40)
+    assert pool.staging_bytes == 0
+    host = PinnedMemory(2 * n * seg)
+    ids = rng.choice(nb, n, replace=False)
+    blocks = [HostBlock((host.host_ptr + i * seg, host.host_ptr + (n + i) * seg),
+                        (host.device_ptr + i * seg, host.device_ptr + (n + i) * seg), (1, 2),
+                        (seg, seg)) for i in range(n)]
+    res = pool.batch_save([LayerTransferData("kv", layout, ids, blocks)]).wait()
+    assert res.paths == ("zerocopy",)
+    img = host.as_numpy().reshape(2, n, seg)
+    kv = cache0.reshape(2, nb, seg)
+    assert np.array_equal(img[0], kv[0, ids]) and np.array_equal(img[1], kv[1, ids])
+    dest = rng.choice(nb, n, replace=False)
+    dev.fill(0)
+    res = pool.submit_load([LayerTransferData("kv", layout, dest, blocks)]).wait()
+    assert res.paths == ("zerocopy",)
+    got = dev.copy_to_host().reshape(2, nb, seg)
+    assert np.array_equal(got[:, dest], kv[:, ids])
+    pool.close()
+    host.close()
+    dev.close()
+
+
 def test_side_copy_streams_move_the_same_bytes(gpu):
     """pf_worker_pool_config.side_copy_streams: the workers' link copies on a
     second stream each.  Four layers of 24 MiB in 32 MiB slots (several fills per
