@@ -685,6 +685,69 @@ def test_layers_split_across_staging_slot_fills(stream, copy_stream, kind):
         h.close()
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_launches_follow_the_planner_on_random_calls(stream, seed):
+    """Random calls of 3-7 layers of 1-50 MiB (split and contiguous, 4-64 KiB
+    fragments) in 64 MiB slots: the number of gather and of scatter launches is
+    the number of fills pf_plan_staged_fills gives for the call, and the bytes
+    are the oracle's."""
+    from pegaflow_amd.transfer import plan_staged_fills
+    rng = np.random.default_rng(9000 + seed)
+    cases = []
+    for _ in range(int(rng.integers(3, 8))):
+        segments = int(rng.choice([1, 2]))
+        seg = int(rng.choice([4096, 16384, 32768, 65536]))
+        payload = int(rng.integers(1 << 20, 50 << 20))
+        n_ids = max(1, payload // (seg * segments))
+        cases.append(Case(rng, num_blocks=n_ids + int(rng.integers(1, 64)), seg=seg, segments=segments,
+                          n_ids=n_ids))
+    hosts, layers, Ls = [], [], []
+    for c in cases:
+        L = c.product_layout()
+        Ls.append(L)
+        nseg = 2 if L.is_split else 1
+        h = PinnedMemory(nseg * len(c.ids) * L.host_stride)
+        h.as_numpy()[:] = SENT
+        hosts.append(h)
+        c.dev.copy_from_host(c.cache0)
+        layers.append(_dense_layer(c, L, h, c.ids))
+    _units, fills = plan_staged_fills([len(c.ids) for c in cases],
+                                      [L.host_stride * (2 if L.is_split else 1) for L in Ls],
+                                      staging_slot_bytes=64 << 20)
+    xfer = BlockTransfer(staging_slot_bytes=64 << 20, staging_slots=2, auto_staged_min_bytes=1)
+    xfer.set_kernel_timing(1)
+    xfer.save(layers, stream, TransferPath.STAGED)
+    stream.synchronize()
+    assert xfer.last_kernel_ms()[1] == fills
+    images = []
+    for c, L, h in zip(cases, Ls, hosts):
+        n, stride = len(c.ids), L.host_stride
+        oc = c.cache0.copy()
+        ok = np.full(n * stride, SENT, dtype=np.uint8)
+        ov = np.full(n * stride, SENT, dtype=np.uint8) if L.is_split else None
+        O.transfer_layer(c.oracle_layout(oc), c.ids, ok, ov, host_is_src=False)
+        hv = h.as_numpy()
+        assert np.array_equal(hv[: n * stride], ok), c.args
+        if ov is not None:
+            assert np.array_equal(hv[n * stride:], ov), c.args
+        images.append((ok, ov))
+    for li, c in enumerate(cases):
+        c.dev.fill(SENT)
+        layers[li].block_ids = rng.choice(c.num_blocks, len(c.ids), replace=False).astype(np.uint32)
+    xfer.load(layers, stream, TransferPath.STAGED)
+    stream.synchronize()
+    assert xfer.last_kernel_ms()[1] == fills
+    for li, c in enumerate(cases):
+        oc = np.full_like(c.cache0, SENT)
+        ok, ov = images[li]
+        O.transfer_layer(c.oracle_layout(oc), layers[li].block_ids, ok, ov, host_is_src=True)
+        assert np.array_equal(c.dev.copy_to_host(), oc), li
+    xfer.close()
+    for c, h in zip(cases, hosts):
+        c.close()
+        h.close()
+
+
 def test_long_layer_of_small_blocks_behind_another_layer_in_one_fill(stream):
     """A layer of 68 000 blocks of 1 KiB (more rows than one grid extent)
     that fits the room a small layer left in the slot: it becomes two units
