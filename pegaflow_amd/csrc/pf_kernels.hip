@@ -32,7 +32,7 @@ typedef __attribute__((address_space(4))) const uint64_t c_u64;
 typedef __attribute__((address_space(4))) const BlockUnit c_unit;
 
 constexpr int kLanes = 256;
-constexpr uint32_t kMaxRowUnits = 8;  // units of one block_tiles_rows_kernel launch
+constexpr uint32_t kMaxRowUnits = kRowsLaunchUnits;  // units of one block_tiles_rows_kernel launch
 
 // 16-byte store with the cache policy "sc1 nt".  Measured on MI355X at the
 // Llama shape (5000 x 2 x 32 KiB gathered or scattered per launch) over all 49

@@ -1112,11 +1112,12 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     auto launch_group = [&](bool to_far) -> int {
       if (ue - ui == 1) return launch_tiles(units_dev + ui, units_host[ui], to_far, s);
       uint32_t max_blocks = 0, max_seg = 0;
-      uint64_t max_frag = 0;
+      uint64_t max_frag = 0, total_rows = 0;
       for (size_t k = ui; k < ue; ++k) {
         max_blocks = std::max(max_blocks, units_host[k].n_blocks);
         max_seg = std::max(max_seg, units_host[k].n_seg);
         max_frag = std::max(max_frag, units_host[k].frag_bytes);
+        total_rows += units_host[k].n_blocks;
       }
       int rc = timing_begin(s);
       if (rc != PF_OK) return rc;
@@ -1124,6 +1125,22 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
       rc = launch_block_tiles_rows(units_dev + ui, units_host + ui, static_cast<uint32_t>(ue - ui),
                                    to_far, s, &launched);
       if (rc != PF_OK) return rc;
+      // More units than the rows form takes: the grid of the units-inner form is
+      // sized by the longest unit, which suits units of one length (the layers
+      // of a model that share a block list).  When the lengths differ so much
+      // that a quarter of that grid would find no row (a task over cache groups
+      // of unlike size: 8 full-attention layers of 625 blocks among 40
+      // sliding-window layers of 8 leave 82 % of it idle), the fill goes out as
+      // several rows launches of a few units each instead (that task's gather:
+      // 240 -> 138 us, its scatter 241 -> 147 us).
+      if (!launched && total_rows * 4 < static_cast<uint64_t>(max_blocks) * (ue - ui) * 3) {
+        for (size_t k = ui; k < ue; k += kRowsLaunchUnits) {
+          const uint32_t count = static_cast<uint32_t>(std::min<size_t>(kRowsLaunchUnits, ue - k));
+          rc = launch_block_tiles_rows(units_dev + k, units_host + k, count, to_far, s, &launched);
+          if (rc != PF_OK) return rc;
+          if (!launched) break;
+        }
+      }
       if (!launched) {
         rc = launch_block_tiles(units_dev + ui, static_cast<uint32_t>(ue - ui), max_blocks, max_frag,
                                 max_seg, to_far, s);

@@ -748,6 +748,60 @@ def test_launches_follow_the_planner_on_random_calls(stream, seed):
         h.close()
 
 
+def test_fill_of_many_layers_of_unlike_length(stream):
+    """Twelve layers in one fill, two of 600 blocks among ten of 8 (a task over
+    cache groups of unlike size): more units than one rows launch takes and
+    too unlike for the grid of the units-inner form, so the fill goes out as
+    two rows launches (one timed group); bytes against the oracle both ways.
+    A second call of twelve equal layers takes the units-inner form."""
+    rng = np.random.default_rng(612)
+    for counts in ([8, 8, 600, 8, 8, 8, 8, 8, 600, 8, 8, 8], [40] * 12):
+        cases = [Case(rng, num_blocks=n + 24, seg=32768, segments=2 if li % 3 else 1, n_ids=n)
+                 for li, n in enumerate(counts)]
+        hosts, layers, Ls = [], [], []
+        for c in cases:
+            L = c.product_layout()
+            Ls.append(L)
+            nseg = 2 if L.is_split else 1
+            h = PinnedMemory(nseg * len(c.ids) * L.host_stride)
+            h.as_numpy()[:] = SENT
+            hosts.append(h)
+            c.dev.copy_from_host(c.cache0)
+            layers.append(_dense_layer(c, L, h, c.ids))
+        xfer = BlockTransfer(staging_slot_bytes=128 << 20, staging_slots=2, auto_staged_min_bytes=1)
+        xfer.set_kernel_timing(1)
+        xfer.save(layers, stream, TransferPath.STAGED)
+        stream.synchronize()
+        assert xfer.last_path == ST and xfer.last_kernel_ms()[1] == 1
+        images = []
+        for c, L, h in zip(cases, Ls, hosts):
+            n, stride = len(c.ids), L.host_stride
+            oc = c.cache0.copy()
+            ok = np.full(n * stride, SENT, dtype=np.uint8)
+            ov = np.full(n * stride, SENT, dtype=np.uint8) if L.is_split else None
+            O.transfer_layer(c.oracle_layout(oc), c.ids, ok, ov, host_is_src=False)
+            hv = h.as_numpy()
+            assert np.array_equal(hv[: n * stride], ok), c.args
+            if ov is not None:
+                assert np.array_equal(hv[n * stride:], ov), c.args
+            images.append((ok, ov))
+        for li, c in enumerate(cases):
+            c.dev.fill(SENT)
+            layers[li].block_ids = rng.choice(c.num_blocks, len(c.ids), replace=False).astype(np.uint32)
+        xfer.load(layers, stream, TransferPath.STAGED)
+        stream.synchronize()
+        assert xfer.last_kernel_ms()[1] == 1
+        for li, c in enumerate(cases):
+            oc = np.full_like(c.cache0, SENT)
+            ok, ov = images[li]
+            O.transfer_layer(c.oracle_layout(oc), layers[li].block_ids, ok, ov, host_is_src=True)
+            assert np.array_equal(c.dev.copy_to_host(), oc), li
+        xfer.close()
+        for c, h in zip(cases, hosts):
+            c.close()
+            h.close()
+
+
 def test_long_layer_of_small_blocks_behind_another_layer_in_one_fill(stream):
     """A layer of 68 000 blocks of 1 KiB (more rows than one grid extent)
     that fits the room a small layer left in the slot: it becomes two units
