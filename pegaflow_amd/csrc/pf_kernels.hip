@@ -473,6 +473,7 @@ __global__ __launch_bounds__(LT) void plain_tiles_kernel(uint64_t dst, uint64_t 
 }
 
 constexpr int kTileLanes = 128;  // lanes of a block_tiles_kernel workgroup
+static_assert(kTileLanes * 16 == kStagedTileBytes, "tile size the planner of launches assumes");
 constexpr uint32_t kMaxGridX = 1u << 22;  // the kernels grid-stride past this
 constexpr int kDescUnroll = 4;
 

@@ -65,6 +65,7 @@ int launch_block_units_args(const ArgSlab& slab, uint32_t first_unit, uint32_t n
 // Limits of one block_tiles launch (grid.y and grid.z are 16-bit).
 constexpr uint32_t kMaxTileBlocks = 65535;
 constexpr uint32_t kRowsLaunchUnits = 8;  // units one launch_block_tiles_rows call takes
+constexpr uint64_t kStagedTileBytes = 2048;  // bytes one workgroup of the staged kernels moves
 constexpr uint32_t kMaxTileUnits = 32767;
 
 // Launch the one-tile-per-workgroup form over `n_units` units: the HBM-bound

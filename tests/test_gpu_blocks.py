@@ -753,11 +753,18 @@ def test_fill_of_many_layers_of_unlike_length(stream):
     cache groups of unlike size): more units than one rows launch takes and
     too unlike for the grid of the units-inner form, so the fill goes out as
     two rows launches (one timed group); bytes against the oracle both ways.
-    A second call of twelve equal layers takes the units-inner form."""
+    A second call of twelve equal layers takes the units-inner form; a third
+    mixes 72 KiB and 8 KiB fragments in one fill."""
     rng = np.random.default_rng(612)
-    for counts in ([8, 8, 600, 8, 8, 8, 8, 8, 600, 8, 8, 8], [40] * 12):
-        cases = [Case(rng, num_blocks=n + 24, seg=32768, segments=2 if li % 3 else 1, n_ids=n)
-                 for li, n in enumerate(counts)]
+    # (blocks, fragment bytes) per layer; the third call mixes 72 KiB and 8 KiB
+    # fragments of one length (latent and indexer caches of one model), which
+    # leaves most workgroups of the small fragments' rows without a tile
+    calls = ([(n, 32768) for n in (8, 8, 600, 8, 8, 8, 8, 8, 600, 8, 8, 8)],
+             [(40, 32768)] * 12,
+             [(512, 73728), (512, 8192)] * 3)
+    for call in calls:
+        cases = [Case(rng, num_blocks=n + 24, seg=seg, segments=2 if li % 3 else 1, n_ids=n)
+                 for li, (n, seg) in enumerate(call)]
         hosts, layers, Ls = [], [], []
         for c in cases:
             L = c.product_layout()
@@ -768,7 +775,7 @@ def test_fill_of_many_layers_of_unlike_length(stream):
             hosts.append(h)
             c.dev.copy_from_host(c.cache0)
             layers.append(_dense_layer(c, L, h, c.ids))
-        xfer = BlockTransfer(staging_slot_bytes=128 << 20, staging_slots=2, auto_staged_min_bytes=1)
+        xfer = BlockTransfer(staging_slot_bytes=256 << 20, staging_slots=2, auto_staged_min_bytes=1)
         xfer.set_kernel_timing(1)
         xfer.save(layers, stream, TransferPath.STAGED)
         stream.synchronize()
