@@ -488,9 +488,8 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
       chunks.push_back({run.first + off, std::min(per_unit, run.second - off)});
     }
   }
-  uint64_t max_chunk_bytes = 0, max_frag = 0;
+  uint64_t max_chunk_bytes = 0;
   for (const Chunk& c : chunks) max_chunk_bytes = std::max(max_chunk_bytes, c.count * pack.page_bytes);
-  for (const LayerPlan& p : plans) max_frag = std::max(max_frag, p.frag_bytes);
   for (auto& sl : slots_) {
     int st = ensure_slot(sl, max_chunk_bytes);
     if (st != PF_OK) return st;
@@ -512,14 +511,44 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
   }
   BlockUnit* units_host = reinterpret_cast<BlockUnit*>(slab_host);
   const BlockUnit* units_dev = reinterpret_cast<const BlockUnit*>(slab_dev);
+  // The units of a chunk in descending slice size, and cut into runs that one
+  // launch serves: its grid gives every unit the tiles of the largest slice, so
+  // slices of unlike size (72 KiB latent and 8 KiB indexer rows in one page)
+  // would leave most workgroups of the small ones without a tile.  A run ends
+  // where less than three quarters of its grid would be busy.
+  std::vector<size_t> plan_order(n_plans);
+  for (size_t pi = 0; pi < n_plans; ++pi) plan_order[pi] = pi;
+  auto tiles_of_plan = [&](size_t pi) {
+    return (plans[pi].frag_bytes + kStagedTileBytes - 1) / kStagedTileBytes;
+  };
+  std::stable_sort(plan_order.begin(), plan_order.end(),
+                   [&](size_t a, size_t b) { return tiles_of_plan(a) > tiles_of_plan(b); });
+  struct UnitRun {
+    size_t begin, count;
+    uint64_t max_frag;
+  };
+  std::vector<UnitRun> unit_runs;
+  for (size_t k = 0; k < n_plans;) {
+    const uint64_t run_tiles = tiles_of_plan(plan_order[k]);  // the largest: sorted
+    uint64_t useful = 0;
+    size_t e = k;
+    while (e < n_plans && e - k < kMaxTileUnits) {
+      const uint64_t with = useful + tiles_of_plan(plan_order[e]);
+      if (e > k && with * 4 < (e - k + 1) * run_tiles * 3) break;
+      useful = with;
+      ++e;
+    }
+    unit_runs.push_back({k, e - k, plans[plan_order[k]].frag_bytes});
+    k = e;
+  }
   std::vector<uint32_t> chunk_slot(chunks.size());
   for (size_t ci = 0; ci < chunks.size(); ++ci) {
     chunk_slot[ci] = next_slot_;
     next_slot_ = (next_slot_ + 1) % n_slots_;
     const uint64_t base = reinterpret_cast<uint64_t>(slots_[chunk_slot[ci]].buf);
-    for (size_t pi = 0; pi < n_plans; ++pi) {
-      const LayerPlan& p = plans[pi];
-      BlockUnit& u = units_host[ci * n_plans + pi];
+    for (size_t k = 0; k < n_plans; ++k) {
+      const LayerPlan& p = plans[plan_order[k]];
+      BlockUnit& u = units_host[ci * n_plans + k];
       std::memset(&u, 0, sizeof(u));
       u.near_base = p.layout.data_ptr();
       u.block_stride = p.layout.block_stride_bytes();
@@ -562,9 +591,12 @@ int Xfer::run_page_pack(std::vector<LayerPlan>& plans, const PagePack& pack, uin
     auto launch = [&](bool to_far) -> int {
       int rc = timing_begin(s);
       if (rc != PF_OK) return rc;
-      rc = launch_block_tiles(units_dev + ci * n_plans, static_cast<uint32_t>(n_plans),
-                              static_cast<uint32_t>(c.count), max_frag, 1, to_far, s);
-      if (rc != PF_OK) return rc;
+      for (const UnitRun& run : unit_runs) {
+        rc = launch_block_tiles(units_dev + ci * n_plans + run.begin,
+                                static_cast<uint32_t>(run.count), static_cast<uint32_t>(c.count),
+                                run.max_frag, 1, to_far, s);
+        if (rc != PF_OK) return rc;
+      }
       return timing_end(s);
     };
     if (save) {

@@ -407,14 +407,17 @@ def _paged_setup(rng, sizes, num_blocks, n, page_gap_after=None, stride_extra=0)
     return offsets, page, pool, idx, page_host, page_dev, ids, cases
 
 
-@pytest.mark.parametrize("variant", ["aligned", "two_runs", "unaligned_slices"])
+@pytest.mark.parametrize("variant", ["aligned", "two_runs", "unaligned_slices", "unlike_slices"])
 def test_page_first_whole_page_packing(variant, xfer, stream):
     """Page-first layers that tile contiguous pages go through staging as whole
     pages (several staging units, slot reuse), byte-exact against the oracle;
-    AUTO picks that path, ZEROCOPY must give the same bytes."""
+    AUTO picks that path, ZEROCOPY must give the same bytes.  `unlike_slices`:
+    72 KiB and 8 KiB slices in one page, which go out as two launches per
+    chunk, the large slices and the small ones."""
     rng = np.random.default_rng(61)
     sizes = {"aligned": [512, 1024, 1536, 4096], "two_runs": [4096, 2048, 1024],
-             "unaligned_slices": [1000, 520, 24, 3000]}[variant]
+             "unaligned_slices": [1000, 520, 24, 3000],
+             "unlike_slices": [73728, 8192, 73728, 8192, 8192]}[variant]
     n = 1000  # x page bytes >= 4 MiB, the AUTO threshold for staging
     gap = 400 if variant == "two_runs" else None
     offsets, page, pool, idx, page_host, page_dev, ids, cases = _paged_setup(
