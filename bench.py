@@ -93,7 +93,7 @@ def parse_args():
     ap.add_argument("--workload",
                     choices=sorted(WORKLOADS) + ["ref_transfer_bench", "ref_cpu_path",
                                                  "link_after_free", "launch_fit",
-                                                 "fragment_sweep"],
+                                                 "fragment_sweep", "unlike_layers"],
                     default="llama8b",
                     help="ref_transfer_bench = the shapes of the reference's own "
                          "benches/transfer_h2d.rs through the descriptor backends; "
@@ -103,7 +103,9 @@ def parse_args():
                          "follow it; launch_fit = duration of one staged gather / scatter launch "
                          "against its bytes: the fixed cost of a launch and the steady rate; "
                          "fragment_sweep = rate of the staged gather / scatter launches against "
-                         "the fragment size, 1 KiB to 256 KiB")
+                         "the fragment size, 1 KiB to 256 KiB; unlike_layers = the staged launches "
+                         "of a task whose layers differ in length (cache groups of a hybrid "
+                         "model) or in fragment size")
     ap.add_argument("--path", choices=["auto", "staged", "zerocopy"], default="auto")
     ap.add_argument("--layers", type=int, default=0, help="override the layer count")
     ap.add_argument("--slot-mb", type=int, default=0)
@@ -205,6 +207,9 @@ def main():
         return
     if args.workload == "fragment_sweep":
         print(json.dumps(run_fragment_sweep(torch, np, runtime)))
+        return
+    if args.workload == "unlike_layers":
+        print(json.dumps(run_unlike_layers(torch, np, runtime)))
         return
     if args.engine_child:
         print(json.dumps(run_workload(args, args.workload, {"engine_child"}, torch, np)))
@@ -505,6 +510,77 @@ def run_fragment_sweep(torch, np, runtime):
     pool.close()
     return {"metric": "staged gather / scatter rate against the fragment size", "unit": "GB/s",
             "rows": rows, "verified": True, "device": runtime.device_name(0)}
+
+
+def run_unlike_layers(torch, np, runtime):
+    """Device time of the staged gather and scatter of one task whose layers
+    are unlike: (a) 48 K/V-split layers of 32 KiB fragments, every sixth with
+    625 blocks and the others with 8 (full-attention and sliding-window cache
+    groups); (b) 24 one-segment layers of 512 blocks, 72 KiB and 8 KiB
+    fragments in turn (latent and indexer caches).  Each task is one staging
+    fill; its launches run alone between one pair of HIP events.  `ideal_us` =
+    the task's algorithmic bytes at 6.2 TB/s, the steady rate of these kernels."""
+    from pegaflow_amd.layout import KVCacheLayout
+    from pegaflow_amd.runtime import PinnedMemory, Stream
+    from pegaflow_amd.transfer import BlockTransfer, LayerBlocks, TransferPath, plan_staged_fills
+    dev = torch.device("cuda:0")
+    stream = Stream()
+    rng = np.random.default_rng(0)
+    tasks = {
+        "layers_of_unlike_length": [(n, 32768, 2) for n in ([8] * 5 + [625]) * 8],
+        "layers_of_unlike_fragment_size": [(512, 73728, 1), (512, 8192, 1)] * 12,
+    }
+    out = {}
+    for name, shapes in tasks.items():
+        nb = 2048
+        src = [torch.empty(nseg * nb * seg, device=dev, dtype=torch.uint8).random_(0, 256)
+               for _n, seg, nseg in shapes]
+        dst = [torch.zeros(nseg * nb * seg, device=dev, dtype=torch.uint8) for _n, seg, nseg in shapes]
+        payload = sum(n * seg * nseg for n, seg, nseg in shapes)
+        pool = PinnedMemory(payload)
+        save_ids = [rng.permutation(nb)[:n].astype(np.uint32) for n, _s, _g in shapes]
+        load_ids = [rng.permutation(nb)[:n].astype(np.uint32) for n, _s, _g in shapes]
+
+        def layers(caches, ids):
+            res, off = [], 0
+            for t, (n, seg, nseg), lids in zip(caches, shapes, ids):
+                kv = nb * seg if nseg == 2 else 0
+                res.append(LayerBlocks(
+                    layout=KVCacheLayout(t.data_ptr(), nseg * nb * seg, nb, seg, kv, nseg), block_ids=lids,
+                    host=tuple(pool.host_ptr + off + g * n * seg for g in range(nseg)),
+                    host_device=tuple(pool.device_ptr + off + g * n * seg for g in range(nseg)),
+                    host_len=tuple(n * seg for _ in range(nseg)), host_stride=seg))
+                off += nseg * n * seg
+            return res
+
+        xfer = BlockTransfer(copy_stream=2)
+        xfer.set_kernel_timing(1)
+        sv, ld = layers(src, save_ids), layers(dst, load_ids)
+        for _rep in range(4):
+            xfer.save(sv, stream, TransferPath.STAGED)
+            stream.synchronize()
+            save_ms, _ = xfer.last_kernel_ms()
+            xfer.load(ld, stream, TransferPath.STAGED)
+            stream.synchronize()
+            load_ms, _ = xfer.last_kernel_ms()
+        for li in (0, 5, len(shapes) - 1):
+            n, seg, nseg = shapes[li]
+            got = dst[li].cpu().numpy().reshape(nseg, nb, seg)
+            want = src[li].cpu().numpy().reshape(nseg, nb, seg)
+            if not np.array_equal(got[:, load_ids[li]], want[:, save_ids[li]]):
+                print(f"bench.py: unlike_layers, {name}, layer {li}: bytes differ", file=sys.stderr)
+                sys.exit(1)
+        _units, fills = plan_staged_fills([n for n, _s, _g in shapes], [s_ * g for _n, s_, g in shapes])
+        out[name] = {"layers": len(shapes), "payload_bytes": payload, "fills": fills,
+                     "gather_us": round(save_ms * 1e3, 1), "scatter_us": round(load_ms * 1e3, 1),
+                     "ideal_us": round(2 * payload / 6.2e6, 1)}
+        xfer.close()
+        pool.close()
+        del src, dst, sv, ld
+        torch.cuda.empty_cache()
+    stream.close()
+    return {"metric": "device time of the staged launches of a task of unlike layers", "unit": "us",
+            "tasks": out, "verified": True, "device": runtime.device_name(0)}
 
 
 def run_workload(args, workload, sections, torch, np):

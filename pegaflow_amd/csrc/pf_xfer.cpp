@@ -1143,16 +1143,15 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
     };
     auto launch_group = [&](bool to_far) -> int {
       if (ue - ui == 1) return launch_tiles(units_dev + ui, units_host[ui], to_far, s);
-      // Workgroups that find a tile to move, and workgroups the one-launch form
-      // would start: the rows form (up to kRowsLaunchUnits units) starts every
-      // row with the tiles of the largest fragment and the segments of the
-      // widest unit; the units-inner form also gives every unit the rows of the
-      // longest.
+      // Workgroups the one-launch form would start: the rows form (up to
+      // kRowsLaunchUnits units) starts every row with the tiles of the largest
+      // fragment and the segments of the widest unit; the units-inner form also
+      // gives every unit the rows of the longest.
       auto tiles_of = [](const BlockUnit& u) {
         return (u.frag_bytes + kStagedTileBytes - 1) / kStagedTileBytes;
       };
       uint32_t max_blocks = 0, max_seg = 0;
-      uint64_t max_frag = 0, max_tiles = 0, total_rows = 0, useful = 0;
+      uint64_t max_frag = 0, max_tiles = 0, total_rows = 0;
       for (size_t k = ui; k < ue; ++k) {
         const BlockUnit& u = units_host[k];
         max_blocks = std::max(max_blocks, u.n_blocks);
@@ -1160,58 +1159,68 @@ int Xfer::run_impl(const pf_layer_blocks* layers, uint64_t n_layers, int path, b
         max_frag = std::max(max_frag, u.frag_bytes);
         max_tiles = std::max(max_tiles, tiles_of(u));
         total_rows += u.n_blocks;
-        useful += static_cast<uint64_t>(u.n_blocks) * tiles_of(u) * u.n_seg;
       }
       const size_t n_group = ue - ui;
       const bool rows_form = n_group <= kRowsLaunchUnits;
       const uint64_t started =
           (rows_form ? total_rows : static_cast<uint64_t>(max_blocks) * n_group) * max_tiles * max_seg;
+      // Units too unlike for one grid leave it full of workgroups that find no
+      // tile.  Those are cheap but not free (they start and end at ~6 000 per
+      // microsecond), and so is every further launch (~8 us of ramp, tail and
+      // hand-over): the fill is cut into runs of units that keep three quarters
+      // of their grids busy, and goes out as one rows launch per run when that
+      // saves more idle workgroups than the launches cost.  A task over cache
+      // groups of unlike size (8 full-attention layers of 625 blocks among 40
+      // sliding-window layers of 8: 82 % of the units-inner grid idle) does:
+      // gather 240 -> 136 us, scatter 241 -> 140 us.  Layers of 72 KiB and of
+      // 8 KiB blocks in turn (44 % idle) do not: one launch 170 us, a launch
+      // per layer 242 us.
+      struct Run {
+        size_t begin, end;
+      };
+      std::vector<Run> runs;
+      uint64_t runs_started = 0;
+      for (size_t k = ui; k < ue;) {
+        size_t e = k;
+        uint64_t run_useful = 0, run_rows = 0, run_tiles = 0, run_seg = 0;
+        while (e < ue && e - k < kRowsLaunchUnits) {
+          const BlockUnit& u = units_host[e];
+          const uint64_t nu = run_useful + static_cast<uint64_t>(u.n_blocks) * tiles_of(u) * u.n_seg;
+          const uint64_t nr = run_rows + u.n_blocks;
+          const uint64_t nt = std::max(run_tiles, tiles_of(u));
+          const uint64_t ns = std::max<uint64_t>(run_seg, u.n_seg);
+          if (e > k && nu * 4 < nr * nt * ns * 3) break;
+          run_useful = nu;
+          run_rows = nr;
+          run_tiles = nt;
+          run_seg = ns;
+          ++e;
+        }
+        runs.push_back({k, e});
+        runs_started += run_rows * run_tiles * run_seg;
+        k = e;
+      }
+      constexpr uint64_t kIdleWorkgroupsPerUs = 6000, kLaunchUs = 8;
+      const bool in_runs = runs.size() > 1 && started > runs_started &&
+                           (started - runs_started) / kIdleWorkgroupsPerUs >
+                               (runs.size() - 1) * kLaunchUs;
       int rc = timing_begin(s);
       if (rc != PF_OK) return rc;
       bool launched = false;
-      if (useful * 4 >= started * 3) {
-        // Units alike enough: one launch.
-        if (rows_form) {
-          rc = launch_block_tiles_rows(units_dev + ui, units_host + ui,
-                                       static_cast<uint32_t>(n_group), to_far, s, &launched);
+      if (in_runs) {
+        for (const Run& run : runs) {
+          rc = launch_block_tiles_rows(units_dev + run.begin, units_host + run.begin,
+                                       static_cast<uint32_t>(run.end - run.begin), to_far, s,
+                                       &launched);
           if (rc != PF_OK) return rc;
+          // (Only a launch beyond the grid limits is refused; what went out
+          // before it is then simply done again by the form below.)
+          if (!launched) break;
         }
-      } else {
-        // Units too unlike for one grid (a task over cache groups of unlike size:
-        // 8 full-attention layers of 625 blocks among 40 sliding-window layers of 8
-        // leave 82 % of the units-inner grid idle; layers of 72 KiB and of 8 KiB
-        // blocks in one fill idle 8 of 9 workgroups of the small ones' rows): the
-        // fill goes out as several rows launches, each over a run of units that
-        // keeps three quarters of its grid busy (the 48-layer task above: gather
-        // 240 -> 138 us, scatter 241 -> 147 us).
-        launched = true;
-        size_t k = ui;
-        while (k < ue && launched) {
-          size_t e = k;
-          uint64_t run_useful = 0, run_rows = 0, run_tiles = 0, run_seg = 0;
-          while (e < ue && e - k < kRowsLaunchUnits) {
-            const BlockUnit& u = units_host[e];
-            const uint64_t nu = run_useful + static_cast<uint64_t>(u.n_blocks) * tiles_of(u) * u.n_seg;
-            const uint64_t nr = run_rows + u.n_blocks;
-            const uint64_t nt = std::max(run_tiles, tiles_of(u));
-            const uint64_t ns = std::max<uint64_t>(run_seg, u.n_seg);
-            if (e > k && nu * 4 < nr * nt * ns * 3) break;
-            run_useful = nu;
-            run_rows = nr;
-            run_tiles = nt;
-            run_seg = ns;
-            ++e;
-          }
-          rc = launch_block_tiles_rows(units_dev + k, units_host + k, static_cast<uint32_t>(e - k),
-                                       to_far, s, &launched);
-          if (rc != PF_OK) return rc;
-          k = e;
-        }
-        if (!launched) {
-          // Nothing but a launch beyond the grid limits gets here; what went out
-          // before it is simply done again below.
-          (void)hipGetLastError();
-        }
+      } else if (rows_form) {
+        rc = launch_block_tiles_rows(units_dev + ui, units_host + ui, static_cast<uint32_t>(n_group),
+                                     to_far, s, &launched);
+        if (rc != PF_OK) return rc;
       }
       if (!launched) {
         rc = launch_block_tiles(units_dev + ui, static_cast<uint32_t>(n_group), max_blocks, max_frag,
